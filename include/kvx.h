@@ -1,0 +1,229 @@
+/*
+ * kvx.h -- C ABI of libkvx: attention-with-score-sums and KV-cache kernels for AMD MI355X (gfx950).
+ *
+ * Everything here is plain C: raw device pointers, element strides, sizes and an opaque stream
+ * handle (a hipStream_t passed as void*; NULL = the null stream). No entry point allocates or
+ * frees memory, none synchronises the stream, none throws. Every call returns KVX_OK (0) or a
+ * KVX_ERR_* code; kvx_last_error() then holds a message for the calling thread.
+ *
+ * Each entry point names the interface of awslabs/keys_values (the "reference", paths relative
+ * to its repository root) that it stands in for.
+ *
+ * Conventions
+ *   B      batch size                 Hq     query heads          Hkv   key/value heads
+ *   G      Hq / Hkv (group size)      D      head size (64 or 128)
+ *   q_len  queries per call           kv_len cache slots visible to the call
+ *   Tensors are addressed as base + b*stride_b + h*stride_h + t*stride_t + d with the head
+ *   dimension contiguous; strides are in ELEMENTS of the tensor's own type. This covers both the
+ *   reference's (B, H, T, D) cache views (keys_values/kvcache/buffers.py:538-541) and the
+ *   (B, T, H, D) layout of its extension (keys_values/csrc/bindings.cpp:98-122) without a copy.
+ *   token_positions is int32 (B, Hkv, kv_len) (keys_values/kvcache/attn_weights.py:466-470);
+ *   a NULL pointer means arange(kv_len) (keys_values/attention/attention_utils.py:425-432).
+ *   A query at chunk offset i may see slot k iff token_positions[b,h,k] <= input_pos + i
+ *   (keys_values/attention/attention_utils.py:238-247).
+ *   Score-sums W are fp32 (B, Hkv, kv_len): sum over queries, MEAN over the G grouped heads
+ *   (keys_values/attention/base.py:707-725, keys_values/attention/flashinfer_wrapper.py:269-273).
+ *   LSE is fp32 (B, q_len, Hq), base 2 (keys_values/csrc/kernels/sdpa_prefill.cu:509-512).
+ */
+#ifndef KVX_H
+#define KVX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVX_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum kvx_status {
+  KVX_OK = 0,
+  KVX_ERR_INVALID = 1,     /* bad shape / stride / NULL pointer / range  (reference: TORCH_CHECK, bindings.cpp:37-62) */
+  KVX_ERR_UNSUPPORTED = 2, /* head size or dtype outside what the kernels cover (reference: NotImplementedError,
+                              flashinfer_wrapper.py:425-432) */
+  KVX_ERR_HIP = 3,         /* a HIP runtime call failed (reference: TORCH_CHECK(err == cudaSuccess), bindings.cpp:486,955) */
+  KVX_ERR_WORKSPACE = 4    /* workspace pointer NULL or smaller than kvx_*_workspace_bytes() */
+};
+
+/* Storage type of the K/V cache handed to the attention kernels. */
+enum kvx_kv_dtype {
+  KVX_KV_BF16 = 0, /* bfloat16 rows */
+  KVX_KV_U8 = 1    /* uint8 codes + per-row fp32 scale and int32 zero point (the reference's
+                      "torch-quantized8" store, keys_values/kvcache/quantize/pytorch.py:281-295);
+                      rows are dequantised inside the kernel exactly as
+                      keys_values/kvcache/quantize/pytorch.py:143-154,467-478 would, i.e. to bf16 */
+};
+
+/* One attention call. Unused pointers are NULL. All strides in elements. */
+typedef struct kvx_sdpa_args {
+  int32_t B, Hq, Hkv, q_len, kv_len, D;
+  int32_t input_pos;   /* position of the first query; >= 0 */
+  int32_t kv_dtype;    /* enum kvx_kv_dtype */
+  float sm_scale;      /* softmax scale, e.g. 1/sqrt(D) */
+  int32_t num_splits;  /* KV splits for prefill/decode; 0 = library heuristic */
+
+  const void* q;       /* bf16 (B, Hq, q_len, D) by strides */
+  int64_t q_stride_b, q_stride_h, q_stride_t;
+  const void* k;       /* bf16 or uint8 (B, Hkv, kv_len, D) by strides */
+  int64_t k_stride_b, k_stride_h, k_stride_t;
+  const void* v;
+  int64_t v_stride_b, v_stride_h, v_stride_t;
+  /* KVX_KV_U8 only: per-row state (B, Hkv, kv_len), strides shared by the four arrays */
+  const float* k_scale;
+  const int32_t* k_zp;
+  const float* v_scale;
+  const int32_t* v_zp;
+  int64_t qs_stride_b, qs_stride_h;
+
+  const int32_t* token_positions; /* (B, Hkv, kv_len) or NULL */
+  int64_t tp_stride_b, tp_stride_h;
+
+  void* o;             /* bf16 (B, Hq, q_len, D) by strides */
+  int64_t o_stride_b, o_stride_h, o_stride_t;
+  float* lse;          /* fp32 (B, q_len, Hq) contiguous, base 2; output of prefill/decode, input of score_sum */
+  float* w;            /* fp32 (B, Hkv, kv_len) contiguous score-sums, or NULL */
+
+  void* workspace;     /* scratch, kvx_sdpa_*_workspace_bytes(); may be NULL when that returns 0 */
+  size_t workspace_bytes;
+} kvx_sdpa_args;
+
+/* ---- library ------------------------------------------------------------------------------- */
+
+/* Library version (KVX_VERSION of the build). */
+int kvx_version(void);
+
+/* Message of the last failing call on this thread ("" if none). The pointer stays valid until
+ * the next failing call on the same thread. */
+const char* kvx_last_error(void);
+
+/* Replaces is_available() / get_device_count() of the reference extension module
+ * (keys_values/csrc/bindings.cpp:1722-1735): number of visible HIP devices whose architecture is
+ * gfx950, 0 if none (never fails). */
+int kvx_device_count(void);
+
+/* Replaces get_device_info(device_id) (keys_values/csrc/bindings.cpp:1733-1735). Writes a
+ * NUL-terminated description ("name, arch, CUs, LDS per CU, memory") into buf. */
+int kvx_device_info(int device, char* buf, size_t buf_len);
+
+/* ---- attention ----------------------------------------------------------------------------- */
+
+/* Chunked-prefill attention: O = softmax(s*Q K^T + mask) V and the base-2 log-sum-exp per query row.
+ * Stands in for sdpa_prefill(..., return_lse=True) of the reference extension
+ * (keys_values/csrc/bindings.cpp:511-958, keys_values/attention/flashinfer_ops.py:302-370) and for
+ * the FlashInfer prefill kernel behind it (keys_values/csrc/kernels/sdpa_prefill.cu:34-181,
+ * 1182-1256); unlike those it takes token_positions directly, so the caller does not reorder the
+ * cache (keys_values/attention/sdpa_wrapper.py:352-369). args->lse may be NULL if not wanted;
+ * args->w is ignored. */
+int kvx_sdpa_prefill(const kvx_sdpa_args* args, void* stream);
+size_t kvx_sdpa_prefill_workspace_bytes(const kvx_sdpa_args* args);
+
+/* Per-key score-sums from Q, K and the log-sum-exp of a preceding kvx_sdpa_prefill:
+ * W[b,h,k] = (1/G) * sum_{i,g} exp2(s*log2(e)*q_{i,g}.k - lse[b,i,h*G+g]) * [tp[b,h,k] <= input_pos+i].
+ * Stands in for triton_score_sum / _score_sum_kernel
+ * (keys_values/attention/flashinfer_wrapper.py:51-273). Deterministic: every W element is owned by
+ * one wavefront, no atomics. Reads args->lse, writes args->w; o and v are ignored. */
+int kvx_score_sum(const kvx_sdpa_args* args, void* stream);
+
+/* kvx_sdpa_prefill followed by kvx_score_sum on the same stream: the whole
+ * FlashInferSDPA._flashinfer_sdpa_fused_prefill step
+ * (keys_values/attention/flashinfer_wrapper.py:476-494). args->lse must be given (it carries the
+ * log-sum-exp between the two kernels); workspace as for kvx_sdpa_prefill. */
+int kvx_sdpa_prefill_weights(const kvx_sdpa_args* args, void* stream);
+
+/* Single-token decode (q_len == 1): O over the whole cache and, if args->w is set, the score-sums
+ * W = (1/G) sum_g softmax_g. No mask: the new token is the newest
+ * (keys_values/attention/flashinfer_wrapper.py:471-481, keys_values/attention/flashinfer_ops.py:250-275).
+ * Stands in for sdpa_decode of the reference extension (keys_values/csrc/bindings.cpp:86-489) and
+ * optimized_batched_decode_kernel (keys_values/csrc/kernels/sdpa_decode.cu:616-898). One workgroup
+ * per (batch, KV head, split) serves all G query heads, so K and V are read once.
+ * The workspace holds the fp32 logits (B, Hq, kv_len) and the split partials. args->lse optional. */
+int kvx_sdpa_decode(const kvx_sdpa_args* args, void* stream);
+size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* args);
+
+/* ---- cache: quantiser ---------------------------------------------------------------------- */
+
+/* Affine 8-bit row quantiser: for each row x[0..D) (bf16, upcast to fp32)
+ *   scale = max((max - min) / 255, 1.1920929e-07);  zp = -(int32) rint(min / scale);
+ *   code  = (uint8) clamp(rint(x * (1 / scale)) + zp, 0, 255)
+ * bit-for-bit as TorchBasicQuantizer._quantize with MyPerChannelMinMaxObserver._calculate_qparams and
+ * quantize_per_channel (keys_values/kvcache/quantize/pytorch.py:100-139,312-355).
+ * x: bf16, `rows` rows of D elements, row r at x + r*x_row_stride. codes: uint8 rows*D contiguous.
+ * scale / zp: one per row, contiguous. D in {64, 128}. */
+int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D,
+                      uint8_t* codes, float* scale, int32_t* zp, void* stream);
+
+/* Inverse: out[r][d] = bf16( (float)((int32)code - zp) * scale ), as TorchBasicQuantizer._dequantize /
+ * dequantize_per_channel (keys_values/kvcache/quantize/pytorch.py:143-154,411-478). */
+int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows,
+                        int32_t D, void* out, int64_t out_row_stride, void* stream);
+
+/* ---- cache: write and H2O bookkeeping ------------------------------------------------------- */
+
+/* Write `num` new tokens into the slots chosen by the previous selection, and do the bookkeeping
+ * that AttnWeightsKVCache._forward_internal does around it
+ * (keys_values/kvcache/attn_weights.py:510-635 without grace period; update_token_positions
+ * :214-317; DefaultKVCacheBuffers.set_slots, keys_values/kvcache/buffers.py:498-519;
+ * _update_score_buffers_in_forward :679-681):
+ *   slot = index[b,h,j];  token_pos[b,h,slot] = input_pos + j;  scores[b,h,slot] = 0;
+ *   K[b,h,slot,:] = key[b,h,j,:];  V likewise.
+ * With kv_dtype == KVX_KV_U8 the rows are quantised on the way in (same arithmetic as
+ * kvx_quantize_rows) into codes + k_scale/k_zp/v_scale/v_zp.
+ * index: int32 (B, Hkv, index_stride_h >= num) with index_stride_b / _h in elements.
+ * key/value: bf16 (B, Hkv, num, D) by strides. scores may be NULL (no score buffer). */
+typedef struct kvx_cache_write_args {
+  int32_t B, Hkv, num, D, cache_len;
+  int32_t input_pos;
+  int32_t kv_dtype;
+  const int32_t* index;
+  int64_t index_stride_b, index_stride_h;
+  const void* key;
+  int64_t key_stride_b, key_stride_h, key_stride_t;
+  const void* value;
+  int64_t value_stride_b, value_stride_h, value_stride_t;
+  void* k_cache; /* bf16 or uint8 (B, Hkv, cache_len, D) */
+  int64_t kc_stride_b, kc_stride_h, kc_stride_t;
+  void* v_cache;
+  int64_t vc_stride_b, vc_stride_h, vc_stride_t;
+  float* k_scale;
+  int32_t* k_zp;
+  float* v_scale;
+  int32_t* v_zp;
+  int64_t qs_stride_b, qs_stride_h;
+  int32_t* token_pos; /* (B, Hkv, cache_len) */
+  int64_t tp_stride_b, tp_stride_h;
+  float* scores; /* (B, Hkv, cache_len) or NULL */
+  int64_t sc_stride_b, sc_stride_h;
+} kvx_cache_write_args;
+int kvx_cache_write(const kvx_cache_write_args* args, void* stream);
+
+/* H2O score update and eviction choice, AttnWeightsKVCache._update with H2OKVCache._compute_scores
+ * (keys_values/kvcache/attn_weights.py:721-783, keys_values/kvcache/h2o.py:146-199):
+ *   scores[b,h,:kv_len] += w[b,h,:kv_len]           (skipped when w is NULL)
+ *   next_index[b,h,0..k) = the k slots of scores[b,h,:limit] with the smallest value,
+ *                          in ascending (value, slot) order, ties to the lower slot.
+ * This is scores.argsort(-1)[..., :k]; the reference's topk(k, largest=False, sorted=False) returns
+ * the same set in unspecified order. With normalize != 0 the value compared is
+ * scores / (input_pos - max(token_pos, prefill_len - 1)) (keys_values/kvcache/h2o.py:183-196);
+ * token_pos then must be given. 1 <= k <= min(limit, 4096); limit <= kv_len.
+ * scores rows at scores + b*sc_stride_b + h*sc_stride_h; w contiguous (B, Hkv, kv_len).
+ * next_index: int32 (B, Hkv, k) contiguous. */
+typedef struct kvx_h2o_args {
+  int32_t B, Hkv, kv_len, limit, k;
+  int32_t normalize, input_pos, prefill_len;
+  float* scores;
+  int64_t sc_stride_b, sc_stride_h;
+  const float* w;
+  const int32_t* token_pos;
+  int64_t tp_stride_b, tp_stride_h;
+  int32_t* next_index;
+  void* workspace;
+  size_t workspace_bytes;
+} kvx_h2o_args;
+int kvx_h2o_update_select(const kvx_h2o_args* args, void* stream);
+size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVX_H */

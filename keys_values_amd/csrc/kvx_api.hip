@@ -1,0 +1,214 @@
+// C ABI of libkvx: argument validation, error reporting and dispatch to the kernel launchers.
+// The checks mirror what the reference extension enforces before launching
+// (keys_values/csrc/bindings.cpp:37-62,98-178) and what keys_values/attention/sdpa_wrapper.py:24-47
+// requires of the shapes; they also make sure no kernel can be launched on operands whose shape
+// does not fit its indexing.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "kvx_common.h"
+
+namespace kvx {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_error(hipError_t e, const char* what) {
+  return set_error(KVX_ERR_HIP, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+}
+
+int num_cus() {
+  static thread_local int cached_dev = -1;
+  static thread_local int cached = 256;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return cached;
+  if (dev != cached_dev) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cached = n;
+    cached_dev = dev;
+  }
+  return cached;
+}
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool mult8(int64_t x) { return (x & 7) == 0; }
+
+int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
+  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "%s: args is NULL", who);
+  KVX_REQUIRE(a->B > 0 && a->Hq > 0 && a->Hkv > 0 && a->q_len > 0 && a->kv_len > 0, KVX_ERR_INVALID,
+              "%s: sizes must be positive (B=%d Hq=%d Hkv=%d q_len=%d kv_len=%d)", who, a->B, a->Hq, a->Hkv, a->q_len,
+              a->kv_len);
+  KVX_REQUIRE(a->Hq % a->Hkv == 0, KVX_ERR_INVALID, "%s: Hq=%d must be a multiple of Hkv=%d", who, a->Hq, a->Hkv);
+  KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, a->D);
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8, KVX_ERR_UNSUPPORTED, "%s: unknown kv_dtype %d", who,
+              a->kv_dtype);
+  KVX_REQUIRE(a->input_pos >= 0, KVX_ERR_INVALID, "%s: input_pos=%d must be >= 0", who, a->input_pos);
+  KVX_REQUIRE(a->sm_scale > 0.0f, KVX_ERR_INVALID, "%s: sm_scale must be positive", who);
+  KVX_REQUIRE((int64_t)a->input_pos + a->q_len < INT32_MAX, KVX_ERR_INVALID, "%s: positions overflow int32", who);
+  KVX_REQUIRE(a->q && a->k, KVX_ERR_INVALID, "%s: q and k must be given", who);
+  KVX_REQUIRE(aligned16(a->q) && mult8(a->q_stride_b) && mult8(a->q_stride_h) && mult8(a->q_stride_t), KVX_ERR_INVALID,
+              "%s: q must be 16-byte aligned with strides that are multiples of 8 elements", who);
+  KVX_REQUIRE(aligned16(a->k) && mult8(a->k_stride_b) && mult8(a->k_stride_h) && mult8(a->k_stride_t), KVX_ERR_INVALID,
+              "%s: k must be 16-byte aligned with strides that are multiples of 8 elements", who);
+  KVX_REQUIRE(a->k_stride_t >= a->D && a->q_stride_t >= 0, KVX_ERR_INVALID, "%s: bad k/q slot stride", who);
+  if (need_v_o) {
+    KVX_REQUIRE(a->v && a->o, KVX_ERR_INVALID, "%s: v and o must be given", who);
+    KVX_REQUIRE(aligned16(a->v) && mult8(a->v_stride_b) && mult8(a->v_stride_h) && mult8(a->v_stride_t), KVX_ERR_INVALID,
+                "%s: v must be 16-byte aligned with strides that are multiples of 8 elements", who);
+    KVX_REQUIRE(aligned16(a->o) && mult8(a->o_stride_b) && mult8(a->o_stride_h) && mult8(a->o_stride_t), KVX_ERR_INVALID,
+                "%s: o must be 16-byte aligned with strides that are multiples of 8 elements", who);
+    KVX_REQUIRE(a->v_stride_t >= a->D, KVX_ERR_INVALID, "%s: bad v slot stride", who);
+  }
+  if (a->kv_dtype == KVX_KV_U8) {
+    KVX_REQUIRE(a->k_scale && a->k_zp, KVX_ERR_INVALID, "%s: uint8 cache needs k_scale and k_zp", who);
+    if (need_v_o) KVX_REQUIRE(a->v_scale && a->v_zp, KVX_ERR_INVALID, "%s: uint8 cache needs v_scale and v_zp", who);
+  }
+  KVX_REQUIRE(a->num_splits >= 0, KVX_ERR_INVALID, "%s: num_splits must be >= 0", who);
+  return KVX_OK;
+}
+
+}  // namespace
+}  // namespace kvx
+
+using namespace kvx;
+
+extern "C" {
+
+int kvx_version(void) { return KVX_VERSION; }
+
+const char* kvx_last_error(void) { return g_err; }
+
+int kvx_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  int good = 0;
+  for (int i = 0; i < n; ++i) {
+    hipDeviceProp_t pr;
+    if (hipGetDeviceProperties(&pr, i) == hipSuccess && strncmp(pr.gcnArchName, "gfx950", 6) == 0) ++good;
+  }
+  return good;
+}
+
+int kvx_device_info(int device, char* buf, size_t buf_len) {
+  KVX_REQUIRE(buf && buf_len > 0, KVX_ERR_INVALID, "kvx_device_info: empty buffer");
+  hipDeviceProp_t pr;
+  KVX_HIP(hipGetDeviceProperties(&pr, device));
+  snprintf(buf, buf_len, "%s, %s, %d CUs, %zu KiB LDS per workgroup, %.1f GiB", pr.name, pr.gcnArchName,
+           pr.multiProcessorCount, pr.sharedMemPerBlock / 1024, (double)pr.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+  return KVX_OK;
+}
+
+size_t kvx_sdpa_prefill_workspace_bytes(const kvx_sdpa_args* a) {
+  if (check_sdpa_common(a, "kvx_sdpa_prefill_workspace_bytes", false) != KVX_OK) return 0;
+  return sdpa_prefill_workspace(*a);
+}
+
+int kvx_sdpa_prefill(const kvx_sdpa_args* a, void* stream) {
+  int rc = check_sdpa_common(a, "kvx_sdpa_prefill", true);
+  if (rc != KVX_OK) return rc;
+  KVX_REQUIRE(a->q_len <= a->kv_len, KVX_ERR_INVALID, "kvx_sdpa_prefill: q_len=%d exceeds kv_len=%d", a->q_len, a->kv_len);
+  return launch_sdpa_prefill(*a, (hipStream_t)stream);
+}
+
+int kvx_score_sum(const kvx_sdpa_args* a, void* stream) {
+  int rc = check_sdpa_common(a, "kvx_score_sum", false);
+  if (rc != KVX_OK) return rc;
+  KVX_REQUIRE(a->lse && a->w, KVX_ERR_INVALID, "kvx_score_sum: lse and w must be given");
+  return launch_score_sum(*a, (hipStream_t)stream);
+}
+
+int kvx_sdpa_prefill_weights(const kvx_sdpa_args* a, void* stream) {
+  int rc = check_sdpa_common(a, "kvx_sdpa_prefill_weights", true);
+  if (rc != KVX_OK) return rc;
+  KVX_REQUIRE(a->q_len <= a->kv_len, KVX_ERR_INVALID, "kvx_sdpa_prefill_weights: q_len=%d exceeds kv_len=%d", a->q_len,
+              a->kv_len);
+  KVX_REQUIRE(a->lse && a->w, KVX_ERR_INVALID, "kvx_sdpa_prefill_weights: lse and w must be given");
+  rc = launch_sdpa_prefill(*a, (hipStream_t)stream);
+  if (rc != KVX_OK) return rc;
+  return launch_score_sum(*a, (hipStream_t)stream);
+}
+
+size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* a) {
+  if (check_sdpa_common(a, "kvx_sdpa_decode_workspace_bytes", false) != KVX_OK) return 0;
+  return sdpa_decode_workspace(*a);
+}
+
+int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
+  int rc = check_sdpa_common(a, "kvx_sdpa_decode", true);
+  if (rc != KVX_OK) return rc;
+  KVX_REQUIRE(a->q_len == 1, KVX_ERR_INVALID, "kvx_sdpa_decode: q_len must be 1, got %d", a->q_len);
+  const int G = a->Hq / a->Hkv;
+  KVX_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in {1, 2, 4, 8}", G);
+  KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_decode: workspace must be 16-byte aligned");
+  return launch_sdpa_decode(*a, (hipStream_t)stream);
+}
+
+int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale,
+                      int32_t* zp, void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_quantize_rows: row length %d not in {64, 128}", D);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_quantize_rows: rows must be >= 0");
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(x && codes && scale && zp, KVX_ERR_INVALID, "kvx_quantize_rows: NULL pointer");
+  KVX_REQUIRE(aligned16(x) && mult8(x_row_stride) && x_row_stride >= D, KVX_ERR_INVALID,
+              "kvx_quantize_rows: x must be 16-byte aligned, row stride a multiple of 8 and >= D");
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_quantize_rows: codes must be 8-byte aligned");
+  return launch_quantize_rows(x, x_row_stride, rows, D, codes, scale, zp, (hipStream_t)stream);
+}
+
+int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out,
+                        int64_t out_row_stride, void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_dequantize_rows: row length %d not in {64, 128}", D);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_dequantize_rows: rows must be >= 0");
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(codes && scale && zp && out, KVX_ERR_INVALID, "kvx_dequantize_rows: NULL pointer");
+  KVX_REQUIRE(aligned16(out) && mult8(out_row_stride) && out_row_stride >= D, KVX_ERR_INVALID,
+              "kvx_dequantize_rows: out must be 16-byte aligned, row stride a multiple of 8 and >= D");
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_dequantize_rows: codes must be 8-byte aligned");
+  return launch_dequantize_rows(codes, scale, zp, rows, D, out, out_row_stride, (hipStream_t)stream);
+}
+
+int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
+  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
+  KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");
+  KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "kvx_cache_write: head size %d not in {64, 128}", a->D);
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8, KVX_ERR_UNSUPPORTED, "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
+  KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
+  KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache && a->token_pos, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
+  KVX_REQUIRE(aligned16(a->key) && aligned16(a->value) && mult8(a->key_stride_b) && mult8(a->key_stride_h) &&
+                  mult8(a->key_stride_t) && mult8(a->value_stride_b) && mult8(a->value_stride_h) && mult8(a->value_stride_t),
+              KVX_ERR_INVALID, "kvx_cache_write: key/value must be 16-byte aligned with strides that are multiples of 8");
+  KVX_REQUIRE(aligned16(a->k_cache) && aligned16(a->v_cache) && mult8(a->kc_stride_b) && mult8(a->kc_stride_h) &&
+                  mult8(a->kc_stride_t) && mult8(a->vc_stride_b) && mult8(a->vc_stride_h) && mult8(a->vc_stride_t),
+              KVX_ERR_INVALID, "kvx_cache_write: caches must be 16-byte aligned with strides that are multiples of 8");
+  if (a->kv_dtype == KVX_KV_U8)
+    KVX_REQUIRE(a->k_scale && a->k_zp && a->v_scale && a->v_zp, KVX_ERR_INVALID, "kvx_cache_write: uint8 cache needs scale / zero-point arrays");
+  KVX_REQUIRE((int64_t)a->input_pos + a->num < INT32_MAX && a->input_pos >= 0, KVX_ERR_INVALID, "kvx_cache_write: bad input_pos");
+  return launch_cache_write(*a, (hipStream_t)stream);
+}
+
+size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* a) { return a ? h2o_workspace(*a) : 0; }
+
+int kvx_h2o_update_select(const kvx_h2o_args* a, void* stream) {
+  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_h2o_update_select: args is NULL");
+  KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->kv_len > 0, KVX_ERR_INVALID, "kvx_h2o_update_select: sizes must be positive");
+  KVX_REQUIRE(a->limit > 0 && a->limit <= a->kv_len, KVX_ERR_INVALID, "kvx_h2o_update_select: limit=%d must be in [1, kv_len=%d]", a->limit, a->kv_len);
+  KVX_REQUIRE(a->k >= 1 && a->k <= a->limit && a->k <= 4096, KVX_ERR_INVALID, "kvx_h2o_update_select: k=%d must be in [1, min(limit, 4096)]", a->k);
+  KVX_REQUIRE(a->scores && a->next_index, KVX_ERR_INVALID, "kvx_h2o_update_select: NULL pointer");
+  KVX_REQUIRE(!a->normalize || a->token_pos, KVX_ERR_INVALID, "kvx_h2o_update_select: normalize needs token_pos");
+  return launch_h2o_update_select(*a, (hipStream_t)stream);
+}
+
+}  // extern "C"

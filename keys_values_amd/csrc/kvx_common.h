@@ -1,0 +1,99 @@
+// Shared device/host helpers for the libkvx kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <limits.h>
+
+#include "../../include/kvx.h"
+
+namespace kvx {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWave = 64;
+
+// Records the message kvx_last_error() returns on this thread, returns `code`.
+int set_error(int code, const char* fmt, ...);
+int hip_error(hipError_t e, const char* what);
+
+#define KVX_REQUIRE(cond, code, ...)            \
+  do {                                          \
+    if (!(cond)) return ::kvx::set_error((code), __VA_ARGS__); \
+  } while (0)
+
+#define KVX_HIP(call)                                      \
+  do {                                                     \
+    hipError_t e__ = (call);                               \
+    if (e__ != hipSuccess) return ::kvx::hip_error(e__, #call); \
+  } while (0)
+
+// ---- launchers implemented one per translation unit ---------------------------------------
+int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st);
+size_t sdpa_prefill_workspace(const kvx_sdpa_args& a);
+int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st);
+int launch_sdpa_decode(const kvx_sdpa_args& a, hipStream_t st);
+size_t sdpa_decode_workspace(const kvx_sdpa_args& a);
+int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,
+                         int32_t* zp, hipStream_t st);
+int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
+                           int64_t out_row_stride, hipStream_t st);
+int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st);
+int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st);
+size_t h2o_workspace(const kvx_h2o_args& a);
+
+// Number of compute units of the current device (cached).
+int num_cus();
+
+// ---- device helpers ------------------------------------------------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// Round-to-nearest-even fp32 -> bf16 (two at a time), bit pattern in a dword (lo = a, hi = b).
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  bf16x2_t r = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Exchange with the lane 32 away (the other half of the wavefront).
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// The affine 8-bit row quantiser, one element. `inv` = 1.0f / scale, `zf` = (float) zero point.
+// rint before the add, so the multiply can never fuse with it.
+__device__ __forceinline__ uint32_t quant_code(float x, float inv, float zf) {
+  float c = __builtin_rintf(x * inv) + zf;
+  c = fminf(fmaxf(c, 0.0f), 255.0f);
+  return (uint32_t)c;
+}
+
+// scale and zero point of a row from its min and max (IEEE division, no fast-math).
+__device__ __forceinline__ void quant_params(float mn, float mx, float& scale, int32_t& zp) {
+  float s = (mx - mn) / 255.0f;
+  s = fmaxf(s, 1.1920929e-07f);
+  scale = s;
+  zp = 0 - (int32_t)__builtin_rintf(mn / s);
+}
+
+// bf16( (float)((int)code - zp) * scale ), two codes -> packed dword.
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
+  float a = (float)((int32_t)c0 - zp) * scale;
+  float b = (float)((int32_t)c1 - zp) * scale;
+  return pack_bf16(a, b);
+}
+
+}  // namespace kvx

@@ -1,0 +1,221 @@
+// Affine 8-bit row quantiser / dequantiser and the cache-slot write for gfx950 (HBM-bound byte work).
+//
+// Reference behaviour: keys_values/kvcache/quantize/pytorch.py:100-139,312-355 (quantise),
+// :143-154,411-478 (dequantise); keys_values/kvcache/attn_weights.py:305-316,679-681 and
+// keys_values/kvcache/buffers.py:498-519 (slot write).
+//
+// A row of D bf16 values is spread over D/8 adjacent lanes, 8 values (one 16-byte load) per lane,
+// so a wavefront reads 1 KiB of contiguous input per load instruction and writes 512 contiguous
+// bytes of codes. Row min and max are reduced with DPP moves inside the 16-lane row (no LDS).
+#include "kvx_common.h"
+
+namespace kvx {
+namespace {
+
+constexpr int NTHREADS = 256;
+constexpr int ROWS_PER_THREAD = 4;  // independent rows in flight per lane
+
+// Reductions over the LPR (8 or 16) adjacent lanes holding one row; every lane gets the result.
+template <int LPR>
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)));  // row_half_mirror
+  if constexpr (LPR == 16)
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)));  // row_mirror
+  return v;
+}
+template <int LPR>
+__device__ __forceinline__ float row_min(float v) {
+  v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)));
+  v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)));
+  v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)));
+  if constexpr (LPR == 16)
+    v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)));
+  return v;
+}
+
+// Quantise the 8 values of this lane's share of a row; every lane of the row returns the same
+// scale / zero point.
+template <int LPR>
+__device__ __forceinline__ u32x2_t quantize8(u32x4_t raw, float& scale, int32_t& zp) {
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = bf16_lo(raw[e]);
+    x[2 * e + 1] = bf16_hi(raw[e]);
+  }
+  float mn = x[0], mx = x[0];
+#pragma unroll
+  for (int e = 1; e < 8; ++e) {
+    mn = fminf(mn, x[e]);
+    mx = fmaxf(mx, x[e]);
+  }
+  mn = row_min<LPR>(mn);
+  mx = row_max<LPR>(mx);
+  quant_params(mn, mx, scale, zp);
+  const float inv = 1.0f / scale;
+  const float zf = (float)zp;
+  u32x2_t out;
+  out[0] = quant_code(x[0], inv, zf) | (quant_code(x[1], inv, zf) << 8) | (quant_code(x[2], inv, zf) << 16) |
+           (quant_code(x[3], inv, zf) << 24);
+  out[1] = quant_code(x[4], inv, zf) | (quant_code(x[5], inv, zf) << 8) | (quant_code(x[6], inv, zf) << 16) |
+           (quant_code(x[7], inv, zf) << 24);
+  return out;
+}
+
+template <int D>
+__global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
+                                                                 int64_t rows, uint8_t* __restrict__ codes,
+                                                                 float* __restrict__ scale, int32_t* __restrict__ zp) {
+  constexpr int LPR = D / 8;
+  constexpr int RPB = NTHREADS / LPR;  // rows per block per step
+  const int col = threadIdx.x % LPR;
+  const int64_t row0 = (int64_t)blockIdx.x * (RPB * ROWS_PER_THREAD) + threadIdx.x / LPR;
+  u32x4_t raw[ROWS_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    raw[i] = r < rows ? *(const u32x4_t*)(x + r * x_row_stride + col * 8) : u32x4_t{0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    float s;
+    int32_t z;
+    const u32x2_t c = quantize8<LPR>(raw[i], s, z);  // executed by all lanes: the DPP reduction needs them
+    if (r < rows) {
+      *(u32x2_t*)(codes + r * D + col * 8) = c;
+      if (col == 0) {
+        scale[r] = s;
+        zp[r] = z;
+      }
+    }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t* __restrict__ codes,
+                                                                   const float* __restrict__ scale,
+                                                                   const int32_t* __restrict__ zp, int64_t rows,
+                                                                   uint16_t* __restrict__ out, int64_t out_row_stride) {
+  constexpr int LPR = D / 8;
+  constexpr int RPB = NTHREADS / LPR;
+  const int col = threadIdx.x % LPR;
+  const int64_t row0 = (int64_t)blockIdx.x * (RPB * ROWS_PER_THREAD) + threadIdx.x / LPR;
+  u32x2_t c[ROWS_PER_THREAD];
+  float s[ROWS_PER_THREAD];
+  int32_t z[ROWS_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    const bool ok = r < rows;
+    c[i] = ok ? *(const u32x2_t*)(codes + r * D + col * 8) : u32x2_t{0, 0};
+    s[i] = ok ? scale[r] : 0.0f;
+    z[i] = ok ? zp[r] : 0;
+  }
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    if (r >= rows) continue;
+    u32x4_t o;
+    o[0] = dequant_pair(c[i][0] & 0xff, (c[i][0] >> 8) & 0xff, z[i], s[i]);
+    o[1] = dequant_pair((c[i][0] >> 16) & 0xff, c[i][0] >> 24, z[i], s[i]);
+    o[2] = dequant_pair(c[i][1] & 0xff, (c[i][1] >> 8) & 0xff, z[i], s[i]);
+    o[3] = dequant_pair((c[i][1] >> 16) & 0xff, c[i][1] >> 24, z[i], s[i]);
+    *(u32x4_t*)(out + r * out_row_stride + col * 8) = o;
+  }
+}
+
+// One lane per 8 elements of one new (b, h, j) row, for K and V.
+template <int D, bool U8>
+__global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
+  constexpr int LPR = D / 8;
+  const int64_t gid = (int64_t)blockIdx.x * NTHREADS + threadIdx.x;
+  const int col = (int)(gid % LPR);
+  const int64_t rid = gid / LPR;
+  const int64_t total = (int64_t)a.B * a.Hkv * a.num;
+  const bool live = rid < total;
+  const int64_t ridc = live ? rid : 0;
+  const int j = (int)(ridc % a.num);
+  const int hh = (int)((ridc / a.num) % a.Hkv);
+  const int b = (int)(ridc / ((int64_t)a.num * a.Hkv));
+  const int slot = a.index[b * a.index_stride_b + hh * a.index_stride_h + j];
+  const bool ok = live && slot >= 0 && slot < a.cache_len;  // a bad index is dropped, never written out of bounds
+  const uint16_t* ks = (const uint16_t*)a.key + b * a.key_stride_b + hh * a.key_stride_h + (int64_t)j * a.key_stride_t + col * 8;
+  const uint16_t* vs = (const uint16_t*)a.value + b * a.value_stride_b + hh * a.value_stride_h + (int64_t)j * a.value_stride_t + col * 8;
+  const u32x4_t kr = live ? *(const u32x4_t*)ks : u32x4_t{0, 0, 0, 0};
+  const u32x4_t vr = live ? *(const u32x4_t*)vs : u32x4_t{0, 0, 0, 0};
+  if constexpr (!U8) {
+    if (ok) {
+      *(u32x4_t*)((uint16_t*)a.k_cache + b * a.kc_stride_b + hh * a.kc_stride_h + (int64_t)slot * a.kc_stride_t + col * 8) = kr;
+      *(u32x4_t*)((uint16_t*)a.v_cache + b * a.vc_stride_b + hh * a.vc_stride_h + (int64_t)slot * a.vc_stride_t + col * 8) = vr;
+    }
+  } else {
+    float s1, s2;
+    int32_t z1, z2;
+    const u32x2_t kc = quantize8<LPR>(kr, s1, z1);
+    const u32x2_t vc = quantize8<LPR>(vr, s2, z2);
+    if (ok) {
+      *(u32x2_t*)((uint8_t*)a.k_cache + b * a.kc_stride_b + hh * a.kc_stride_h + (int64_t)slot * a.kc_stride_t + col * 8) = kc;
+      *(u32x2_t*)((uint8_t*)a.v_cache + b * a.vc_stride_b + hh * a.vc_stride_h + (int64_t)slot * a.vc_stride_t + col * 8) = vc;
+      if (col == 0) {
+        const int64_t so = b * a.qs_stride_b + hh * a.qs_stride_h + slot;
+        a.k_scale[so] = s1;
+        a.k_zp[so] = z1;
+        a.v_scale[so] = s2;
+        a.v_zp[so] = z2;
+      }
+    }
+  }
+  if (ok && col == 0) {
+    a.token_pos[b * a.tp_stride_b + hh * a.tp_stride_h + slot] = a.input_pos + j;
+    if (a.scores) a.scores[b * a.sc_stride_b + hh * a.sc_stride_h + slot] = 0.0f;
+  }
+}
+
+}  // namespace
+
+int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,
+                         int32_t* zp, hipStream_t st) {
+  if (rows == 0) return KVX_OK;
+  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
+  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
+  if (D == 128)
+    hipLaunchKernelGGL((quantize_rows_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  else
+    hipLaunchKernelGGL((quantize_rows_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
+                           int64_t out_row_stride, hipStream_t st) {
+  if (rows == 0) return KVX_OK;
+  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
+  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
+  if (D == 128)
+    hipLaunchKernelGGL((dequantize_rows_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  else
+    hipLaunchKernelGGL((dequantize_rows_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st) {
+  const int64_t total = (int64_t)a.B * a.Hkv * a.num * (a.D / 8);
+  if (total == 0) return KVX_OK;
+  const unsigned grid = (unsigned)((total + NTHREADS - 1) / NTHREADS);
+  const bool u8 = a.kv_dtype == KVX_KV_U8;
+  if (a.D == 128) {
+    if (u8) hipLaunchKernelGGL((cache_write_kernel<128, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else hipLaunchKernelGGL((cache_write_kernel<128, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  } else {
+    if (u8) hipLaunchKernelGGL((cache_write_kernel<64, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else hipLaunchKernelGGL((cache_write_kernel<64, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  }
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+}  // namespace kvx

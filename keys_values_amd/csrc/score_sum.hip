@@ -1,0 +1,247 @@
+// Per-key score-sums W[b,h,k] = (1/G) sum_{i,g} exp2(c * q_{i,g}.k - lse2[b,i,h*G+g]) over the visible
+// (query, key) pairs, for gfx950.
+//
+// Reference behaviour: keys_values/attention/flashinfer_wrapper.py:51-150 (_score_sum_kernel) and
+// :156-273 (host side, division by the group size); the value it must equal is
+// keys_values/attention/base.py:707-725 (mean over the group, sum over queries).
+//
+// Key-stationary: a wavefront keeps the K rows of its 64 keys in registers as MFMA B operands for
+// the whole kernel and owns those 64 outputs, so W needs no atomics and is bit-reproducible. The
+// G*q_len packed query rows (row r = query r / G, head r % G) stream through LDS in tiles of 64 rows,
+// double-buffered, shared by the four wavefronts of the workgroup (256 keys per workgroup).
+// S = Q K^T is computed with rows along M, so a lane owns one key column: the sum over queries is a
+// per-lane running sum and the two halves of the wavefront are added once at the end.
+#include "kvx_common.h"
+
+namespace kvx {
+namespace {
+
+constexpr int BQ = 64;    // query rows per LDS tile
+constexpr int NW = 64;    // keys per wavefront
+constexpr int WAVES = 4;
+constexpr int NTHREADS = WAVES * 64;
+constexpr int BK = NW * WAVES;  // keys per workgroup
+
+struct ScoreParams {
+  const uint16_t* q;
+  const void* k;
+  const float* k_scale;
+  const int32_t* k_zp;
+  const int32_t* tp;
+  const float* lse;
+  float* w;
+  int32_t B, Hq, Hkv, G, q_len, kv_len, R, input_pos;
+  float c, inv_g;
+  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, qs_sb, qs_sh, tp_sb, tp_sh;
+};
+
+template <int D>
+struct Smem {
+  static constexpr int QROW = D + 8;
+  uint16_t q[2][BQ * QROW];
+  float lse[2][BQ];
+  int32_t qpos[2][BQ];
+};
+
+template <int D>
+struct QStage {
+  static constexpr int QCH = (BQ * D / 8) / NTHREADS;  // 4 (D=128), 2 (D=64)
+  u32x4_t qr[QCH];
+  float lse;
+  int32_t qpos;
+};
+
+template <int D>
+__device__ __forceinline__ void fetch_q(QStage<D>& s, const ScoreParams& p, int b, int kvh, int row0, int tid) {
+  constexpr int CPR = D / 8;
+  constexpr int RPI = NTHREADS / CPR;
+  const int col = tid % CPR;
+  const int row_in = tid / CPR;
+#pragma unroll
+  for (int i = 0; i < QStage<D>::QCH; ++i) {
+    const int row = row0 + row_in + i * RPI;
+    const bool ok = row < p.R;
+    const int qi = row / p.G, g = row % p.G;
+    const uint16_t* src = p.q + b * p.q_sb + (int64_t)(kvh * p.G + g) * p.q_sh + (int64_t)qi * p.q_st + col * 8;
+    s.qr[i] = ok ? *(const u32x4_t*)src : u32x4_t{0, 0, 0, 0};
+  }
+  if (tid < BQ) {
+    const int row = row0 + tid;
+    const bool ok = row < p.R;
+    const int qi = row / p.G, g = row % p.G;
+    // rows past the end get lse = +inf so that exp2(... - lse) = 0
+    s.lse = ok ? p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] : INFINITY;
+    s.qpos = ok ? p.input_pos + qi : INT_MAX;
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void commit_q(const QStage<D>& s, Smem<D>& sm, int buf, int tid) {
+  constexpr int CPR = D / 8;
+  constexpr int RPI = NTHREADS / CPR;
+  const int col = tid % CPR;
+  const int row_in = tid / CPR;
+#pragma unroll
+  for (int i = 0; i < QStage<D>::QCH; ++i)
+    *(u32x4_t*)&sm.q[buf][(row_in + i * RPI) * Smem<D>::QROW + col * 8] = s.qr[i];
+  if (tid < BQ) {
+    sm.lse[buf][tid] = s.lse;
+    sm.qpos[buf][tid] = s.qpos;
+  }
+}
+
+template <int D, bool U8>
+__global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParams p) {
+  __shared__ Smem<D> sm;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int n = lane & 31;
+  const int h = lane >> 5;
+  const int group = blockIdx.x;  // fastest: (b, kvh), keeps one KV head's Q stream on one XCD
+  const int b = group / p.Hkv, kvh = group % p.Hkv;
+  const int key0 = blockIdx.y * BK + wave * NW;
+
+  // K fragments (B operand): lane holds key column n of tile nt, d = 16 j + 8 h .. +8
+  bf16x8_t kf[2][D / 16];
+  int32_t tpk[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int key = key0 + nt * 32 + n;
+    const bool ok = key < p.kv_len;
+    tpk[nt] = ok ? (p.tp ? p.tp[b * p.tp_sb + kvh * p.tp_sh + key] : key) : INT_MAX;
+    if constexpr (!U8) {
+      const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st;
+#pragma unroll
+      for (int j = 0; j < D / 16; ++j) {
+        u32x4_t t = ok ? *(const u32x4_t*)(kp + 16 * j + 8 * h) : u32x4_t{0, 0, 0, 0};
+        kf[nt][j] = as_bf16x8(t);
+      }
+    } else {
+      const uint8_t* kp = (const uint8_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st;
+      const int64_t so = b * p.qs_sb + kvh * p.qs_sh + key;
+      const float sc = ok ? p.k_scale[so] : 0.0f;
+      const int32_t zp = ok ? p.k_zp[so] : 0;
+#pragma unroll
+      for (int j = 0; j < D / 16; ++j) {
+        u32x2_t cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
+        u32x4_t t;
+        t[0] = dequant_pair(cc[0] & 0xff, (cc[0] >> 8) & 0xff, zp, sc);
+        t[1] = dequant_pair((cc[0] >> 16) & 0xff, cc[0] >> 24, zp, sc);
+        t[2] = dequant_pair(cc[1] & 0xff, (cc[1] >> 8) & 0xff, zp, sc);
+        t[3] = dequant_pair((cc[1] >> 16) & 0xff, cc[1] >> 24, zp, sc);
+        kf[nt][j] = as_bf16x8(t);
+      }
+    }
+  }
+  // Largest position among this wavefront's keys: query tiles whose smallest position is at least
+  // that need no mask at all (true for every key written before the current chunk).
+  int tpmax = max(tpk[0], tpk[1]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) tpmax = max(tpmax, __shfl_xor(tpmax, off, 64));
+
+  float wacc[2] = {0.0f, 0.0f};
+  const int num_qt = (p.R + BQ - 1) / BQ;
+  QStage<D> st;
+  fetch_q<D>(st, p, b, kvh, 0, tid);
+  commit_q<D>(st, sm, 0, tid);
+  if (num_qt > 1) fetch_q<D>(st, p, b, kvh, BQ, tid);
+  __syncthreads();
+
+  for (int t = 0; t < num_qt; ++t) {
+    const int buf = t & 1;
+    const int qpos_tile_min = p.input_pos + (t * BQ) / p.G;
+    const bool need_mask = tpmax > qpos_tile_min;
+#pragma unroll
+    for (int mt = 0; mt < BQ / 32; ++mt) {
+      f32x16_t s[2];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < D / 16; ++j) {
+        const u32x4_t qq = *(const u32x4_t*)&sm.q[buf][(mt * 32 + n) * Smem<D>::QROW + 16 * j + 8 * h];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], s[nt], 0, 0, 0);
+      }
+      // rows of the accumulator: 8 a + 4 h + (0..3)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const f32x4_t ls = *(const f32x4_t*)&sm.lse[buf][mt * 32 + 8 * a + 4 * h];
+        if (need_mask) {
+          const int4 qp = *(const int4*)&sm.qpos[buf][mt * 32 + 8 * a + 4 * h];
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
+            float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
+            float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
+            float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
+            e0 = tpk[nt] > qp.x ? 0.0f : e0;
+            e1 = tpk[nt] > qp.y ? 0.0f : e1;
+            e2 = tpk[nt] > qp.z ? 0.0f : e2;
+            e3 = tpk[nt] > qp.w ? 0.0f : e3;
+            wacc[nt] += (e0 + e1) + (e2 + e3);
+          }
+        } else {
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
+            const float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
+            const float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
+            const float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
+            wacc[nt] += (e0 + e1) + (e2 + e3);
+          }
+        }
+      }
+    }
+    if (t + 1 < num_qt) {
+      commit_q<D>(st, sm, buf ^ 1, tid);
+      if (t + 2 < num_qt) fetch_q<D>(st, p, b, kvh, (t + 2) * BQ, tid);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const float tot = wacc[nt] + xor32(wacc[nt]);
+    const int key = key0 + nt * 32 + n;
+    if (h == 0 && key < p.kv_len) p.w[((int64_t)b * p.Hkv + kvh) * p.kv_len + key] = tot * p.inv_g;
+  }
+}
+
+template <int D, bool U8>
+int launch_t(const ScoreParams& p, hipStream_t st) {
+  dim3 grid(p.B * p.Hkv, (p.kv_len + BK - 1) / BK);
+  hipLaunchKernelGGL((score_sum_kernel<D, U8>), grid, dim3(NTHREADS), 0, st, p);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+}  // namespace
+
+int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
+  ScoreParams p;
+  p.q = (const uint16_t*)a.q;
+  p.k = a.k;
+  p.k_scale = a.k_scale;
+  p.k_zp = a.k_zp;
+  p.tp = a.token_positions;
+  p.lse = a.lse;
+  p.w = a.w;
+  p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.G = a.Hq / a.Hkv;
+  p.q_len = a.q_len; p.kv_len = a.kv_len; p.R = a.q_len * p.G; p.input_pos = a.input_pos;
+  p.c = a.sm_scale * kLog2e;
+  p.inv_g = 1.0f / (float)p.G;
+  p.q_sb = a.q_stride_b; p.q_sh = a.q_stride_h; p.q_st = a.q_stride_t;
+  p.k_sb = a.k_stride_b; p.k_sh = a.k_stride_h; p.k_st = a.k_stride_t;
+  p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
+  p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
+  const bool u8 = a.kv_dtype == KVX_KV_U8;
+  if (a.D == 128) return u8 ? launch_t<128, true>(p, st) : launch_t<128, false>(p, st);
+  if (a.D == 64) return u8 ? launch_t<64, true>(p, st) : launch_t<64, false>(p, st);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128}", a.D);
+}
+
+}  // namespace kvx

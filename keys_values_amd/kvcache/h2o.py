@@ -1,0 +1,295 @@
+"""
+``H2OKVCache``: the heavy-hitter-oracle cache of the reference on the HIP kernels, with the call
+surface of ``DefaultKVCache`` / ``AttnWeightsKVCache`` / ``H2OKVCache``
+(keys_values/kvcache/base.py:554-595, keys_values/kvcache/attn_weights.py:325-1029,
+keys_values/kvcache/h2o.py:28-263): ``forward(query, key, value, token_idx)``, ``next_positions``,
+``token_positions``, ``max_forward_length``, ``_update``, the buffers ``token_pos`` (int32),
+``scores`` (float32) and the K/V buffers ``(max_batch, n_query_groups, cache_length, head_size)``.
+
+One ``forward`` is, in the reference's order (keys_values/kvcache/base.py:554-595): write the new
+tokens into the slots chosen last time (resetting their score), attend over the cache with the
+position mask, add the score-sums to the cumulative scores, choose the next slots to evict.
+
+The K/V store is either bf16 (``h2o-default``) or uint8 codes with per-row scale / zero point
+(``h2o-torch-quantized8``, keys_values/kvcache/factory.py:50-66). In the second case the codes stay
+resident and the attention kernels dequantise them on load; the reference instead dequantises the
+whole cache into a bf16 working buffer per layer and re-quantises it afterwards
+(keys_values/kvcache/quant_buffers.py:473-503,732-804).
+
+Not covered (raises): grace period, replay log, fp16/fp32 caches.
+"""
+import ctypes
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ..attention import ops
+
+DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
+MAX_SELECT = 4096  # largest k of kvx_h2o_update_select
+
+
+@dataclass(frozen=True)
+class KVCacheParams:
+    """keys_values/kvcache/base.py:29-66."""
+
+    max_batch_size: int
+    n_query_groups: int
+    cache_length: int
+    head_size: int
+    n_head: int
+    dtype: Optional[torch.dtype] = torch.bfloat16
+
+
+class H2OKVCache:
+    def __init__(
+        self,
+        params: KVCacheParams,
+        max_chunk_size: Optional[int] = None,
+        normalize_scores: bool = False,
+        grace_period: int = 0,
+        quantized: bool = False,
+        keep_initial_fraction: float = DEFAULT_KEEP_INITIAL_FRACTION,
+        device: Optional[torch.device] = None,
+    ):
+        if grace_period != 0:
+            raise NotImplementedError("grace_period > 0 is not implemented")
+        if params.dtype not in (None, torch.bfloat16):
+            raise NotImplementedError(f"cache dtype {params.dtype}: the kernels take bfloat16")
+        if params.head_size not in (64, 128):
+            raise NotImplementedError(f"head_size = {params.head_size} not in (64, 128)")
+        if params.n_head % params.n_query_groups != 0:
+            raise ValueError("n_head must be a multiple of n_query_groups")
+        self.params = params
+        self.max_batch_size = params.max_batch_size
+        self.n_query_groups = params.n_query_groups
+        self.n_head = params.n_head
+        self.cache_length = params.cache_length
+        self.head_size = params.head_size
+        self.dtype = torch.bfloat16
+        self.grace_period = 0
+        self.normalize_scores = normalize_scores
+        self.quantized = quantized
+        # keys_values/kvcache/attn_weights.py:458-462: silently disabled when too large
+        if max_chunk_size is not None and max_chunk_size > self.cache_length // 2:
+            max_chunk_size = None
+        self.max_chunk_size = max_chunk_size
+        self._select_k = min(self.cache_length, MAX_SELECT) if max_chunk_size is None else min(max_chunk_size, MAX_SELECT)
+        self._keep_initial_fraction = keep_initial_fraction
+        self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        if self.device.type != "cuda":
+            raise RuntimeError(f"H2OKVCache buffers live on a ROCm device, not on {self.device}: there is no CPU path")
+        b, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
+        kv_dtype = torch.uint8 if quantized else torch.bfloat16
+        self.k = torch.zeros((b, h, length, d), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
+        self.v = torch.zeros((b, h, length, d), dtype=kv_dtype, device=self.device)
+        if quantized:
+            self.k_scale = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)
+            self.k_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
+            self.v_scale = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)
+            self.v_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
+        self.token_pos = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)  # attn_weights.py:466-470
+        self.scores = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)  # h2o.py:85-91
+        self._next_index = torch.zeros((b, h, self._select_k), dtype=torch.int32, device=self.device)
+        self._have_next = False
+        self._use_initial_rule = None
+        self._input_pos = 0
+        self.batch_size = None
+        self.current_length = None
+        self.prefill_length = None
+        self.scale_factor = 1.0 / (self.head_size ** 0.5)
+
+    # -- bookkeeping -----------------------------------------------------------------------------
+
+    @property
+    def input_pos(self) -> int:
+        return self._input_pos
+
+    @property
+    def max_prefill_length(self) -> int:
+        return self.cache_length  # keys_values/kvcache/base.py:707-709
+
+    def max_forward_length(self) -> int:
+        """keys_values/kvcache/attn_weights.py:501-508."""
+        diff = self.cache_length - self.current_length
+        result = self.cache_length
+        if diff > 0:
+            result = min(result, diff)
+        if self.max_chunk_size is not None:
+            result = min(result, self.max_chunk_size)
+        return min(result, self._select_k) if diff == 0 else result
+
+    def token_positions(self) -> torch.Tensor:
+        if self.current_length is None:
+            raise IndexError("Cache is not initialized, call 'prefill' first")
+        return self.token_pos[: self.batch_size, :, : self.current_length]
+
+    def next_positions(self, num: int) -> Optional[torch.Tensor]:
+        """Slots the next ``forward`` writes to, int64 (batch, n_query_groups, num), or None
+        (keys_values/kvcache/attn_weights.py:490-499)."""
+        idx = self._next_index_for(num, peek=True)
+        return None if idx is None else idx.to(torch.int64)
+
+    def _quant_state(self, T: int) -> Optional[ops.QuantState]:
+        if not self.quantized:
+            return None
+        b = self.batch_size
+        return ops.QuantState(self.k_scale[:b, :, :T], self.k_zp[:b, :, :T], self.v_scale[:b, :, :T], self.v_zp[:b, :, :T])
+
+    def _next_index_for(self, num: int, peek: bool = False) -> Optional[torch.Tensor]:
+        b, h = self.batch_size, self.n_query_groups
+        if self.current_length is None:
+            return None
+        if self.current_length < self.cache_length:  # free slots, attn_weights.py:1001-1016
+            start = self.current_length
+            return torch.arange(start, start + num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, h, -1).contiguous()
+        if self._use_initial_rule:  # attn_weights.py:536-550
+            n0 = min(int(self._keep_initial_fraction * self.cache_length), self.cache_length - num)
+            if not peek:
+                self._use_initial_rule = False
+            return torch.arange(n0, n0 + num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, h, -1).contiguous()
+        if not self._have_next:
+            return None
+        return self._next_index[:b, :, :num]
+
+    # -- the step (keys_values/kvcache/base.py:554-595) -----------------------------------------
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, token_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """query (B, n_head, num, hs); key/value (B, n_query_groups, num, hs). Returns the attention
+        output (B, num, n_head * hs) (keys_values/attention/base.py:378-380)."""
+        _lib.require_gpu(query, key, value)
+        if query.ndim != 4 or key.ndim != 4 or key.shape != value.shape:
+            raise ValueError("query, key, value must be 4D and key.shape == value.shape")
+        b, hq, num, d = query.shape
+        if key.shape != (b, self.n_query_groups, num, d) or hq != self.n_head or d != self.head_size:
+            raise ValueError(f"shapes {tuple(query.shape)}, {tuple(key.shape)} do not fit the cache")
+        input_pos = self._input_pos
+        if input_pos == 0:
+            return self._prefill_step(query, key, value)
+        if b != self.batch_size:
+            raise ValueError(f"batch size {b} differs from the prefill batch size {self.batch_size}")
+        if self._use_initial_rule is None:
+            raise IndexError("Cache needs to be initialized with 'prefill' before being used")
+        diff = self.cache_length - self.current_length
+        if not 1 <= num <= self.max_forward_length():
+            if 0 < diff < num:
+                raise ValueError(f"key.shape[2] = {num}, must be <= {diff} as long as the cache is not full")
+            raise ValueError(f"key.shape[2] = {num}, must be in [1, {self.max_forward_length()}]")
+        index = self._next_index_for(num)
+        if index is None:
+            raise IndexError("Cache needs to be initialized with 'prefill' before being used")
+        self._write(index, key, value, input_pos)
+        if diff > 0:
+            self.current_length += num
+        self._have_next = False
+        self._input_pos += num
+        T = self.current_length
+        kc, vc = self.k[:b, :, :T], self.v[:b, :, :T]
+        tp = self.token_pos[:b, :, :T]
+        quant = self._quant_state(T)
+        if num == 1:
+            out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
+            out = out.unsqueeze(1)
+        else:
+            out, w, _ = ops.prefill_core(query, kc, vc, self.scale_factor, input_pos, tp, return_weights=True,
+                                         output_transposed=True, quant=quant)
+        self._update(w, num)
+        return out.reshape(b, num, hq * d)
+
+    __call__ = forward
+
+    def _prefill_step(self, query, key, value):
+        """keys_values/kvcache/attn_weights.py:817-869 and keys_values/kvcache/base.py:567-581: fill the
+        first slots, positions = arange, scores = 0, plain causal attention on the chunk, no weights."""
+        b, hq, num, d = query.shape
+        if not (0 < b <= self.max_batch_size):
+            raise ValueError(f"batch size {b} must be in (0, {self.max_batch_size}]")
+        if num > self.max_prefill_length:
+            raise ValueError(f"prefill length {num} exceeds cache_length {self.cache_length}")
+        self.batch_size = b
+        index = torch.arange(num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, self.n_query_groups, -1).contiguous()
+        self.scores.zero_()
+        self.current_length = num
+        self._write(index, key, value, 0)
+        self.prefill_length = num
+        self._use_initial_rule = num == self.cache_length
+        self._have_next = False
+        self._input_pos = num
+        out, _, _ = ops.prefill_core(query, key.to(torch.bfloat16), value.to(torch.bfloat16), self.scale_factor, 0, None,
+                                     return_weights=False, output_transposed=True)
+        return out.reshape(b, num, hq * d)
+
+    def _write(self, index: torch.Tensor, key: torch.Tensor, value: torch.Tensor, input_pos: int):
+        b, h, num = index.shape
+        key = key.to(torch.bfloat16)
+        value = value.to(torch.bfloat16)
+        if key.stride(-1) != 1:
+            key = key.contiguous()
+        if value.stride(-1) != 1:
+            value = value.contiguous()
+        a = _lib.CacheWriteArgs()
+        a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, self.head_size, self.cache_length
+        a.input_pos = input_pos
+        a.kv_dtype = _lib.KVX_KV_U8 if self.quantized else _lib.KVX_KV_BF16
+        a.index = index.data_ptr()
+        a.index_stride_b, a.index_stride_h = index.stride(0), index.stride(1)
+        a.key = key.data_ptr()
+        a.key_stride_b, a.key_stride_h, a.key_stride_t = key.stride(0), key.stride(1), key.stride(2)
+        a.value = value.data_ptr()
+        a.value_stride_b, a.value_stride_h, a.value_stride_t = value.stride(0), value.stride(1), value.stride(2)
+        a.k_cache = self.k.data_ptr()
+        a.kc_stride_b, a.kc_stride_h, a.kc_stride_t = self.k.stride(0), self.k.stride(1), self.k.stride(2)
+        a.v_cache = self.v.data_ptr()
+        a.vc_stride_b, a.vc_stride_h, a.vc_stride_t = self.v.stride(0), self.v.stride(1), self.v.stride(2)
+        if self.quantized:
+            a.k_scale, a.k_zp = self.k_scale.data_ptr(), self.k_zp.data_ptr()
+            a.v_scale, a.v_zp = self.v_scale.data_ptr(), self.v_zp.data_ptr()
+            a.qs_stride_b, a.qs_stride_h = self.k_scale.stride(0), self.k_scale.stride(1)
+        a.token_pos = self.token_pos.data_ptr()
+        a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
+        a.scores = self.scores.data_ptr()
+        a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
+
+    def _update(self, attn_weights: torch.Tensor, query_length: int):
+        """keys_values/kvcache/attn_weights.py:721-783 with keys_values/kvcache/h2o.py:146-199."""
+        if not isinstance(attn_weights, torch.Tensor):
+            raise TypeError("attn_weights argument needs to be torch.Tensor")
+        if not isinstance(query_length, int) or query_length <= 0:
+            raise TypeError("query_length argument needs to be positive int")
+        shape = (self.batch_size, self.n_query_groups, self.current_length)
+        if tuple(attn_weights.shape) != shape:
+            raise ValueError(f"Shape of attn_weights must be {shape}, but attn_weights.shape = {tuple(attn_weights.shape)}")
+        if attn_weights.dtype != torch.float32:
+            raise ValueError(f"attn_weights.dtype={attn_weights.dtype}, must be {torch.float32}")
+        _lib.require_gpu(attn_weights)
+        attn_weights = attn_weights.contiguous()
+        full = self.current_length == self.cache_length
+        a = _lib.H2OArgs()
+        a.B, a.Hkv, a.kv_len = self.batch_size, self.n_query_groups, self.current_length
+        a.limit = self.current_length
+        a.k = self._select_k if full else 1
+        a.normalize = int(self.normalize_scores and full)
+        a.input_pos = self._input_pos
+        a.prefill_len = self.prefill_length
+        a.scores = self.scores.data_ptr()
+        a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
+        a.w = attn_weights.data_ptr()
+        a.token_pos = self.token_pos.data_ptr()
+        a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            if full:
+                nxt = self._next_index
+            else:  # only the accumulation matters while slots are free; the choice is discarded
+                nxt = torch.empty((self.batch_size, self.n_query_groups, 1), dtype=torch.int32, device=self.device)
+            a.next_index = nxt.data_ptr()
+            nbytes = lib.kvx_h2o_workspace_bytes(ctypes.byref(a))
+            ws = _lib.workspace(self.device, nbytes)
+            a.workspace = _lib.ptr(ws)
+            a.workspace_bytes = 0 if ws is None else ws.numel()
+            _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
+        self._have_next = full
