@@ -1,0 +1,305 @@
+#!/usr/bin/env python3
+"""
+Benchmark of the attention-with-score-sums hot path on one MI355X.
+
+Default workload (`--workload prefill`): the Qwen3-4B-shaped chunked prefill of BASELINE.json
+(batch 1, 32 query / 8 KV heads, head size 128, 32768 cached positions, a 1024-query chunk appended
+causally at the end, bf16, RoPE theta 1e6, seed 1). One step = attention output + base-2 LSE +
+per-key score-sums for the whole chunk: the prefill kernel followed by the score-sum kernel.
+Inputs are resident in HBM before the timed region.
+
+`--workload decode`  : single-token decode over a bf16 cache with score-sums, H2O score update and
+                       argmin (batch 8, 32/8 heads, 131072 positions), GB/s against HBM peak.
+`--workload quantize`: affine uint8 row quantiser on (1, 8, 65536, 128) K and V, GB/s.
+
+Prints ONE JSON line (see the keys below). `roofline` describes the dominant kernel, timed with
+events on the launch stream inside the timed steps; `cpu_baseline` times the CPU oracle (the
+reference's eager op sequence restated) on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--splits", type=int, default=0)
+    return ap.parse_args()
+
+
+def rope_inputs(torch, O, dev):
+    B, Hq, Hkv, q_len, T, D, input_pos = 1, 32, 8, 1024, 32768, 128, 31744
+    gen = torch.Generator().manual_seed(1)
+    q = torch.randn(B, Hq, q_len, D, generator=gen)
+    k = torch.randn(B, Hkv, T, D, generator=gen)
+    v = torch.randn(B, Hkv, T, D, generator=gen).to(torch.bfloat16)
+    q = O.apply_rope(q, torch.arange(input_pos, input_pos + q_len)).to(torch.bfloat16)
+    k = O.apply_rope(k, torch.arange(T)).to(torch.bfloat16)
+    return (B, Hq, Hkv, q_len, T, D, input_pos), q, k, v
+
+
+def bench_prefill(args, torch, dev):
+    from keys_values_amd import _lib
+    from keys_values_amd.attention import ops
+    from oracle import kvx_oracle as O
+
+    lib = _lib.load()
+    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev)
+    scale = D ** -0.5
+    q, k, v = q_c.to(dev), k_c.to(dev), v_c.to(dev)
+    out = torch.empty((B, q_len, Hq, D), dtype=torch.bfloat16, device=dev)
+    o_view = out.permute(0, 2, 1, 3)
+    lse = torch.empty((B, q_len, Hq), dtype=torch.float32, device=dev)
+    w = torch.empty((B, Hkv, T), dtype=torch.float32, device=dev)
+    a = _lib.SdpaArgs()
+    ops._fill_common(a, q, k, v, scale, input_pos, None, None, args.splits)
+    a.o = o_view.data_ptr()
+    a.o_stride_b, a.o_stride_h, a.o_stride_t = o_view.stride(0), o_view.stride(1), o_view.stride(2)
+    a.lse, a.w = lse.data_ptr(), w.data_ptr()
+    nbytes = lib.kvx_sdpa_prefill_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    st = _lib.stream_ptr(dev)
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        _lib.check(lib.kvx_sdpa_prefill(ctypes.byref(a), st))
+        if ev is not None:
+            ev[1].record()
+        _lib.check(lib.kvx_score_sum(ctypes.byref(a), st))
+        if ev is not None:
+            ev[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_step = (t1 - t0) * 1e3 / args.steps
+    ms_attn = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    ms_score = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+
+    flops_alg = 4.0 * B * Hq * q_len * T * D        # QK^T + PV: credited for O, LSE and W together
+    flops_issued = 6.0 * B * Hq * q_len * T * D     # the score-sum pass repeats QK^T
+    tflops = flops_alg / (ms_step * 1e-3) / 1e12
+    attn_tflops = flops_alg / (ms_attn * 1e-3) / 1e12
+
+    # sanity of the timed outputs (cheap invariants; the parity tests do the real checking)
+    rows = w.sum(-1).cpu()
+    assert torch.allclose(rows, torch.full_like(rows, float(q_len)), rtol=1e-4, atol=5e-2), rows
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        # bounded sample: KV head 0 with its 4 query heads = 1/8 of the workload, same op sequence
+        # as the reference's eager path (fp32 upcast, <= 3 GB score slices, mask, softmax, mean/sum)
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        hs = 1
+        qs, ks, vs = q_c[:, : 4 * hs], k_c[:, :hs], v_c[:, :hs]
+        t_c0 = time.perf_counter()
+        o_ref, w_ref = O.sdpa_in_blocks(qs, ks, vs, scale, input_pos, None)
+        t_c = time.perf_counter() - t_c0
+        cpu = {
+            "value": round(flops_alg * hs / Hkv / t_c / 1e12, 4),
+            "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"KV head 0 of {Hkv} (4 query heads x 1024 queries x 32768 keys), one pass, {t_c:.1f} s",
+        }
+        # the sample doubles as an end-to-end check of the timed outputs
+        err = ((out.permute(0, 2, 1, 3)[:, : 4 * hs].float().cpu() - o_ref.float()).norm() / o_ref.float().norm()).item()
+        assert err < 2e-2, err
+        torch.testing.assert_close(w[:, :hs].cpu(), w_ref, rtol=1e-3, atol=1e-6)
+
+    return {
+        "metric": "attn+score-sum TFLOP/s (% MFMA peak); H2O prefill tok/s, Qwen3-4B shape",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE.json configs[1]: chunked prefill attention + score-sum, B1 Hq32 Hkv8 D128 T32768 q1024, RoPE theta 1e6, seed 1",
+            "flops_algorithmic": flops_alg,
+            "flops_issued": flops_issued,
+            "pct_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+            "chunk_tokens_per_s": round(q_len / (ms_step * 1e-3), 1),
+            "ms_attention_kernel": round(ms_attn, 4),
+            "ms_score_sum_kernel": round(ms_score, 4),
+            "score_sum_tflops": round(2.0 * B * Hq * q_len * T * D / (ms_score * 1e-3) / 1e12, 2),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "sdpa_prefill_kernel<128,false> (+ split merge)",
+            "achieved": round(attn_tflops, 2),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
+            "traffic": None,
+        },
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_quantize(args, torch, dev):
+    from keys_values_amd import _lib
+    from oracle import kvx_oracle as O
+
+    lib = _lib.load()
+    rows, D = 8 * 65536, 128
+    gen = torch.Generator().manual_seed(2)
+    kx = torch.randn(rows, D, generator=gen)
+    mask = torch.rand(rows, D, generator=gen) < 0.01
+    kx = torch.where(mask, torch.randn(rows, D, generator=gen) * 8, kx).to(torch.bfloat16)
+    vx = torch.randn(rows, D, generator=gen).to(torch.bfloat16)
+    xs = [kx.to(dev), vx.to(dev)]
+    outs = [(torch.empty((rows, D), dtype=torch.uint8, device=dev), torch.empty(rows, dtype=torch.float32, device=dev),
+             torch.empty(rows, dtype=torch.int32, device=dev)) for _ in xs]
+    st = _lib.stream_ptr(dev)
+
+    def step():
+        for x, (c, s, z) in zip(xs, outs):
+            _lib.check(lib.kvx_quantize_rows(x.data_ptr(), D, rows, D, c.data_ptr(), s.data_ptr(), z.data_ptr(), st))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_kernel = e0.elapsed_time(e1) / args.steps / 2
+    bytes_alg = rows * (2 * D + D + 8)  # per tensor: bf16 in, codes + fp32 scale + int32 zero point out
+    gbs = 2 * bytes_alg / (ms_step * 1e-3) / 1e9
+    kgbs = bytes_alg / (ms_kernel * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        t_c0 = time.perf_counter()
+        c_ref, s_ref, z_ref = O.quantize_rows(kx)
+        t_c = time.perf_counter() - t_c0
+        cpu = {"value": round(bytes_alg / t_c / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"K tensor only (half the workload), one pass, {t_c:.1f} s"}
+        assert torch.equal(outs[0][0].cpu(), c_ref) and torch.equal(outs[0][1].cpu(), s_ref) and torch.equal(outs[0][2].cpu(), z_ref)
+    return {
+        "metric": "uint8 row quantiser GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "BASELINE.json configs[2] quantiser: K and V (1, 8, 65536, 128) bf16 -> uint8 + fp32 scale + int32 zero point, seed 2",
+                   "bytes_algorithmic_per_tensor": bytes_alg},
+        "roofline": {"bound": "hbm", "kernel": "quantize_rows_kernel<128>", "achieved": round(kgbs, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(kgbs / PEAK_HBM_GBS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_decode(args, torch, dev):
+    from keys_values_amd import _lib
+    from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
+    from oracle import kvx_oracle as O
+
+    B, Hq, Hkv, L, D = 8, 32, 8, 131072, 128
+    gen = torch.Generator(device=dev).manual_seed(3)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, device=dev)
+    # state as after a prefill that filled the cache (the prefill itself is not part of this workload)
+    cache.k.copy_(torch.randn(cache.k.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
+    cache.v.copy_(torch.randn(cache.v.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
+    cache.token_pos.copy_(torch.arange(L, dtype=torch.int32, device=dev).view(1, 1, L).expand(B, Hkv, L))
+    cache.batch_size, cache.current_length, cache.prefill_length = B, L, L
+    cache._input_pos = L
+    cache._use_initial_rule = False
+    cache._next_index.zero_()
+    cache._have_next = True
+    n = args.steps + args.warmup
+    qs = torch.randn((n, B, Hq, 1, D), generator=gen, device=dev).to(torch.bfloat16)
+    ks = torch.randn((n, B, Hkv, 1, D), generator=gen, device=dev).to(torch.bfloat16)
+    vs = torch.randn((n, B, Hkv, 1, D), generator=gen, device=dev).to(torch.bfloat16)
+    for i in range(args.warmup):
+        cache.forward(qs[i], ks[i], vs[i])
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(args.warmup, n):
+        cache.forward(qs[i], ks[i], vs[i])
+    e1.record()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_gpu = e0.elapsed_time(e1) / args.steps
+    bytes_alg = 2 * B * Hkv * L * D * 2 + 2 * B * Hkv * L * 4  # K + V once, scores read-modify-write
+    gbs = bytes_alg / (ms_step * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        kc, vc = cache.k[:1, :2].cpu(), cache.v[:1, :2].cpu()
+        t_c0 = time.perf_counter()
+        O.sdpa_in_blocks(qs[0, :1, :8].cpu(), kc, vc, D ** -0.5, L, None)
+        t_c = time.perf_counter() - t_c0
+        frac = (1 * 2) / (B * Hkv)
+        cpu = {"value": round(bytes_alg * frac / t_c / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"attention part of one step for batch 0, KV heads 0-1 (1/32 of a step), {t_c:.1f} s"}
+    return {
+        "metric": "decode + H2O step GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3",
+                   "bytes_algorithmic_per_step": bytes_alg, "ms_per_step_gpu_events": round(ms_gpu, 4),
+                   "decode_tokens_per_s": round(B / (ms_step * 1e-3), 1)},
+        "roofline": {"bound": "hbm", "kernel": "whole decode step (cache write, split attention, merge, weights, score update + argmin)",
+                     "achieved": round(bytes_alg / (ms_gpu * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(bytes_alg / (ms_gpu * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards without communication over KV heads; "
+              "see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device visible; the kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode}[args.workload]
+    res = fn(args, torch, dev)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

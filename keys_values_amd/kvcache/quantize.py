@@ -172,5 +172,5 @@ class RowQuantizer8:
             back = torch.empty((rows, d), dtype=self.source_dtype, device=dev)
             _lib.check(lib.kvx_quantize_rows(xs.data_ptr(), d, rows, d, codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), st))
             _lib.check(lib.kvx_dequantize_rows(codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), rows, d, back.data_ptr(), d, st))
-        err = torch.linalg.vector_norm(xs.to(torch.float32) - back.to(torch.float32), dim=-1)
+        err = torch.linalg.vector_norm(xs - back, dim=-1, dtype=torch.float32)  # difference in the source dtype, as the reference
         return err.reshape(x.shape[:-1])

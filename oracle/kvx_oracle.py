@@ -227,9 +227,10 @@ def dequantize_rows(codes: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, 
 
 
 def quantization_error(x: torch.Tensor) -> torch.Tensor:
-    """keys_values/kvcache/quantize/pytorch.py:530-548: per-row L2 norm of x - dequant(quant(x))."""
+    """keys_values/kvcache/quantize/pytorch.py:530-548: per-row L2 norm of x - dequant(quant(x)); the
+    dequantised rows and the difference are in the source dtype, the norm accumulates in float32."""
     c, s, z = quantize_rows(x)
-    return torch.linalg.vector_norm(x.to(torch.float32) - dequantize_rows(c, s, z, torch.float32), dim=-1)
+    return torch.linalg.vector_norm(x - dequantize_rows(c, s, z, x.dtype), dim=-1, dtype=torch.float32)
 
 
 # --------------------------------------------------------------------------------------------

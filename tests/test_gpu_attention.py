@@ -1,0 +1,200 @@
+"""GPU parity of the attention kernels against the CPU oracle, through the C ABI (ctypes)."""
+import math
+
+import pytest
+import torch
+
+from helpers import make_qkv, rel_err, scattered_positions
+from keys_values_amd.attention import ops
+from keys_values_amd.attention.sdpa import HipSDPA
+from oracle import kvx_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# tolerances of the path: outputs 2e-2 relative (bf16), score-sums 1e-3 relative (fp32 accumulation)
+O_RTOL = 2e-2
+W_RTOL = 1e-3
+
+
+def check_o(o_gpu, o_ref):
+    o_gpu = o_gpu.float().cpu()
+    o_ref = o_ref.float()
+    assert rel_err(o_gpu, o_ref) < O_RTOL
+    torch.testing.assert_close(o_gpu, o_ref, rtol=O_RTOL, atol=2e-2)
+
+
+def check_w(w_gpu, w_ref, q_len):
+    w_gpu = w_gpu.cpu()
+    assert w_gpu.dtype == torch.float32
+    assert (w_gpu >= 0).all()
+    torch.testing.assert_close(w_gpu, w_ref, rtol=W_RTOL, atol=1e-6)
+    torch.testing.assert_close(w_gpu.sum(-1), torch.full(w_gpu.shape[:2], float(q_len)), rtol=5e-5, atol=3e-4)
+
+
+CASES = [
+    # B, Hq, Hkv, q_len, T, D, input_pos, scattered, splits
+    (1, 8, 2, 128, 1024, 64, 896, False, 0),     # configuration 1 shapes
+    (1, 8, 2, 128, 1024, 64, 896, True, 2),
+    (2, 4, 4, 16, 200, 128, 300, True, 1),       # G = 1, ragged T
+    (1, 8, 2, 100, 333, 128, 233, False, 3),     # ragged rows and keys, 3 splits
+    (2, 8, 1, 37, 700, 128, 1000, True, 0),      # G = 8
+    (1, 32, 8, 64, 192, 128, 128, False, 1),     # the reference's fused-prefill test shape
+    (1, 4, 2, 2, 64, 64, 62, False, 1),
+    (1, 4, 2, 300, 300, 128, 0, False, 2),       # square causal prefill (input_pos = 0)
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,q_len,T,D,input_pos,scattered,splits", CASES)
+def test_prefill_with_weights(gpu, B, Hq, Hkv, q_len, T, D, input_pos, scattered, splits):
+    q, k, v, gen = make_qkv(100 + T + q_len, B, Hq, Hkv, q_len, T, D)
+    tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len) if scattered else None
+    if tp is None and input_pos != T - q_len:
+        tp = (torch.arange(T, dtype=torch.int32) + (input_pos - (T - q_len))).view(1, 1, T).expand(B, Hkv, T).contiguous()
+    scale = 1.0 / math.sqrt(D)
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, None if tp is None else tp.to(torch.int64))
+    l_ref = O.lse2(q, k, scale, input_pos, tp)
+    out, w, lse = ops.prefill_core(
+        q.to(gpu), k.to(gpu), v.to(gpu), scale, input_pos, None if tp is None else tp.to(gpu),
+        return_weights=True, return_lse=True, output_transposed=False, num_splits=splits,
+    )
+    torch.cuda.synchronize()
+    check_o(out, o_ref)
+    torch.testing.assert_close(lse.cpu(), l_ref, rtol=1e-4, atol=1e-3)
+    check_w(w, w_ref, q_len)
+
+
+def test_prefill_strided_cache_views_and_layouts(gpu):
+    # K/V as views k[:B, :, :T] of a larger (Bmax, Hkv, L, D) allocation
+    # (keys_values/kvcache/buffers.py:538-541) and the extension's [B, len, H, D] layout
+    B, Hq, Hkv, q_len, T, D, L = 2, 8, 2, 48, 160, 128, 256
+    q, k, v, gen = make_qkv(5, B, Hq, Hkv, q_len, T, D)
+    tp = scattered_positions(gen, B, Hkv, T, 400, q_len)
+    scale = 0.09
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, 400, tp.to(torch.int64))
+    kbuf = torch.zeros(3, Hkv, L, D, dtype=torch.bfloat16, device=gpu)
+    vbuf = torch.zeros(3, Hkv, L, D, dtype=torch.bfloat16, device=gpu)
+    tpbuf = torch.zeros(3, Hkv, L, dtype=torch.int32, device=gpu)
+    kbuf[:B, :, :T] = k.to(gpu)
+    vbuf[:B, :, :T] = v.to(gpu)
+    tpbuf[:B, :, :T] = tp.to(gpu)
+    out, w, _ = ops.prefill_core(q.to(gpu), kbuf[:B, :, :T], vbuf[:B, :, :T], scale, 400, tpbuf[:B, :, :T], return_weights=True)
+    assert out.shape == (B, q_len, Hq, D)
+    check_o(out.permute(0, 2, 1, 3), o_ref)
+    check_w(w, w_ref, q_len)
+    # reference extension layout, right-aligned causal
+    o2_ref, w2_ref = O.sdpa_in_blocks(q, k, v, scale, T - q_len, None)
+    out2, w2, lse2 = ops.sdpa_prefill(
+        q.to(gpu).transpose(1, 2).contiguous(), k.to(gpu).transpose(1, 2).contiguous(), v.to(gpu).transpose(1, 2).contiguous(),
+        scale, return_weights=True, return_lse=True,
+    )
+    check_o(out2.permute(0, 2, 1, 3), o2_ref)
+    check_w(w2, w2_ref, q_len)
+    torch.testing.assert_close(lse2.cpu(), O.lse2(q, k, scale, T - q_len, None), rtol=1e-4, atol=1e-3)
+
+
+def test_score_sum_from_given_lse(gpu):
+    # the score-sum kernel alone, fed the oracle's LSE (as the reference tests its Triton kernel,
+    # test/attention/test_flashinfer_wrapper.py:1207-1307)
+    B, Hq, Hkv, q_len, T, D = 1, 8, 2, 70, 530, 128
+    q, k, v, gen = make_qkv(77, B, Hq, Hkv, q_len, T, D)
+    tp = scattered_positions(gen, B, Hkv, T, 600, q_len)
+    scale = 1.0 / math.sqrt(D)
+    _, w_ref = O.sdpa_in_blocks(q, k, v, scale, 600, tp.to(torch.int64))
+    lse = O.lse2(q, k, scale, 600, tp)
+    w = ops.score_sum_core(q.to(gpu), k.to(gpu), lse.to(gpu), scale, 600, tp.to(gpu))
+    check_w(w, w_ref, q_len)
+
+
+def test_causal_weights_decay(gpu):
+    # test/attention/test_flashinfer_wrapper.py:1074-1124: early keys collect far more weight
+    q, k, v, _ = make_qkv(3, 1, 8, 2, 64, 64, 64)
+    _, w, _ = ops.prefill_core(q.to(gpu), k.to(gpu), v.to(gpu), 0.125, 0, None, return_weights=True)
+    w = w.cpu()
+    assert (w[:, :, 0] > 2 * w[:, :, -1]).all()
+
+
+def test_hip_sdpa_dropin(gpu):
+    # FlashInferSDPA surface incl. head-size padding (keys_values/attention/flashinfer_wrapper.py:276-308)
+    B, Hq, Hkv, q_len, T, D = 1, 4, 2, 20, 90, 48
+    q, k, v, gen = make_qkv(42, B, Hq, Hkv, q_len, T, D)
+    tp = scattered_positions(gen, B, Hkv, T, 111, q_len)
+    sdpa = HipSDPA()
+    assert sdpa.available
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, 1 / math.sqrt(D), 111, tp.to(torch.int64))
+    out, w = sdpa.scaled_dot_product_attention(q.to(gpu), k.to(gpu), v.to(gpu), None, 111, tp.to(gpu), return_attn_weights=True)
+    assert out.shape == (B, Hq, q_len, D) and w.shape == (B, Hkv, T)
+    check_o(out, o_ref)
+    check_w(w, w_ref, q_len)
+    out_t, w_none = sdpa.scaled_dot_product_attention(q.to(gpu), k.to(gpu), v.to(gpu), None, 111, tp.to(gpu), output_transposed=True)
+    assert w_none is None and out_t.shape == (B, q_len, Hq, D)
+    check_o(out_t.transpose(1, 2), o_ref)
+    # q_len == 1 routes to the decode kernel and ignores positions
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], k, v, 1 / math.sqrt(D), 10**6, None)
+    out1, w1 = sdpa.scaled_dot_product_attention(q[:, :, :1].to(gpu), k.to(gpu), v.to(gpu), None, 500, tp.to(gpu), return_attn_weights=True)
+    check_o(out1, o1_ref)
+    check_w(w1, w1_ref, 1)
+
+
+DECODE_CASES = [
+    # B, Hq, Hkv, T, D, splits
+    (2, 8, 2, 1000, 128, 0),
+    (1, 32, 8, 4096 + 77, 128, 0),
+    (3, 4, 4, 130, 64, 1),
+    (1, 8, 1, 5000, 128, 3),
+    (2, 4, 2, 17, 64, 0),
+    (1, 8, 2, 9000, 64, 2),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,D,splits", DECODE_CASES)
+def test_decode_with_weights(gpu, B, Hq, Hkv, T, D, splits):
+    q, k, v, _ = make_qkv(900 + T, B, Hq, Hkv, 1, T, D)
+    scale = 1.0 / math.sqrt(D)
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, T - 1, None)
+    l_ref = O.lse2(q, k, scale, T - 1, None)
+    out, w, lse = ops.decode_core(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_weights=True, return_lse=True, num_splits=splits)
+    torch.cuda.synchronize()
+    check_o(out.unsqueeze(2), o_ref)
+    torch.testing.assert_close(lse.cpu(), l_ref, rtol=1e-4, atol=1e-3)
+    check_w(w, w_ref, 1)
+    # reference extension layout
+    out2, w2 = ops.sdpa_decode(q[:, :, 0].to(gpu), k.to(gpu).transpose(1, 2).contiguous(), v.to(gpu).transpose(1, 2).contiguous(), scale, return_weights=True)
+    check_o(out2.unsqueeze(2), o_ref)
+    check_w(w2, w_ref, 1)
+    out3, w3 = ops.sdpa_decode(q[:, :, 0].to(gpu), k.to(gpu).transpose(1, 2).contiguous(), v.to(gpu).transpose(1, 2).contiguous(), scale)
+    assert w3 is None
+    check_o(out3.unsqueeze(2), o_ref)
+
+
+def test_full_size_prefill_properties(gpu):
+    """Configuration 2 at its real shape (B1, 32/8 heads, D128, 32768 slots, 1024 queries, RoPE):
+    one KV head against the oracle, row sums, and layout independence (scattered slots give the
+    same O and, after un-permuting, the same W as the contiguous layout)."""
+    B, Hq, Hkv, q_len, T, D, input_pos = 1, 32, 8, 1024, 32768, 128, 31744
+    gen = torch.Generator().manual_seed(1)
+    q = torch.randn(B, Hq, q_len, D, generator=gen)
+    k = torch.randn(B, Hkv, T, D, generator=gen)
+    v = torch.randn(B, Hkv, T, D, generator=gen).to(torch.bfloat16)
+    q = O.apply_rope(q, torch.arange(input_pos, input_pos + q_len)).to(torch.bfloat16)
+    k = O.apply_rope(k, torch.arange(T)).to(torch.bfloat16)
+    scale = D ** -0.5
+    out, w, lse = ops.prefill_core(q.to(gpu), k.to(gpu), v.to(gpu), scale, input_pos, None, return_weights=True, return_lse=True)
+    torch.cuda.synchronize()
+    w_c = w.cpu()
+    assert (w_c >= 0).all()
+    torch.testing.assert_close(w_c.sum(-1), torch.full((B, Hkv), float(q_len)), rtol=5e-5, atol=3e-2)
+    # oracle on KV head 3 (4 query heads)
+    h = 3
+    o_ref, w_ref = O.sdpa_in_blocks(q[:, 4 * h : 4 * h + 4], k[:, h : h + 1], v[:, h : h + 1], scale, input_pos, None)
+    check_o(out.permute(0, 2, 1, 3)[:, 4 * h : 4 * h + 4], o_ref)
+    torch.testing.assert_close(w_c[:, h : h + 1], w_ref, rtol=W_RTOL, atol=1e-6)
+    # scattered layout: permute slots independently per head
+    perm = torch.stack([torch.randperm(T, generator=gen) for _ in range(Hkv)]).view(B, Hkv, T)
+    gi = perm.unsqueeze(-1).expand(-1, -1, -1, D)
+    out_s, w_s, _ = ops.prefill_core(q.to(gpu), k.gather(2, gi).to(gpu), v.gather(2, gi).to(gpu), scale, input_pos,
+                                     perm.to(torch.int32).to(gpu), return_weights=True)
+    torch.cuda.synchronize()
+    # same values, other summation order and other running maxima: equal up to bf16 rounding
+    assert rel_err(out_s.float().cpu(), out.float().cpu()) < 1e-2
+    w_back = torch.zeros_like(w_c).scatter_(-1, perm, w_s.cpu())
+    torch.testing.assert_close(w_back, w_c, rtol=W_RTOL, atol=1e-6)

@@ -1,0 +1,328 @@
+"""GPU parity of the cache kernels (quantiser, slot write, H2O update/selection, the H2O cache step)
+against the CPU oracle, through the C ABI."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from helpers import make_qkv, rel_err, scattered_positions
+from keys_values_amd import _lib
+from keys_values_amd.attention import ops
+from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
+from keys_values_amd.kvcache.quantize import RowQuantizer8
+from oracle import kvx_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def outlier_rows(seed, rows, D):
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, D, generator=gen)
+    mask = torch.rand(rows, D, generator=gen) < 0.01
+    return torch.where(mask, torch.randn(rows, D, generator=gen) * 8, x).to(torch.bfloat16)
+
+
+def gpu_quantize(lib, x_gpu):
+    rows, D = x_gpu.shape
+    codes = torch.empty((rows, D), dtype=torch.uint8, device=x_gpu.device)
+    sc = torch.empty(rows, dtype=torch.float32, device=x_gpu.device)
+    zp = torch.empty(rows, dtype=torch.int32, device=x_gpu.device)
+    _lib.check(lib.kvx_quantize_rows(x_gpu.data_ptr(), x_gpu.stride(0), rows, D, codes.data_ptr(), sc.data_ptr(), zp.data_ptr(),
+                                      _lib.stream_ptr(x_gpu.device)))
+    return codes, sc, zp
+
+
+@pytest.mark.parametrize("rows,D", [(1, 128), (7, 64), (1000, 128), (4099, 64), (65536, 128)])
+def test_quantize_rows_bit_exact(kvx, gpu, rows, D):
+    x = outlier_rows(2, rows, D)
+    if rows >= 7:  # edge rows: constant, all negative, tiny range, extremes of bf16 dynamics
+        x[0] = 0.0
+        x[1] = -3.5
+        x[2] = torch.linspace(-1e-3, 1e-3, D).to(torch.bfloat16)
+        x[3] = torch.linspace(100.0, 101.0, D).to(torch.bfloat16)
+        x[4] = 7.0
+        x[5, ::2] = -1e4
+    c_ref, s_ref, z_ref = O.quantize_rows(x)
+    codes, sc, zp = gpu_quantize(kvx, x.to(gpu))
+    torch.cuda.synchronize()
+    assert torch.equal(sc.cpu(), s_ref), "scales differ"
+    assert torch.equal(zp.cpu(), z_ref), "zero points differ"
+    assert torch.equal(codes.cpu(), c_ref), "codes differ"
+    out = torch.empty((rows, D), dtype=torch.bfloat16, device=gpu)
+    _lib.check(kvx.kvx_dequantize_rows(codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), rows, D, out.data_ptr(), D, _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), O.dequantize_rows(c_ref, s_ref, z_ref, torch.bfloat16)), "dequantised rows differ"
+
+
+def test_quantize_empty_and_strided(kvx, gpu):
+    assert kvx.kvx_quantize_rows(None, 128, 0, 128, None, None, None, None) == 0
+    x = outlier_rows(4, 300, 256).to(gpu)  # rows of 128 inside rows of 256
+    codes, sc, zp = gpu_quantize(kvx, x[:, :128])
+    c_ref, s_ref, z_ref = O.quantize_rows(x[:, :128].cpu())
+    assert torch.equal(codes.cpu(), c_ref) and torch.equal(sc.cpu(), s_ref) and torch.equal(zp.cpu(), z_ref)
+
+
+def test_row_quantizer_class_known_answer(gpu):
+    # test/kvcache/test_quantization.py:647-766 through the Quantizer surface: integers 0..255 with
+    # both extremes in every row survive a round trip exactly (bf16 holds them exactly)
+    gen = torch.Generator().manual_seed(31415927)
+    shape = (3, 4, 32, 64)
+    data = torch.randint(0, 256, shape, generator=gen)
+    i0 = torch.randint(0, 64, shape[:-1], generator=gen)
+    i1 = (i0 + 1 + torch.randint(0, 63, shape[:-1], generator=gen)) % 64
+    data.scatter_(-1, i0.unsqueeze(-1), 0)
+    data.scatter_(-1, i1.unsqueeze(-1), 255)
+    qz = RowQuantizer8(shape, torch.bfloat16, 8, allocate_buffers=True, device=gpu)
+    assert qz.quant_buffer.shape == (12, 32, 64) and qz.quant_buffer.dtype == torch.uint8
+    assert qz.quant_scales.dtype == torch.float32 and qz.quant_zero_points.dtype == torch.int32
+    x = data.to(torch.bfloat16).to(gpu)
+    qz.quantize(0, 32, x)
+    assert torch.equal(qz.dequantize(0, 32), x)
+    assert torch.equal(qz.quant_buffer.view(shape).cpu().long(), data)
+    # partial range write keeps the other slots
+    x2 = (data[:, :, 5:9] // 2).to(torch.bfloat16).to(gpu)
+    qz.quantize(5, 9, x2)
+    back = qz.dequantize(0, 32)
+    c_ref, s_ref, z_ref = O.quantize_rows(x2.cpu())
+    assert torch.equal(back[:, :, 5:9].cpu(), O.dequantize_rows(c_ref, s_ref, z_ref))
+    assert torch.equal(back[:, :, :5], x[:, :, :5]) and torch.equal(back[:, :, 9:], x[:, :, 9:])
+    err = qz.quantization_error(x2)
+    torch.testing.assert_close(err.cpu(), O.quantization_error(x2.cpu()), rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        qz.quantize(0, 4, x)
+    with pytest.raises(NotImplementedError):
+        RowQuantizer8(shape, torch.bfloat16, 4)
+
+
+def run_cache_write(kvx, gpu, quantized):
+    B, Hkv, L, D, num, input_pos = 2, 3, 50, 128, 7, 90
+    gen = torch.Generator().manual_seed(17)
+    kc = torch.randn(B, Hkv, L, D, generator=gen).to(torch.bfloat16)
+    vc = torch.randn(B, Hkv, L, D, generator=gen).to(torch.bfloat16)
+    key = torch.randn(B, Hkv, num, D, generator=gen).to(torch.bfloat16)
+    val = torch.randn(B, Hkv, num, D, generator=gen).to(torch.bfloat16)
+    tp = torch.randint(0, 90, (B, Hkv, L), generator=gen, dtype=torch.int32)
+    sc = torch.rand(B, Hkv, L, generator=gen)
+    index = torch.stack([torch.randperm(L, generator=gen)[:num] for _ in range(B * Hkv)]).view(B, Hkv, num)
+    k_ref, v_ref, tp_ref, sc_ref = kc.clone(), vc.clone(), tp.clone(), sc.clone()
+    O.cache_write(k_ref, v_ref, tp_ref, sc_ref, index, key, val, input_pos)
+    a = _lib.CacheWriteArgs()
+    a.B, a.Hkv, a.num, a.D, a.cache_len, a.input_pos = B, Hkv, num, D, L, input_pos
+    idx32 = index.to(torch.int32).to(gpu)
+    key_g, val_g, tp_g, sc_g = key.to(gpu), val.to(gpu), tp.to(gpu), sc.to(gpu)
+    a.index, a.index_stride_b, a.index_stride_h = idx32.data_ptr(), idx32.stride(0), idx32.stride(1)
+    a.key, a.key_stride_b, a.key_stride_h, a.key_stride_t = key_g.data_ptr(), *key_g.stride()[:3]
+    a.value, a.value_stride_b, a.value_stride_h, a.value_stride_t = val_g.data_ptr(), *val_g.stride()[:3]
+    a.token_pos, a.tp_stride_b, a.tp_stride_h = tp_g.data_ptr(), tp_g.stride(0), tp_g.stride(1)
+    a.scores, a.sc_stride_b, a.sc_stride_h = sc_g.data_ptr(), sc_g.stride(0), sc_g.stride(1)
+    if not quantized:
+        a.kv_dtype = _lib.KVX_KV_BF16
+        kc_g, vc_g = kc.to(gpu), vc.to(gpu)
+    else:
+        a.kv_dtype = _lib.KVX_KV_U8
+        qk, qv = O.quantize_rows(kc), O.quantize_rows(vc)
+        kc_g, vc_g = qk[0].to(gpu), qv[0].to(gpu)
+        ks_g, kz_g, vs_g, vz_g = qk[1].to(gpu), qk[2].to(gpu), qv[1].to(gpu), qv[2].to(gpu)
+        a.k_scale, a.k_zp, a.v_scale, a.v_zp = ks_g.data_ptr(), kz_g.data_ptr(), vs_g.data_ptr(), vz_g.data_ptr()
+        a.qs_stride_b, a.qs_stride_h = ks_g.stride(0), ks_g.stride(1)
+    a.k_cache, a.kc_stride_b, a.kc_stride_h, a.kc_stride_t = kc_g.data_ptr(), *kc_g.stride()[:3]
+    a.v_cache, a.vc_stride_b, a.vc_stride_h, a.vc_stride_t = vc_g.data_ptr(), *vc_g.stride()[:3]
+    _lib.check(kvx.kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    assert torch.equal(tp_g.cpu(), tp_ref) and torch.equal(sc_g.cpu(), sc_ref)
+    if not quantized:
+        assert torch.equal(kc_g.cpu(), k_ref) and torch.equal(vc_g.cpu(), v_ref)
+    else:
+        for got, ref in (((kc_g, ks_g, kz_g), k_ref), ((vc_g, vs_g, vz_g), v_ref)):
+            c_ref, s_ref, z_ref = O.quantize_rows(ref)  # rows not written keep their old codes
+            assert torch.equal(got[0].cpu(), c_ref) and torch.equal(got[1].cpu(), s_ref) and torch.equal(got[2].cpu(), z_ref)
+
+
+def test_cache_write_bf16(kvx, gpu):
+    run_cache_write(kvx, gpu, False)
+
+
+def test_cache_write_uint8(kvx, gpu):
+    run_cache_write(kvx, gpu, True)
+
+
+def gpu_h2o(kvx, gpu, scores, w, kv_len, limit, k, normalize=False, token_pos=None, input_pos=0, prefill_len=0):
+    B, Hkv, L = scores.shape
+    sc_g = scores.to(gpu)
+    w_g = None if w is None else w.contiguous().to(gpu)
+    tp_g = None if token_pos is None else token_pos.to(torch.int32).to(gpu)
+    nxt = torch.empty((B, Hkv, k), dtype=torch.int32, device=gpu)
+    a = _lib.H2OArgs()
+    a.B, a.Hkv, a.kv_len, a.limit, a.k = B, Hkv, kv_len, limit, k
+    a.normalize, a.input_pos, a.prefill_len = int(normalize), input_pos, prefill_len
+    a.scores, a.sc_stride_b, a.sc_stride_h = sc_g.data_ptr(), sc_g.stride(0), sc_g.stride(1)
+    a.w = _lib.ptr(w_g)
+    if tp_g is not None:
+        a.token_pos, a.tp_stride_b, a.tp_stride_h = tp_g.data_ptr(), tp_g.stride(0), tp_g.stride(1)
+    a.next_index = nxt.data_ptr()
+    nb = kvx.kvx_h2o_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(max(nb, 8), dtype=torch.uint8, device=gpu)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    _lib.check(kvx.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    return sc_g.cpu(), nxt.cpu()
+
+
+@pytest.mark.parametrize("B,Hkv,L,kv_len,limit,k", [
+    (2, 3, 300, 300, 300, 1), (8, 8, 5000, 5000, 5000, 1), (1, 2, 1024, 1024, 1024, 128), (2, 2, 4097, 4000, 3999, 1000),
+    (1, 8, 16384, 16384, 16384, 1024), (1, 1, 64, 64, 64, 64), (1, 2, 131072, 131072, 131072, 4096), (2, 2, 10001, 10001, 10001, 1),
+])
+def test_h2o_update_select(kvx, gpu, B, Hkv, L, kv_len, limit, k):
+    gen = torch.Generator().manual_seed(L + k)
+    scores = torch.rand(B, Hkv, L, generator=gen) * 3
+    w = torch.rand(B, Hkv, kv_len, generator=gen)
+    s_ref = scores.clone()
+    n_ref = O.h2o_update_select(s_ref, w, kv_len, limit, k)
+    s_gpu, n_gpu = gpu_h2o(kvx, gpu, scores, w, kv_len, limit, k)
+    assert torch.equal(s_gpu, s_ref), "scores += w differs"
+    assert torch.equal(n_gpu.long(), n_ref), "selected slots differ"
+
+
+def test_h2o_select_ties_and_no_weights(kvx, gpu):
+    # many exact ties (quantised scores), zeros and negative zeros: lower slot first, like a stable argsort
+    gen = torch.Generator().manual_seed(3)
+    scores = torch.randint(0, 6, (2, 2, 999), generator=gen).float() * 0.25
+    scores[0, 0, 100:140] = 0.0
+    scores[0, 0, 120] = -0.0
+    for k in (1, 50, 333):
+        s_ref = scores.clone()
+        n_ref = O.h2o_update_select(s_ref, None, 999, 999, k)
+        s_gpu, n_gpu = gpu_h2o(kvx, gpu, scores, None, 999, 999, k)
+        assert torch.equal(n_gpu.long(), n_ref)
+        assert torch.equal(s_gpu, scores)
+
+
+def test_h2o_select_normalized(kvx, gpu):
+    # keys_values/kvcache/h2o.py:183-196
+    gen = torch.Generator().manual_seed(4)
+    B, Hkv, L = 2, 2, 777
+    scores = torch.rand(B, Hkv, L, generator=gen) * 5
+    w = torch.rand(B, Hkv, L, generator=gen)
+    tp = torch.stack([torch.randperm(2000, generator=gen)[:L] for _ in range(B * Hkv)]).view(B, Hkv, L).to(torch.int32)
+    for k in (1, 64):
+        s_ref = scores.clone()
+        n_ref = O.h2o_update_select(s_ref, w, L, L, k, normalize=True, token_pos=tp, input_pos=2100, prefill_len=512)
+        s_gpu, n_gpu = gpu_h2o(kvx, gpu, scores, w, L, L, k, True, tp, 2100, 512)
+        assert torch.equal(s_gpu, s_ref)
+        assert torch.equal(n_gpu.long(), n_ref)
+
+
+def _sets_equal_away_from_ties(n_gpu, n_ref, scores_ref, k):
+    """Selected sets must agree unless the cut falls between numerically indistinguishable scores
+    (GPU and CPU scores differ in the last bits)."""
+    for b in range(n_ref.shape[0]):
+        for h in range(n_ref.shape[1]):
+            a, r = set(n_gpu[b, h, :k].tolist()), set(n_ref[b, h, :k].tolist())
+            if a != r:
+                srt = torch.sort(scores_ref[b, h]).values
+                gap = (srt[k] - srt[k - 1]).item()
+                diff = a ^ r
+                assert gap < 1e-3 * max(srt[k].item(), 1e-6) or all(
+                    abs(scores_ref[b, h, i].item() - srt[k - 1].item()) < 2e-3 * max(srt[k].item(), 1e-6) for i in diff
+                ), f"selection differs away from a tie at ({b},{h}): {sorted(diff)}"
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+def test_h2o_cache_steps_vs_oracle(gpu, quantized):
+    """Prefill that fills the cache, then chunked steps: initial rule, evict-write, attention with
+    scattered positions, score accumulation, selection (configuration 1 shapes: 8/2 heads, D 64,
+    1024 slots, 128-token chunks). With the uint8 store every row is quantised once, when written,
+    so the oracle is fed the dequantised rows: what the reference's attention reads from its
+    dequantised working buffer (keys_values/kvcache/quant_buffers.py:776-793)."""
+    B, Hq, Hkv, L, D, chunk = 1, 8, 2, 1024, 64, 128
+    gen = torch.Generator().manual_seed(0)
+    total = L + 4 * chunk
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    ks_o = O.dequantize_rows(*O.quantize_rows(ks)) if quantized else ks
+    vs_o = O.dequantize_rows(*O.quantize_rows(vs)) if quantized else vs
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=chunk)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, quantized=quantized, device=gpu)
+    ref.prefill(qs[:, :, :L], ks_o[:, :, :L], vs_o[:, :, :L])
+    # the first chunk attends over the keys/values as given, not over the store (kvcache/base.py:567-571)
+    o_ref, _ = O.sdpa_in_blocks(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L], 1 / math.sqrt(D), 0, None, return_attn_weights=False)
+    o = cache.forward(qs[:, :, :L].to(gpu), ks[:, :, :L].to(gpu), vs[:, :, :L].to(gpu))
+    assert rel_err(o.float().cpu().view(B, L, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+    assert cache.next_positions(chunk)[0, 0].tolist() == list(range(51, 51 + chunk))  # int(0.05 * 1024) = 51
+    pos = L
+    for step in range(4):
+        sl = slice(pos, pos + chunk)
+        o_ref, w_ref, index = ref.forward(qs[:, :, sl], ks_o[:, :, sl], vs_o[:, :, sl])
+        if step > 0:
+            # write to the oracle's slots so that the two caches stay comparable step after step
+            # (the GPU's own choice is checked below)
+            cache._next_index[:B, :, :chunk] = index.to(torch.int32).to(gpu)
+        o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        assert cache.input_pos == ref.input_pos
+        assert torch.equal(cache.token_pos.cpu(), ref.token_pos)
+        assert rel_err(o.float().cpu().view(B, chunk, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+        torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
+        if quantized:
+            assert torch.equal(O.dequantize_rows(cache.k.cpu(), cache.k_scale.cpu(), cache.k_zp.cpu()), ref.k)
+            assert torch.equal(O.dequantize_rows(cache.v.cpu(), cache.v_scale.cpu(), cache.v_zp.cpu()), ref.v)
+        else:
+            assert torch.equal(cache.k.cpu(), ref.k) and torch.equal(cache.v.cpu(), ref.v)
+        _sets_equal_away_from_ties(cache._next_index[:B].cpu().long(), ref.next_index, ref.scores, chunk)
+        pos += chunk
+
+
+def test_h2o_cache_decode_steps(gpu):
+    # single-token steps: argmin selection, slot reuse, scores = running sum (test/kvcache/test_h2o.py:109-137)
+    B, Hq, Hkv, L, D = 2, 8, 2, 256, 128
+    gen = torch.Generator().manual_seed(3)
+    total = L + 6
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=1)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, device=gpu)
+    ref.prefill(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L])
+    cache.forward(qs[:, :, :L].to(gpu), ks[:, :, :L].to(gpu), vs[:, :, :L].to(gpu))
+    for t in range(L, total):
+        sl = slice(t, t + 1)
+        o_ref, w_ref, index = ref.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        if t > L:
+            assert torch.equal(cache.next_positions(1).cpu(), index), "evicted slot differs"
+        o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        assert rel_err(o.float().cpu().view(B, 1, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+        torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
+        assert torch.equal(cache.token_pos.cpu(), ref.token_pos)
+
+
+def test_attention_over_uint8_cache(kvx, gpu):
+    """Configuration 3 semantics at a reduced size: K with 1% outliers, quantised on the GPU,
+    attention + score-sums with dequantisation fused into the loads, against the oracle run on the
+    dequantised bf16 cache."""
+    B, Hq, Hkv, q_len, T, D = 1, 8, 2, 96, 2048 + 40, 128
+    gen = torch.Generator().manual_seed(2)
+    k = outlier_rows(2, B * Hkv * T, D).view(B, Hkv, T, D)
+    v = torch.randn(B, Hkv, T, D, generator=gen).to(torch.bfloat16)
+    q = torch.randn(B, Hq, q_len, D, generator=gen).to(torch.bfloat16)
+    input_pos = T - q_len
+    kc, ks, kz = gpu_quantize(kvx, k.view(-1, D).to(gpu))
+    vc, vs, vz = gpu_quantize(kvx, v.view(-1, D).to(gpu))
+    quant = ops.QuantState(ks.view(B, Hkv, T), kz.view(B, Hkv, T), vs.view(B, Hkv, T), vz.view(B, Hkv, T))
+    kd = O.dequantize_rows(*O.quantize_rows(k))
+    vd = O.dequantize_rows(*O.quantize_rows(v))
+    scale = 1 / math.sqrt(D)
+    o_ref, w_ref = O.sdpa_in_blocks(q, kd, vd, scale, input_pos, None)
+    out, w, _ = ops.prefill_core(q.to(gpu), kc.view(B, Hkv, T, D), vc.view(B, Hkv, T, D), scale, input_pos, None,
+                                 return_weights=True, quant=quant, output_transposed=False)
+    torch.cuda.synchronize()
+    assert rel_err(out.float().cpu(), o_ref.float()) < 2e-2
+    torch.testing.assert_close(w.cpu(), w_ref, rtol=1e-3, atol=1e-6)
+    # decode over the same store
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], kd, vd, scale, T - 1, None)
+    out1, w1, _ = ops.decode_core(q[:, :, :1].to(gpu), kc.view(B, Hkv, T, D), vc.view(B, Hkv, T, D), scale, return_weights=True, quant=quant)
+    torch.cuda.synchronize()
+    assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
+    torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)

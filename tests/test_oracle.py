@@ -189,6 +189,20 @@ def test_quantiser_python_and_c_bit_equal():
     assert ((x.float() - d).abs() <= 0.5001 * s.unsqueeze(-1) + 1e-7).all()
 
 
+def test_quantization_error_bound_and_zero():
+    # integers 0..255 with both extremes are represented exactly -> zero error; otherwise every
+    # element is off by at most half a quantisation step
+    x = torch.arange(256, dtype=torch.float32).view(2, 128)
+    x[1] = x[0]
+    x[1, 0], x[1, 127] = 0.0, 255.0
+    assert (O.quantization_error(torch.stack((x[0] * 2, x[1]))[1:]) == 0).all()
+    g = torch.Generator().manual_seed(1)
+    y = torch.randn(64, 128, generator=g)
+    _, s, _ = O.quantize_rows(y)
+    err = O.quantization_error(y)
+    assert (err <= 0.5001 * s * math.sqrt(128)).all() and (err > 0).all()
+
+
 # ---- H2O bookkeeping -------------------------------------------------------------------------------
 
 
