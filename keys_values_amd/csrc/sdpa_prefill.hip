@@ -47,82 +47,23 @@ struct PrefillParams {
 };
 
 template <int D>
-struct Smem {
-  static constexpr int KROW = D + 8;        // bf16 per K row incl. pad (keeps ds_read_b128 conflict free)
-  uint16_t k[2][BN * KROW];                 // [key][d]
-  uint16_t vt[2][D * BN];                   // [d][slot], 16-byte chunks swizzled by vt_swz(d)
+struct alignas(16) Smem {
+  static constexpr int KCH16 = D / 8 + 1;   // 16-byte chunks per K row incl. pad: row stride = 4 banks mod 64,
+                                            // so the 16 rows a ds_read_b128 phase touches hit distinct banks
+  static constexpr int VCH16 = D / 8 + 4;   // V row stride = 16 banks mod 64: the 4 rows x 64 bytes a pair of
+                                            // 16-lane transpose-read groups touches hit distinct banks
+  u32x4_t k[2][BN][KCH16];                  // [key][d]
+  u32x4_t v[2][BN][VCH16];                  // [key][d]
   int32_t tp[2][BN];
 };
 
-// Chunk swizzle of the transposed V tile: distinct over the 8 (d>>3) values a staging wavefront
-// writes together and over the 8 ((d>>1)&3, (d>>3)&1) values an MFMA operand read touches.
-__device__ __forceinline__ int vt_swz(int d) { return ((d >> 3) & 7) ^ (((d >> 1) & 3) << 1); }
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
-template <int D, bool U8>
-struct Stage {
-  // registers holding one prefetched K/V tile of this thread
-  static constexpr int KCH = (BN * D / 8) / NTHREADS;  // 16-byte (bf16) chunks of K per thread: 4 (D=128), 2 (D=64)
-  u32x4_t kr[KCH];
-  u32x4_t vr[4];
-  float ks[KCH];
-  int32_t kz[KCH];
-  float vs[4];
-  int32_t vz[4];
-  int32_t tpv;
-};
-
-template <int D, bool U8>
-__device__ __forceinline__ void fetch_tile(Stage<D, U8>& s, const PrefillParams& p, int b, int kvh, int key0, int tid) {
-  constexpr int CPR = D / 8;  // chunks per row
-  constexpr int RPI = NTHREADS / CPR;
-  const int col = tid % CPR;
-  const int row_in = tid / CPR;
-  // K
-#pragma unroll
-  for (int i = 0; i < Stage<D, U8>::KCH; ++i) {
-    const int key = key0 + row_in + i * RPI;
-    const bool ok = key < p.kv_len;
-    if constexpr (!U8) {
-      const uint16_t* src = (const uint16_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st + col * 8;
-      s.kr[i] = ok ? *(const u32x4_t*)src : u32x4_t{0, 0, 0, 0};
-    } else {
-      const uint8_t* src = (const uint8_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st + col * 8;
-      u32x2_t c = ok ? *(const u32x2_t*)src : u32x2_t{0, 0};
-      s.kr[i] = u32x4_t{c[0], c[1], 0, 0};
-      const int64_t so = b * p.qs_sb + kvh * p.qs_sh + key;
-      s.ks[i] = ok ? p.k_scale[so] : 0.0f;
-      s.kz[i] = ok ? p.k_zp[so] : 0;
-    }
-  }
-  // V: thread = (group of 4 keys, chunk of 8 d)
-  {
-    const int kg = tid / CPR;  // 0..15 valid
-    const int dc = tid % CPR;
-    if (kg < BN / 4) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = key0 + kg * 4 + r;
-        const bool ok = key < p.kv_len;
-        if constexpr (!U8) {
-          const uint16_t* src = (const uint16_t*)p.v + b * p.v_sb + kvh * p.v_sh + (int64_t)key * p.v_st + dc * 8;
-          s.vr[r] = ok ? *(const u32x4_t*)src : u32x4_t{0, 0, 0, 0};
-        } else {
-          const uint8_t* src = (const uint8_t*)p.v + b * p.v_sb + kvh * p.v_sh + (int64_t)key * p.v_st + dc * 8;
-          u32x2_t c = ok ? *(const u32x2_t*)src : u32x2_t{0, 0};
-          s.vr[r] = u32x4_t{c[0], c[1], 0, 0};
-          const int64_t so = b * p.qs_sb + kvh * p.qs_sh + key;
-          s.vs[r] = ok ? p.v_scale[so] : 0.0f;
-          s.vz[r] = ok ? p.v_zp[so] : 0;
-        }
-      }
-    }
-  }
-  if (tid < BN) {
-    const int key = key0 + tid;
-    int32_t t = INT_MAX;  // keys past the end are masked for every query
-    if (key < p.kv_len) t = p.tp ? p.tp[b * p.tp_sb + kvh * p.tp_sh + key] : key;
-    s.tpv = t;
-  }
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i (a = i % 4, r = i / 4) supplies the
+// address of 4 consecutive bf16 of "row r, columns 4a..4a+3"; it receives column i of rows 0..3.
+__device__ __forceinline__ u32x2_t lds_read_tr16(const void* p) {
+  const s16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
+  return __builtin_bit_cast(u32x2_t, t);
 }
 
 // 8 codes (two dwords) -> 8 bf16 (four dwords)
@@ -136,46 +77,121 @@ __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp
 }
 
 template <int D, bool U8>
-__device__ __forceinline__ void commit_tile(Stage<D, U8>& s, Smem<D>& sm, int buf, int tid) {
-  constexpr int CPR = D / 8;
-  constexpr int RPI = NTHREADS / CPR;
-  const int col = tid % CPR;
-  const int row_in = tid / CPR;
+struct Stage {
+  // registers holding one prefetched K/V tile of this thread: KCH rows, one 16-byte chunk each
+  static constexpr int KCH = (BN * D / 8) / NTHREADS;  // 4 (D=128), 2 (D=64)
+  u32x4_t kr[KCH];
+  u32x4_t vr[KCH];
+  float ks[KCH], vs[KCH];
+  int32_t kz[KCH], vz[KCH];
+  int32_t tpv;
+};
+
+template <int D, bool U8>
+struct Loader {
+  static constexpr int CPR = D / 8;             // chunks per row
+  static constexpr int RPI = NTHREADS / CPR;    // rows per pass of the workgroup
+  static constexpr int KCH = Stage<D, U8>::KCH;
+  static constexpr int ESZ = U8 ? 1 : 2;        // bytes per element in memory
+  const char* kbase;                            // (b, kvh) slice, uniform
+  const char* vbase;
+  const float* ks;
+  const int32_t* kz;
+  const float* vs;
+  const int32_t* vz;
+  const int32_t* tp;                            // may be NULL
+  uint32_t koff[KCH], voff[KCH];                // byte offsets of this thread's chunks inside a tile
+  int64_t k_tile_bytes, v_tile_bytes;
+  int64_t k_st, v_st;
+  int row_in, col, kv_len;
+
+  __device__ __forceinline__ void init(const PrefillParams& p, int b, int kvh, int tid) {
+    col = tid % CPR;
+    row_in = tid / CPR;
+    kv_len = p.kv_len;
+    k_st = p.k_st;
+    v_st = p.v_st;
+    kbase = (const char*)p.k + (b * p.k_sb + kvh * p.k_sh) * ESZ;
+    vbase = (const char*)p.v + (b * p.v_sb + kvh * p.v_sh) * ESZ;
+    const int64_t so = b * p.qs_sb + kvh * p.qs_sh;
+    ks = p.k_scale + so;
+    kz = p.k_zp + so;
+    vs = p.v_scale + so;
+    vz = p.v_zp + so;
+    tp = p.tp ? p.tp + b * p.tp_sb + kvh * p.tp_sh : nullptr;
+    k_tile_bytes = (int64_t)BN * p.k_st * ESZ;
+    v_tile_bytes = (int64_t)BN * p.v_st * ESZ;
 #pragma unroll
-  for (int i = 0; i < Stage<D, U8>::KCH; ++i) {
-    u32x4_t val = s.kr[i];
-    if constexpr (U8) val = dequant8(val[0], val[1], s.kz[i], s.ks[i]);
-    *(u32x4_t*)&sm.k[buf][(row_in + i * RPI) * Smem<D>::KROW + col * 8] = val;
-  }
-  const int kg = tid / CPR;
-  const int dc = tid % CPR;
-  if (kg < BN / 4) {
-    u32x4_t a[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      a[r] = s.vr[r];
-      if constexpr (U8) a[r] = dequant8(a[r][0], a[r][1], s.vz[r], s.vs[r]);
+    for (int i = 0; i < KCH; ++i) {
+      koff[i] = (uint32_t)((row_in + i * RPI) * p.k_st * ESZ + col * 8 * ESZ);
+      voff[i] = (uint32_t)((row_in + i * RPI) * p.v_st * ESZ + col * 8 * ESZ);
     }
-    // slot of key group kg: within 16 keys the order is (0..3, 8..11, 4..7, 12..15)
-    const int pos = 16 * (kg >> 2) + 8 * (kg & 1) + 4 * ((kg >> 1) & 1);
+  }
+
+  __device__ __forceinline__ void fetch(Stage<D, U8>& s, int tile, int tid) const {
+    const int key0 = tile * BN;
+    const char* kt = kbase + tile * k_tile_bytes;
+    const char* vt = vbase + tile * v_tile_bytes;
+    if (key0 + BN <= kv_len) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      // dword e of each row holds d = 2e (low half) and 2e+1 (high half)
-      u32x2_t lo, hi;
-      lo[0] = __builtin_amdgcn_perm(a[1][e], a[0][e], 0x05040100u);
-      lo[1] = __builtin_amdgcn_perm(a[3][e], a[2][e], 0x05040100u);
-      hi[0] = __builtin_amdgcn_perm(a[1][e], a[0][e], 0x07060302u);
-      hi[1] = __builtin_amdgcn_perm(a[3][e], a[2][e], 0x07060302u);
-      const int d0 = dc * 8 + 2 * e;
-      const int d1 = d0 + 1;
-      const int ch0 = (pos >> 3) ^ vt_swz(d0);
-      const int ch1 = (pos >> 3) ^ vt_swz(d1);
-      *(u32x2_t*)&sm.vt[buf][d0 * BN + ch0 * 8 + (pos & 7)] = lo;
-      *(u32x2_t*)&sm.vt[buf][d1 * BN + ch1 * 8 + (pos & 7)] = hi;
+      for (int i = 0; i < KCH; ++i) {
+        if constexpr (!U8) {
+          s.kr[i] = *(const u32x4_t*)(kt + koff[i]);
+          s.vr[i] = *(const u32x4_t*)(vt + voff[i]);
+        } else {
+          const u32x2_t ck = *(const u32x2_t*)(kt + koff[i]);
+          const u32x2_t cv = *(const u32x2_t*)(vt + voff[i]);
+          s.kr[i] = u32x4_t{ck[0], ck[1], 0, 0};
+          s.vr[i] = u32x4_t{cv[0], cv[1], 0, 0};
+          const int key = key0 + row_in + i * RPI;
+          s.ks[i] = ks[key];
+          s.kz[i] = kz[key];
+          s.vs[i] = vs[key];
+          s.vz[i] = vz[key];
+        }
+      }
+      if (tid < BN) s.tpv = tp ? tp[key0 + tid] : key0 + tid;
+    } else {
+      // last, partial tile: rows past the end re-read the last valid row (finite data); their
+      // position is INT_MAX, so they are masked for every query and contribute exactly zero
+#pragma unroll
+      for (int i = 0; i < KCH; ++i) {
+        const int key = min(key0 + row_in + i * RPI, kv_len - 1);
+        if constexpr (!U8) {
+          s.kr[i] = *(const u32x4_t*)(kbase + ((int64_t)key * k_st + col * 8) * ESZ);
+          s.vr[i] = *(const u32x4_t*)(vbase + ((int64_t)key * v_st + col * 8) * ESZ);
+        } else {
+          const u32x2_t ck = *(const u32x2_t*)(kbase + ((int64_t)key * k_st + col * 8));
+          const u32x2_t cv = *(const u32x2_t*)(vbase + ((int64_t)key * v_st + col * 8));
+          s.kr[i] = u32x4_t{ck[0], ck[1], 0, 0};
+          s.vr[i] = u32x4_t{cv[0], cv[1], 0, 0};
+          s.ks[i] = ks[key];
+          s.kz[i] = kz[key];
+          s.vs[i] = vs[key];
+          s.vz[i] = vz[key];
+        }
+      }
+      if (tid < BN) {
+        const int key = key0 + tid;
+        s.tpv = key < kv_len ? (tp ? tp[key] : key) : INT_MAX;
+      }
     }
   }
-  if (tid < BN) sm.tp[buf][tid] = s.tpv;
-}
+
+  __device__ __forceinline__ void commit(const Stage<D, U8>& s, Smem<D>& sm, int buf, int tid) const {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      u32x4_t kk = s.kr[i], vv = s.vr[i];
+      if constexpr (U8) {
+        kk = dequant8(kk[0], kk[1], s.kz[i], s.ks[i]);
+        vv = dequant8(vv[0], vv[1], s.vz[i], s.vs[i]);
+      }
+      sm.k[buf][row_in + i * RPI][col] = kk;
+      sm.v[buf][row_in + i * RPI][col] = vv;
+    }
+    if (tid < BN) sm.tp[buf][tid] = s.tpv;
+  }
+};
 
 template <int D, bool U8>
 __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const PrefillParams p) {
@@ -223,25 +239,35 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
   float m = -INFINITY;  // running max of the raw (unscaled) scores of this row
   float l = 0.0f;       // this lane's share of the running sum
 
+  // transpose-read addressing of V: in its group of 16 lanes this lane points at key row (i / 4)
+  // and at d columns 4 (i % 4) .. +3 of the 16 d columns the group produces
+  const int li = lane & 15;
+  const int v_row_off = (li >> 2) + 4 * h;                      // + 32 mt + 16 j (+ 8)
+  const int v_col_off = 16 * ((lane >> 4) & 1) + 4 * (li & 3);  // + 32 dt, in bf16 elements
+
+  Loader<D, U8> ld;
+  ld.init(p, b, kvh, tid);
   Stage<D, U8> st;
   if (tile_begin < tile_end) {
-    fetch_tile<D, U8>(st, p, b, kvh, tile_begin * BN, tid);
-    commit_tile<D, U8>(st, sm, 0, tid);
-    if (tile_begin + 1 < tile_end) fetch_tile<D, U8>(st, p, b, kvh, (tile_begin + 1) * BN, tid);
+    ld.fetch(st, tile_begin, tid);
+    ld.commit(st, sm, 0, tid);
+    if (tile_begin + 1 < tile_end) ld.fetch(st, tile_begin + 1, tid);
   }
   __syncthreads();
 
   for (int t = tile_begin; t < tile_end; ++t) {
     const int buf = (t - tile_begin) & 1;
-    // ---- S^T = K Q^T --------------------------------------------------------------------
+    // ---- S^T = K Q^T: two independent accumulator chains -----------------------------------
     f32x16_t s[2];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[mt][i] = 0.0f;
 #pragma unroll
-      for (int j = 0; j < D / 16; ++j) {
-        const u32x4_t kk = *(const u32x4_t*)&sm.k[buf][(mt * 32 + n) * Smem<D>::KROW + 16 * j + 8 * h];
+    for (int j = 0; j < D / 16; ++j) {
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const u32x4_t kk = sm.k[buf][mt * 32 + n][2 * j + h];
         s[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kk), qf[j], s[mt], 0, 0, 0);
       }
     }
@@ -262,17 +288,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
       }
     }
     // ---- online softmax --------------------------------------------------------------------
-    float mx = s[0][0];
+    float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mt][i]);
+    for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, s[0][i]), s[1][i]);
     mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-    const float alpha = fast_exp2((m - m_use) * p.c);
-    const float mc = m_use * p.c;
-    float rs = 0.0f;
+    if (__any(mx > m)) {  // rescale only when some row of the wavefront has a new maximum
+      const float m_new = fmaxf(m, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha = fast_exp2((m - m_use) * p.c);
+      l *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    }
+    const float mc = (m == -INFINITY) ? 0.0f : m * p.c;
+    float rs0 = 0.0f, rs1 = 0.0f;
     uint32_t pb[2][8];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -280,33 +312,30 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
       for (int i = 0; i < 16; i += 2) {
         const float p0 = fast_exp2(fmaf(s[mt][i], p.c, -mc));
         const float p1 = fast_exp2(fmaf(s[mt][i + 1], p.c, -mc));
-        rs += p0 + p1;
+        rs0 += p0;
+        rs1 += p1;
         pb[mt][i >> 1] = pack_bf16(p0, p1);
       }
-    l = l * alpha + rs;
-    m = m_new;
-#pragma unroll
-    for (int dt = 0; dt < D / 32; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    l += rs0 + rs1;
     // ---- O^T += V^T P^T ---------------------------------------------------------------------
+    const uint16_t* vbase_lds = (const uint16_t*)&sm.v[buf][0][0];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
-        const int ch = 2 * (2 * mt + j) + h;
+        const int krow = 32 * mt + 16 * j + v_row_off;
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
-          const int d = dt * 32 + n;
-          const u32x4_t vv = *(const u32x4_t*)&sm.vt[buf][d * BN + ((ch ^ vt_swz(d)) << 3)];
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vv), pf, o[dt], 0, 0, 0);
+          const u32x2_t lo = lds_read_tr16(vbase_lds + krow * (Smem<D>::VCH16 * 8) + 32 * dt + v_col_off);
+          const u32x2_t hi = lds_read_tr16(vbase_lds + (krow + 8) * (Smem<D>::VCH16 * 8) + 32 * dt + v_col_off);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
         }
       }
     // ---- stage the next tile ------------------------------------------------------------------
     if (t + 1 < tile_end) {
-      commit_tile<D, U8>(st, sm, buf ^ 1, tid);
-      if (t + 2 < tile_end) fetch_tile<D, U8>(st, p, b, kvh, (t + 2) * BN, tid);
+      ld.commit(st, sm, buf ^ 1, tid);
+      if (t + 2 < tile_end) ld.fetch(st, t + 2, tid);
     }
     __syncthreads();
   }
