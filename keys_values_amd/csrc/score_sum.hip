@@ -36,9 +36,9 @@ struct ScoreParams {
 };
 
 template <int D>
-struct Smem {
-  static constexpr int QROW = D + 8;
-  uint16_t q[2][BQ * QROW];
+struct alignas(16) Smem {
+  static constexpr int QCH16 = D / 8 + 1;  // 16-byte chunks per row incl. pad (conflict-free ds_read_b128)
+  u32x4_t q[2][BQ][QCH16];
   float lse[2][BQ];
   int32_t qpos[2][BQ];
 };
@@ -51,44 +51,78 @@ struct QStage {
   int32_t qpos;
 };
 
+// Streams the packed query rows (row r = query r / G, head r % G) of one (batch, KV head) pair.
+// The (query, head) of each row this thread loads is advanced incrementally from tile to tile,
+// so the loop has no integer division.
 template <int D>
-__device__ __forceinline__ void fetch_q(QStage<D>& s, const ScoreParams& p, int b, int kvh, int row0, int tid) {
-  constexpr int CPR = D / 8;
-  constexpr int RPI = NTHREADS / CPR;
-  const int col = tid % CPR;
-  const int row_in = tid / CPR;
-#pragma unroll
-  for (int i = 0; i < QStage<D>::QCH; ++i) {
-    const int row = row0 + row_in + i * RPI;
-    const bool ok = row < p.R;
-    const int qi = row / p.G, g = row % p.G;
-    const uint16_t* src = p.q + b * p.q_sb + (int64_t)(kvh * p.G + g) * p.q_sh + (int64_t)qi * p.q_st + col * 8;
-    s.qr[i] = ok ? *(const u32x4_t*)src : u32x4_t{0, 0, 0, 0};
-  }
-  if (tid < BQ) {
-    const int row = row0 + tid;
-    const bool ok = row < p.R;
-    const int qi = row / p.G, g = row % p.G;
-    // rows past the end get lse = +inf so that exp2(... - lse) = 0
-    s.lse = ok ? p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] : INFINITY;
-    s.qpos = ok ? p.input_pos + qi : INT_MAX;
-  }
-}
+struct QLoader {
+  static constexpr int CPR = D / 8;
+  static constexpr int RPI = NTHREADS / CPR;
+  static constexpr int QCH = QStage<D>::QCH;
+  const uint16_t* qbase;  // (b, first head of the group)
+  const float* lbase;     // lse + b * q_len * Hq + kvh * G
+  int64_t q_sh, q_st;
+  int G, R, Hq, input_pos, row_in, col;
+  int qi[QCH], g[QCH];    // row of chunk i in the current tile
+  int lqi, lg;            // row of the lse / position this thread stages (tid < BQ)
+  int dq, dg;             // BQ / G, BQ % G
 
-template <int D>
-__device__ __forceinline__ void commit_q(const QStage<D>& s, Smem<D>& sm, int buf, int tid) {
-  constexpr int CPR = D / 8;
-  constexpr int RPI = NTHREADS / CPR;
-  const int col = tid % CPR;
-  const int row_in = tid / CPR;
+  __device__ __forceinline__ void init(const ScoreParams& p, int b, int kvh, int tid) {
+    col = tid % CPR;
+    row_in = tid / CPR;
+    G = p.G; R = p.R; Hq = p.Hq; input_pos = p.input_pos;
+    q_sh = p.q_sh; q_st = p.q_st;
+    qbase = p.q + b * p.q_sb + (int64_t)(kvh * p.G) * p.q_sh;
+    lbase = p.lse + (int64_t)b * p.q_len * p.Hq + kvh * p.G;
+    dq = BQ / G; dg = BQ % G;
 #pragma unroll
-  for (int i = 0; i < QStage<D>::QCH; ++i)
-    *(u32x4_t*)&sm.q[buf][(row_in + i * RPI) * Smem<D>::QROW + col * 8] = s.qr[i];
-  if (tid < BQ) {
-    sm.lse[buf][tid] = s.lse;
-    sm.qpos[buf][tid] = s.qpos;
+    for (int i = 0; i < QCH; ++i) {
+      const int r = row_in + i * RPI;
+      qi[i] = r / G;
+      g[i] = r % G;
+    }
+    lqi = tid / G;
+    lg = tid % G;
   }
-}
+
+  // fetch the tile whose first row is row0, then step the row bookkeeping to the next tile
+  __device__ __forceinline__ void fetch(QStage<D>& s, int row0, int tid) {
+#pragma unroll
+    for (int i = 0; i < QCH; ++i) {
+      const bool ok = row0 + row_in + i * RPI < R;
+      const uint16_t* src = qbase + (int64_t)g[i] * q_sh + (int64_t)(ok ? qi[i] : 0) * q_st + col * 8;
+      const u32x4_t v = *(const u32x4_t*)(ok ? src : qbase);
+      s.qr[i] = ok ? v : u32x4_t{0, 0, 0, 0};
+      qi[i] += dq;
+      g[i] += dg;
+      if (g[i] >= G) {
+        g[i] -= G;
+        qi[i] += 1;
+      }
+    }
+    if (tid < BQ) {
+      const bool ok = row0 + tid < R;
+      // rows past the end get lse = +inf so that exp2(... - lse) = 0
+      s.lse = ok ? lbase[(int64_t)lqi * Hq + lg] : INFINITY;
+      s.qpos = ok ? input_pos + lqi : INT_MAX;
+      lqi += dq;
+      lg += dg;
+      if (lg >= G) {
+        lg -= G;
+        lqi += 1;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void commit(const QStage<D>& s, Smem<D>& sm, int buf, int tid) const {
+#pragma unroll
+    for (int i = 0; i < QCH; ++i) sm.q[buf][row_in + i * RPI][col] = s.qr[i];
+    if (tid < BQ) {
+      sm.lse[buf][tid] = s.lse;
+      sm.qpos[buf][tid] = s.qpos;
+    }
+  }
+};
 
 template <int D, bool U8>
 __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParams p) {
@@ -142,10 +176,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
 
   float wacc[2] = {0.0f, 0.0f};
   const int num_qt = (p.R + BQ - 1) / BQ;
+  QLoader<D> ld;
+  ld.init(p, b, kvh, tid);
   QStage<D> st;
-  fetch_q<D>(st, p, b, kvh, 0, tid);
-  commit_q<D>(st, sm, 0, tid);
-  if (num_qt > 1) fetch_q<D>(st, p, b, kvh, BQ, tid);
+  ld.fetch(st, 0, tid);
+  ld.commit(st, sm, 0, tid);
+  if (num_qt > 1) ld.fetch(st, BQ, tid);
   __syncthreads();
 
   for (int t = 0; t < num_qt; ++t) {
@@ -161,7 +197,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
         for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
 #pragma unroll
       for (int j = 0; j < D / 16; ++j) {
-        const u32x4_t qq = *(const u32x4_t*)&sm.q[buf][(mt * 32 + n) * Smem<D>::QROW + 16 * j + 8 * h];
+        const u32x4_t qq = sm.q[buf][mt * 32 + n][2 * j + h];
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
           s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], s[nt], 0, 0, 0);
@@ -197,8 +233,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
       }
     }
     if (t + 1 < num_qt) {
-      commit_q<D>(st, sm, buf ^ 1, tid);
-      if (t + 2 < num_qt) fetch_q<D>(st, p, b, kvh, (t + 2) * BQ, tid);
+      ld.commit(st, sm, buf ^ 1, tid);
+      if (t + 2 < num_qt) ld.fetch(st, (t + 2) * BQ, tid);
     }
     __syncthreads();
   }
