@@ -14,17 +14,22 @@
 //   wavefront holds the remaining keys of that row, so the online softmax needs a single
 //   cross-lane exchange per tile. The accumulator layout of S^T is exactly the B-operand layout
 //   of the second product O^T = V^T P^T once the 16 keys of a k-step are taken in the order
-//   (0..3, 8..11 | 4..7, 12..15); V is therefore staged transposed in LDS with that key order.
-//   K/V tiles are double-buffered: the next tile is fetched into registers while the current one
-//   is multiplied, and written to the other LDS buffer before the single barrier of the iteration.
+//   (0..3, 8..11 | 4..7, 12..15); the V^T operand is read from the row-major V tile with the
+//   transposing LDS read (ds_read_b64_tr_b16), which delivers exactly that order.
+//   K/V tiles travel global -> LDS by DMA (global_load_lds_dwordx4, no registers), double-buffered,
+//   rows unpadded and XOR-swizzled against bank conflicts. The loop is software-pipelined: the
+//   matrix cores add V(t-1) P(t-1) to O while the vector ALU turns S(t) into P(t).
+#include <type_traits>
+
 #include "kvx_common.h"
 
 namespace kvx {
 namespace {
 
-constexpr int BM = 128;  // rows per workgroup
+constexpr int NWAVES = 4;        // wavefronts per workgroup, 32 rows each
+constexpr int BM = 32 * NWAVES;  // rows per workgroup
 constexpr int BN = 64;   // keys per tile
-constexpr int NTHREADS = 256;
+constexpr int NTHREADS = 64 * NWAVES;
 
 struct PrefillParams {
   const uint16_t* q;
@@ -46,14 +51,24 @@ struct PrefillParams {
   int64_t qs_sb, qs_sh, tp_sb, tp_sh;
 };
 
+// K and V tiles in LDS: [key][16-byte chunk], rows unpadded (D * 2 bytes), chunk c of row r stored at
+// position c ^ key(r). Unpadded rows are what the global -> LDS DMA writes (a wavefront fills 1024
+// contiguous bytes per instruction); the XOR then has to spread what one LDS phase touches over
+// the 64 banks (measured on gfx950: a ds_read_b128 phase serves 16 lanes, a ds_read_b64_tr_b16
+// phase 16 lanes):
+//   K, ds_read_b128:        16 consecutive rows, the same chunk      -> swz_k distinct over 16 rows
+//   V, ds_read_b64_tr_b16:  4 consecutive rows x chunks {c, c + 1}   -> bits 1..2 of swz_v distinct over r % 4
+// Both depend on r % 16 only, so they repeat for the row groups a wavefront loads (16 or 32 rows apart).
+template <int CPR>
+__device__ __forceinline__ int swz_k(int r) { return CPR == 16 ? (r & 15) : ((r >> 1) & 7); }
+template <int CPR>
+__device__ __forceinline__ int swz_v(int r) { return ((r & 3) << 1) | ((r >> 2) & 1); }
+
 template <int D>
 struct alignas(16) Smem {
-  static constexpr int KCH16 = D / 8 + 1;   // 16-byte chunks per K row incl. pad: row stride = 4 banks mod 64,
-                                            // so the 16 rows a ds_read_b128 phase touches hit distinct banks
-  static constexpr int VCH16 = D / 8 + 4;   // V row stride = 16 banks mod 64: the 4 rows x 64 bytes a pair of
-                                            // 16-lane transpose-read groups touches hit distinct banks
-  u32x4_t k[2][BN][KCH16];                  // [key][d]
-  u32x4_t v[2][BN][VCH16];                  // [key][d]
+  static constexpr int CPR = D / 8;  // 16-byte chunks per row
+  u32x4_t k[2][BN][CPR];
+  u32x4_t v[2][BN][CPR];
   int32_t tp[2][BN];
 };
 
@@ -66,6 +81,27 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const void* p) {
   return __builtin_bit_cast(u32x2_t, t);
 }
 
+// 16 bytes per lane straight from global memory into LDS (global_load_lds_dwordx4): lane l lands at
+// lds_addr + 16 l, lds_addr uniform over the wavefront. Written as inline assembly so that the
+// compiler does not serialise later LDS reads of OTHER buffers behind the transfer; the kernel
+// waits for its transfers itself (s_waitcnt vmcnt(0)) before the barrier that publishes a tile.
+__device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory", "m0");
+}
+// same for 4 bytes per lane (global_load_lds_dword): lane l lands at lds_addr + 4 l
+__device__ __forceinline__ void dma4(const char* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
+  return (uint32_t)(uintptr_t)((const __attribute__((address_space(3))) char*)p);
+}
+
 // 8 codes (two dwords) -> 8 bf16 (four dwords)
 __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
   u32x4_t r;
@@ -76,38 +112,38 @@ __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp
   return r;
 }
 
-template <int D, bool U8>
-struct Stage {
-  // registers holding one prefetched K/V tile of this thread: KCH rows, one 16-byte chunk each
-  static constexpr int KCH = (BN * D / 8) / NTHREADS;  // 4 (D=128), 2 (D=64)
-  u32x4_t kr[KCH];
-  u32x4_t vr[KCH];
-  float ks[KCH], vs[KCH];
-  int32_t kz[KCH], vz[KCH];
-  int32_t tpv;
-};
-
+// Tile loader. A wavefront instruction covers RPW = 64 / CPR whole rows; wavefront w of the
+// workgroup takes row groups w, w + 4, ... of the 64-row tile (NI groups each for K and for V).
+// bf16 cache: DMA into LDS. uint8 cache: codes and row state go through registers (prefetched one
+// tile ahead like the DMA), are dequantised to bf16 and written to the same LDS layout.
 template <int D, bool U8>
 struct Loader {
-  static constexpr int CPR = D / 8;             // chunks per row
-  static constexpr int RPI = NTHREADS / CPR;    // rows per pass of the workgroup
-  static constexpr int KCH = Stage<D, U8>::KCH;
-  static constexpr int ESZ = U8 ? 1 : 2;        // bytes per element in memory
-  const char* kbase;                            // (b, kvh) slice, uniform
+  static constexpr int CPR = D / 8;
+  static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
+  static constexpr int NI = BN / RPW / NWAVES;     // instructions per wavefront per operand: 4 / 2
+  static constexpr int ESZ = U8 ? 1 : 2;
+  const char* kbase;
   const char* vbase;
   const float* ks;
   const int32_t* kz;
   const float* vs;
   const int32_t* vz;
-  const int32_t* tp;                            // may be NULL
-  uint32_t koff[KCH], voff[KCH];                // byte offsets of this thread's chunks inside a tile
-  int64_t k_tile_bytes, v_tile_bytes;
-  int64_t k_st, v_st;
-  int row_in, col, kv_len;
+  const int32_t* tp;
+  uint32_t koff, voff;          // byte offset of this lane's chunk of row group 0 inside a tile (source side swizzled)
+  int64_t k_tile_bytes, v_tile_bytes, k_st, v_st;
+  int64_t k_step, v_step;       // bytes between this wavefront's consecutive row groups (NWAVES RPW rows)
+  int wave, lane, kv_len, rl, cgk, cgv;
+  // uint8 path staging registers
+  u32x2_t kc[NI], vc[NI];
+  float ksr[NI], vsr[NI];
+  int32_t kzr[NI], vzr[NI];
+
+  __device__ __forceinline__ int row_of(int i) const { return (NWAVES * i + wave) * RPW + rl; }
 
   __device__ __forceinline__ void init(const PrefillParams& p, int b, int kvh, int tid) {
-    col = tid % CPR;
-    row_in = tid / CPR;
+    wave = tid >> 6;
+    lane = tid & 63;
+    rl = lane / CPR;  // row inside the group
     kv_len = p.kv_len;
     k_st = p.k_st;
     v_st = p.v_st;
@@ -121,80 +157,88 @@ struct Loader {
     tp = p.tp ? p.tp + b * p.tp_sb + kvh * p.tp_sh : nullptr;
     k_tile_bytes = (int64_t)BN * p.k_st * ESZ;
     v_tile_bytes = (int64_t)BN * p.v_st * ESZ;
-#pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      koff[i] = (uint32_t)((row_in + i * RPI) * p.k_st * ESZ + col * 8 * ESZ);
-      voff[i] = (uint32_t)((row_in + i * RPI) * p.v_st * ESZ + col * 8 * ESZ);
-    }
+    // row groups of one wavefront are NWAVES RPW rows apart, a multiple of 16: the XOR keys and with them
+    // the source chunks are the same for all of them
+    const int r = row_of(0);
+    cgk = (lane % CPR) ^ swz_k<CPR>(r);  // the chunk that belongs at LDS position lane % CPR of row r
+    cgv = (lane % CPR) ^ swz_v<CPR>(r);
+    koff = (uint32_t)(r * p.k_st * ESZ + cgk * 8 * ESZ);
+    voff = (uint32_t)(r * p.v_st * ESZ + cgv * 8 * ESZ);
+    k_step = (int64_t)NWAVES * RPW * p.k_st * ESZ;
+    v_step = (int64_t)NWAVES * RPW * p.v_st * ESZ;
   }
 
-  __device__ __forceinline__ void fetch(Stage<D, U8>& s, int tile, int tid) const {
+  template <bool IS_K>
+  __device__ __forceinline__ void issue_one(Smem<D>& sm, int tile, int buf, int tid) {
     const int key0 = tile * BN;
-    const char* kt = kbase + tile * k_tile_bytes;
-    const char* vt = vbase + tile * v_tile_bytes;
+    const char* base = IS_K ? kbase : vbase;
+    const int64_t st = IS_K ? k_st : v_st;
+    const int64_t step = IS_K ? k_step : v_step;
+    const uint32_t off0 = IS_K ? koff : voff;
+    const char* tb = base + tile * (IS_K ? k_tile_bytes : v_tile_bytes);
     if (key0 + BN <= kv_len) {
 #pragma unroll
-      for (int i = 0; i < KCH; ++i) {
+      for (int i = 0; i < NI; ++i) {
         if constexpr (!U8) {
-          s.kr[i] = *(const u32x4_t*)(kt + koff[i]);
-          s.vr[i] = *(const u32x4_t*)(vt + voff[i]);
+          const uint32_t dst = lds_addr_of(IS_K ? &sm.k[buf][(NWAVES * i + wave) * RPW][0] : &sm.v[buf][(NWAVES * i + wave) * RPW][0]);
+          dma16(tb + i * step, off0, __builtin_amdgcn_readfirstlane(dst));
         } else {
-          const u32x2_t ck = *(const u32x2_t*)(kt + koff[i]);
-          const u32x2_t cv = *(const u32x2_t*)(vt + voff[i]);
-          s.kr[i] = u32x4_t{ck[0], ck[1], 0, 0};
-          s.vr[i] = u32x4_t{cv[0], cv[1], 0, 0};
-          const int key = key0 + row_in + i * RPI;
-          s.ks[i] = ks[key];
-          s.kz[i] = kz[key];
-          s.vs[i] = vs[key];
-          s.vz[i] = vz[key];
+          const int key = key0 + row_of(i);
+          const u32x2_t c = *(const u32x2_t*)(tb + i * step + off0);
+          if (IS_K) { kc[i] = c; ksr[i] = ks[key]; kzr[i] = kz[key]; }
+          else { vc[i] = c; vsr[i] = vs[key]; vzr[i] = vz[key]; }
         }
       }
-      if (tid < BN) s.tpv = tp ? tp[key0 + tid] : key0 + tid;
     } else {
       // last, partial tile: rows past the end re-read the last valid row (finite data); their
       // position is INT_MAX, so they are masked for every query and contribute exactly zero
 #pragma unroll
-      for (int i = 0; i < KCH; ++i) {
-        const int key = min(key0 + row_in + i * RPI, kv_len - 1);
+      for (int i = 0; i < NI; ++i) {
+        const int key = min(key0 + row_of(i), kv_len - 1);
+        const uint32_t off = (uint32_t)(((int64_t)(key - key0) * st + (IS_K ? cgk : cgv) * 8) * ESZ);
         if constexpr (!U8) {
-          s.kr[i] = *(const u32x4_t*)(kbase + ((int64_t)key * k_st + col * 8) * ESZ);
-          s.vr[i] = *(const u32x4_t*)(vbase + ((int64_t)key * v_st + col * 8) * ESZ);
+          const uint32_t dst = lds_addr_of(IS_K ? &sm.k[buf][(NWAVES * i + wave) * RPW][0] : &sm.v[buf][(NWAVES * i + wave) * RPW][0]);
+          dma16(tb, off, __builtin_amdgcn_readfirstlane(dst));
         } else {
-          const u32x2_t ck = *(const u32x2_t*)(kbase + ((int64_t)key * k_st + col * 8));
-          const u32x2_t cv = *(const u32x2_t*)(vbase + ((int64_t)key * v_st + col * 8));
-          s.kr[i] = u32x4_t{ck[0], ck[1], 0, 0};
-          s.vr[i] = u32x4_t{cv[0], cv[1], 0, 0};
-          s.ks[i] = ks[key];
-          s.kz[i] = kz[key];
-          s.vs[i] = vs[key];
-          s.vz[i] = vz[key];
+          const u32x2_t c = *(const u32x2_t*)(tb + off);
+          if (IS_K) { kc[i] = c; ksr[i] = ks[key]; kzr[i] = kz[key]; }
+          else { vc[i] = c; vsr[i] = vs[key]; vzr[i] = vz[key]; }
         }
       }
-      if (tid < BN) {
-        const int key = key0 + tid;
-        s.tpv = key < kv_len ? (tp ? tp[key] : key) : INT_MAX;
-      }
+    }
+    // token positions of the K tile: one 4-byte DMA per lane of wavefront 0 (slots past the end
+    // re-read the last valid one and are overwritten with INT_MAX when the tile lands)
+    if (IS_K && tp && wave == 0) {
+      const uint32_t dst = lds_addr_of(&sm.tp[buf][0]);
+      dma4((const char*)(tp + key0), (uint32_t)min(lane, kv_len - 1 - key0) * 4, __builtin_amdgcn_readfirstlane(dst));
     }
   }
 
-  __device__ __forceinline__ void commit(const Stage<D, U8>& s, Smem<D>& sm, int buf, int tid) const {
+  // make tile `tile`, issued last, visible in LDS (called after s_waitcnt vmcnt(0), before the
+  // barrier that publishes it)
+  template <bool IS_K>
+  __device__ __forceinline__ void land(Smem<D>& sm, int tile, int buf, int tid) {
+    if constexpr (U8) {
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      u32x4_t kk = s.kr[i], vv = s.vr[i];
-      if constexpr (U8) {
-        kk = dequant8(kk[0], kk[1], s.kz[i], s.ks[i]);
-        vv = dequant8(vv[0], vv[1], s.vz[i], s.vs[i]);
+      for (int i = 0; i < NI; ++i) {
+        const int r = row_of(i);
+        if (IS_K) sm.k[buf][r][lane % CPR] = dequant8(kc[i][0], kc[i][1], kzr[i], ksr[i]);
+        else sm.v[buf][r][lane % CPR] = dequant8(vc[i][0], vc[i][1], vzr[i], vsr[i]);
       }
-      sm.k[buf][row_in + i * RPI][col] = kk;
-      sm.v[buf][row_in + i * RPI][col] = vv;
     }
-    if (tid < BN) sm.tp[buf][tid] = s.tpv;
+    if (IS_K && tid < BN) {
+      const int key = tile * BN + tid;
+      if (!tp) sm.tp[buf][tid] = key < kv_len ? key : INT_MAX;
+      else if (key >= kv_len) sm.tp[buf][tid] = INT_MAX;
+    }
   }
 };
 
 template <int D, bool U8>
 __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const PrefillParams p) {
+  constexpr int CPR = D / 8;
+  constexpr int KS = D / 16;  // k-steps of the first product
+  constexpr int DT = D / 32;  // d tiles of the second product
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -218,91 +262,133 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
   const int qpos_min_w = p.input_pos + min(row0w, p.R - 1) / p.G;
 
   // Q fragments (B operand): lane holds row n, d = 16 j + 8 h .. +8
-  bf16x8_t qf[D / 16];
+  bf16x8_t qf[KS];
   {
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)(kvh * p.G + g) * p.q_sh + (int64_t)qi * p.q_st;
 #pragma unroll
-    for (int j = 0; j < D / 16; ++j) {
+    for (int j = 0; j < KS; ++j) {
       u32x4_t t = row_ok ? *(const u32x4_t*)(qp + 16 * j + 8 * h) : u32x4_t{0, 0, 0, 0};
       qf[j] = as_bf16x8(t);
     }
   }
 
+  // LDS byte offsets of this lane's operand fragments inside a tile buffer.
+  // K (A operand of S^T = K Q^T): row 32 mt + n, chunk 2 j + h, stored at position chunk ^ swz_k(row).
+  uint32_t ka[KS];
+#pragma unroll
+  for (int j = 0; j < KS; ++j) ka[j] = (uint32_t)(n * CPR + ((2 * j + h) ^ swz_k<CPR>(n))) * 16;
+  // V (A operand of O^T = V^T P^T) through the transposing read: in its group of 16 lanes this lane
+  // points at key row (i / 4) + 4 h of the 16-key block and at d columns 16 * (group % 2) + 4 (i % 4) .. +3
+  // of the 32-d tile; the second read of a k-step is 8 rows further down (same XOR key, same positions).
+  const int li = lane & 15;
+  const int vrow = (li >> 2) + 4 * h;                              // + 32 mt + 16 j (+ 8)
+  const int vcol = 16 * ((lane >> 4) & 1) + 4 * (li & 3);          // + 32 dt, bf16 elements
+  uint32_t va[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int c = (32 * dt + vcol) >> 3;
+    va[dt] = (uint32_t)((vrow * CPR + (c ^ swz_v<CPR>(vrow))) * 16 + (vcol & 7) * 2);
+  }
+
   const int tile_begin = split * p.tiles_per_split;
   const int tile_end = min(tile_begin + p.tiles_per_split, p.num_tiles);
 
-  f32x16_t o[D / 32];
+  f32x16_t o[DT];
 #pragma unroll
-  for (int dt = 0; dt < D / 32; ++dt)
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
   float m = -INFINITY;  // running max of the raw (unscaled) scores of this row
   float l = 0.0f;       // this lane's share of the running sum
 
-  // transpose-read addressing of V: in its group of 16 lanes this lane points at key row (i / 4)
-  // and at d columns 4 (i % 4) .. +3 of the 16 d columns the group produces
-  const int li = lane & 15;
-  const int v_row_off = (li >> 2) + 4 * h;                      // + 32 mt + 16 j (+ 8)
-  const int v_col_off = 16 * ((lane >> 4) & 1) + 4 * (li & 3);  // + 32 dt, in bf16 elements
-
-  Loader<D, U8> ld;
-  ld.init(p, b, kvh, tid);
-  Stage<D, U8> st;
-  if (tile_begin < tile_end) {
-    ld.fetch(st, tile_begin, tid);
-    ld.commit(st, sm, 0, tid);
-    if (tile_begin + 1 < tile_end) ld.fetch(st, tile_begin + 1, tid);
-  }
-  __syncthreads();
-
-  for (int t = tile_begin; t < tile_end; ++t) {
-    const int buf = (t - tile_begin) & 1;
-    // ---- S^T = K Q^T: two independent accumulator chains -----------------------------------
-    f32x16_t s[2];
+  // S^T of one tile from the K tile in k[buf]: two independent accumulator chains
+  auto qk = [&](f32x16_t (&s)[2], int buf) {
+    const char* kb = (const char*)&sm.k[buf][0][0];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[mt][i] = 0.0f;
 #pragma unroll
-    for (int j = 0; j < D / 16; ++j) {
+    for (int j = 0; j < KS; ++j)
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
-        const u32x4_t kk = sm.k[buf][mt * 32 + n][2 * j + h];
+        const u32x4_t kk = *(const u32x4_t*)(kb + ka[j] + mt * 32 * CPR * 16);
         s[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kk), qf[j], s[mt], 0, 0, 0);
       }
+  };
+  // mask (only tiles that hold a position some row of this wavefront may not see)
+  auto mask = [&](f32x16_t (&s)[2], int buf) {
+    const int tpl = sm.tp[buf][lane];
+    if (__any(tpl > qpos_min_w)) {
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int4 tq = *(const int4*)&sm.tp[buf][mt * 32 + 8 * a + 4 * h];
+          if (tq.x > qpos) s[mt][4 * a + 0] = -INFINITY;
+          if (tq.y > qpos) s[mt][4 * a + 1] = -INFINITY;
+          if (tq.z > qpos) s[mt][4 * a + 2] = -INFINITY;
+          if (tq.w > qpos) s[mt][4 * a + 3] = -INFINITY;
+        }
     }
-    // ---- mask (only tiles that hold a position some row of this wavefront may not see) ----
-    {
-      const int tpl = sm.tp[buf][lane];
-      if (__any(tpl > qpos_min_w)) {
+  };
+
+  // second product for one tile: O^T += V^T P^T with V from v[buf]
+  auto pv = [&](const uint32_t (&pb)[2][8], int buf) {
+    const char* vl = (const char*)&sm.v[buf][0][0];
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            const int4 tq = *(const int4*)&sm.tp[buf][mt * 32 + 8 * a + 4 * h];
-            if (tq.x > qpos) s[mt][4 * a + 0] = -INFINITY;
-            if (tq.y > qpos) s[mt][4 * a + 1] = -INFINITY;
-            if (tq.z > qpos) s[mt][4 * a + 2] = -INFINITY;
-            if (tq.w > qpos) s[mt][4 * a + 3] = -INFINITY;
-          }
+      for (int j = 0; j < 2; ++j) {
+        const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
+        const int rb = (32 * mt + 16 * j) * CPR * 16;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const u32x2_t lo = lds_read_tr16(vl + rb + va[dt]);
+          const u32x2_t hi = lds_read_tr16(vl + rb + va[dt] + 8 * CPR * 16);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
+        }
       }
-    }
-    // ---- online softmax --------------------------------------------------------------------
+  };
+
+  // Pipeline: iteration t multiplies S(t) = K(t) Q^T, then lets the matrix cores add V(t-1) P(t-1)
+  // to O while the vector ALU turns S(t) into P(t). K(t) sits in k[t & 1]; V(t-1) in v[(t-1) & 1];
+  // K(t+1) and V(t) are in flight to the other buffers and are published by the barrier that ends
+  // the iteration.
+  Loader<D, U8> ld;
+  ld.init(p, b, kvh, tid);
+  uint32_t pb_prev[2][8];
+  // every split owns at least one tile (the host sizes the splits that way)
+  ld.template issue_one<true>(sm, tile_begin, 0, tid);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first K tile and the Q fragments have arrived
+  ld.template land<true>(sm, tile_begin, 0, tid);
+  __syncthreads();
+  // one pipeline step; the first one has no previous tile to multiply
+  auto step = [&](auto first_tag, int t) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    const int cur = (t - tile_begin) & 1;
+    const bool has1 = t + 1 < tile_end;
+    ld.template issue_one<false>(sm, t, cur, tid);
+    if (has1) ld.template issue_one<true>(sm, t + 1, cur ^ 1, tid);
+    f32x16_t s[2];
+    qk(s, cur);
+    mask(s, cur);
+    // ---- running maximum; rescale only when some row of the wavefront has a new maximum ------
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, s[0][i]), s[1][i]);
     mx = fmaxf(mx, xor32(mx));
-    if (__any(mx > m)) {  // rescale only when some row of the wavefront has a new maximum
+    float alpha = 1.0f;
+    const bool resc = __any(mx > m);
+    if (resc) {
       const float m_new = fmaxf(m, mx);
       const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float alpha = fast_exp2((m - m_use) * p.c);
+      alpha = fast_exp2((m - m_use) * p.c);
       l *= alpha;
       m = m_new;
-#pragma unroll
-      for (int dt = 0; dt < D / 32; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
     }
+    // ---- O += V(t-1) P(t-1) on the matrix cores, P(t) = exp2(c S(t) - c m) on the vector ALU ----
+    if constexpr (!FIRST) pv(pb_prev, cur ^ 1);
     const float mc = (m == -INFINITY) ? 0.0f : m * p.c;
     float rs0 = 0.0f, rs1 = 0.0f;
     uint32_t pb[2][8];
@@ -317,28 +403,44 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
         pb[mt][i >> 1] = pack_bf16(p0, p1);
       }
     l += rs0 + rs1;
-    // ---- O^T += V^T P^T ---------------------------------------------------------------------
-    const uint16_t* vbase_lds = (const uint16_t*)&sm.v[buf][0][0];
+    if constexpr (!FIRST) {
+      // interleave in the instruction stream: each matrix instruction of the second product is
+      // followed by the two LDS reads of the next one and by its share of the softmax arithmetic,
+      // so the vector ALU works in the shadow of the matrix core instead of after it
+#pragma unroll
+      for (int i = 0; i < 4 * DT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 LDS reads
+        __builtin_amdgcn_sched_group_barrier(0x002, 20 / DT, 0);  // VALU (fma, add, cvt)
+        __builtin_amdgcn_sched_group_barrier(0x400, 8 / DT, 0);   // transcendental (exp2)
+      }
+      // keep the softmax arithmetic in this block: without a use here the optimiser sinks it
+      // past the barrier below, out of the matrix core's shadow
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(pb[mt][i]));
+      asm volatile("" : "+v"(l));
+      if (resc) {  // O (now including tile t-1) moves to the new reference maximum
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+      }
+    }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
-        const int krow = 32 * mt + 16 * j + v_row_off;
-#pragma unroll
-        for (int dt = 0; dt < D / 32; ++dt) {
-          const u32x2_t lo = lds_read_tr16(vbase_lds + krow * (Smem<D>::VCH16 * 8) + 32 * dt + v_col_off);
-          const u32x2_t hi = lds_read_tr16(vbase_lds + (krow + 8) * (Smem<D>::VCH16 * 8) + 32 * dt + v_col_off);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
-        }
-      }
-    // ---- stage the next tile ------------------------------------------------------------------
-    if (t + 1 < tile_end) {
-      ld.commit(st, sm, buf ^ 1, tid);
-      if (t + 2 < tile_end) ld.fetch(st, t + 2, tid);
-    }
+      for (int i = 0; i < 8; ++i) pb_prev[mt][i] = pb[mt][i];
+    // ---- publish the tiles that were in flight -------------------------------------------------
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's DMA / loads have landed
+    ld.template land<false>(sm, t, cur, tid);
+    if (has1) ld.template land<true>(sm, t + 1, cur ^ 1, tid);
     __syncthreads();
-  }
+  };
+  step(std::true_type{}, tile_begin);
+  for (int t = tile_begin + 1; t < tile_end; ++t) step(std::false_type{}, t);
+  pv(pb_prev, (tile_end - 1 - tile_begin) & 1);
 
   // ---- epilogue -----------------------------------------------------------------------------
   const float lt = l + xor32(l);
@@ -347,7 +449,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
     if (row_ok) {
       uint16_t* op = p.o + b * p.o_sb + (int64_t)(kvh * p.G + g) * p.o_sh + (int64_t)qi * p.o_st;
 #pragma unroll
-      for (int dt = 0; dt < D / 32; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
           u32x2_t w2;
@@ -362,7 +464,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
       const int64_t prow = ((int64_t)split * p.B * p.Hkv + group) * p.R + row;
       float* po = p.part_o + prow * D;
 #pragma unroll
-      for (int dt = 0; dt < D / 32; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
           f32x4_t w4 = {o[dt][4 * a], o[dt][4 * a + 1], o[dt][4 * a + 2], o[dt][4 * a + 3]};
