@@ -141,6 +141,19 @@ int kvx_sdpa_prefill_weights(const kvx_sdpa_args* args, void* stream);
 int kvx_sdpa_decode(const kvx_sdpa_args* args, void* stream);
 size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* args);
 
+/* Single-token decode fused with the H2O bookkeeping that follows it in one cache step
+ * (DefaultKVCache.forward for one new token: self.mha(...) then self._update(...),
+ * keys_values/kvcache/base.py:583-595; H2OKVCache._compute_scores, keys_values/kvcache/h2o.py:175-196;
+ * the argsort whose first entry the next step consumes, keys_values/kvcache/attn_weights.py:773-774):
+ * kvx_sdpa_decode followed by kvx_h2o_update_select with k = 1, except that the score-sums go
+ * straight from the kernel that produces them into scores += W and the per-row (value, slot)
+ * minimum, without a round trip through memory. h->k must be 1, h->kv_len == args->kv_len;
+ * h->w is ignored; args->w may be NULL (W is then not written out). h->workspace as for
+ * kvx_h2o_update_select; args->workspace from kvx_sdpa_decode_h2o_workspace_bytes. */
+struct kvx_h2o_args;
+int kvx_sdpa_decode_h2o(const kvx_sdpa_args* args, const struct kvx_h2o_args* h, void* stream);
+size_t kvx_sdpa_decode_h2o_workspace_bytes(const kvx_sdpa_args* args);
+
 /* ---- cache: quantiser ---------------------------------------------------------------------- */
 
 /* Affine 8-bit row quantiser: for each row x[0..D) (bf16, upcast to fp32)

@@ -74,6 +74,8 @@ SYMBOLS = {
     "kvx_sdpa_prefill_weights": (ctypes.c_int, [POINTER(SdpaArgs), c_void_p]),
     "kvx_sdpa_decode": (ctypes.c_int, [POINTER(SdpaArgs), c_void_p]),
     "kvx_sdpa_decode_workspace_bytes": (c_size_t, [POINTER(SdpaArgs)]),
+    "kvx_sdpa_decode_h2o": (ctypes.c_int, [POINTER(SdpaArgs), POINTER(H2OArgs), c_void_p]),
+    "kvx_sdpa_decode_h2o_workspace_bytes": (c_size_t, [POINTER(SdpaArgs)]),
     "kvx_quantize_rows": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "kvx_dequantize_rows": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
     "kvx_cache_write": (ctypes.c_int, [POINTER(CacheWriteArgs), c_void_p]),

@@ -143,7 +143,12 @@ int kvx_sdpa_prefill_weights(const kvx_sdpa_args* a, void* stream) {
 
 size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* a) {
   if (check_sdpa_common(a, "kvx_sdpa_decode_workspace_bytes", false) != KVX_OK) return 0;
-  return sdpa_decode_workspace(*a);
+  return sdpa_decode_workspace(*a, false);
+}
+
+size_t kvx_sdpa_decode_h2o_workspace_bytes(const kvx_sdpa_args* a) {
+  if (check_sdpa_common(a, "kvx_sdpa_decode_h2o_workspace_bytes", false) != KVX_OK) return 0;
+  return sdpa_decode_workspace(*a, true);
 }
 
 int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
@@ -153,7 +158,7 @@ int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
   const int G = a->Hq / a->Hkv;
   KVX_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in {1, 2, 4, 8}", G);
   KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_decode: workspace must be 16-byte aligned");
-  return launch_sdpa_decode(*a, (hipStream_t)stream);
+  return launch_sdpa_decode(*a, nullptr, (hipStream_t)stream);
 }
 
 int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale,
@@ -201,14 +206,35 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
 
 size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* a) { return a ? h2o_workspace(*a) : 0; }
 
+static int check_h2o(const kvx_h2o_args* a, const char* who) {
+  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "%s: h2o args is NULL", who);
+  KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->kv_len > 0, KVX_ERR_INVALID, "%s: sizes must be positive", who);
+  KVX_REQUIRE(a->limit > 0 && a->limit <= a->kv_len, KVX_ERR_INVALID, "%s: limit=%d must be in [1, kv_len=%d]", who, a->limit, a->kv_len);
+  KVX_REQUIRE(a->k >= 1 && a->k <= a->limit && a->k <= 4096, KVX_ERR_INVALID, "%s: k=%d must be in [1, min(limit, 4096)]", who, a->k);
+  KVX_REQUIRE(a->scores && a->next_index, KVX_ERR_INVALID, "%s: NULL pointer", who);
+  KVX_REQUIRE(!a->normalize || a->token_pos, KVX_ERR_INVALID, "%s: normalize needs token_pos", who);
+  return KVX_OK;
+}
+
 int kvx_h2o_update_select(const kvx_h2o_args* a, void* stream) {
-  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_h2o_update_select: args is NULL");
-  KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->kv_len > 0, KVX_ERR_INVALID, "kvx_h2o_update_select: sizes must be positive");
-  KVX_REQUIRE(a->limit > 0 && a->limit <= a->kv_len, KVX_ERR_INVALID, "kvx_h2o_update_select: limit=%d must be in [1, kv_len=%d]", a->limit, a->kv_len);
-  KVX_REQUIRE(a->k >= 1 && a->k <= a->limit && a->k <= 4096, KVX_ERR_INVALID, "kvx_h2o_update_select: k=%d must be in [1, min(limit, 4096)]", a->k);
-  KVX_REQUIRE(a->scores && a->next_index, KVX_ERR_INVALID, "kvx_h2o_update_select: NULL pointer");
-  KVX_REQUIRE(!a->normalize || a->token_pos, KVX_ERR_INVALID, "kvx_h2o_update_select: normalize needs token_pos");
+  int rc = check_h2o(a, "kvx_h2o_update_select");
+  if (rc != KVX_OK) return rc;
   return launch_h2o_update_select(*a, (hipStream_t)stream);
+}
+
+int kvx_sdpa_decode_h2o(const kvx_sdpa_args* a, const kvx_h2o_args* h, void* stream) {
+  int rc = check_sdpa_common(a, "kvx_sdpa_decode_h2o", true);
+  if (rc != KVX_OK) return rc;
+  rc = check_h2o(h, "kvx_sdpa_decode_h2o");
+  if (rc != KVX_OK) return rc;
+  KVX_REQUIRE(a->q_len == 1, KVX_ERR_INVALID, "kvx_sdpa_decode_h2o: q_len must be 1, got %d", a->q_len);
+  const int G = a->Hq / a->Hkv;
+  KVX_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode_h2o: group size %d not in {1, 2, 4, 8}", G);
+  KVX_REQUIRE(h->k == 1 && h->kv_len == a->kv_len && h->B == a->B && h->Hkv == a->Hkv, KVX_ERR_INVALID,
+              "kvx_sdpa_decode_h2o: needs k == 1 and the cache shape of the attention call");
+  KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_decode_h2o: workspace must be 16-byte aligned");
+  KVX_REQUIRE(h->workspace && h->workspace_bytes >= h2o_workspace(*h), KVX_ERR_WORKSPACE, "kvx_sdpa_decode_h2o: h2o workspace of %zu bytes needed", h2o_workspace(*h));
+  return launch_sdpa_decode(*a, h, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -6,17 +6,18 @@
 // weights afterwards, :838-854).
 //
 // Here one workgroup serves all G query heads of a (batch, KV head, split), so K and V cross HBM
-// once. Per block of keys (8192 / G of them) it runs three phases:
-//   1. logits = c * K q for the G heads with 16x16x32 bf16 MFMA: a K row is the A operand straight
-//      from global memory (16-byte loads, no LDS staging), the G query vectors sit in the B operand.
-//      The logits (log2 units) go to LDS and, when weights are wanted, to the fp32 logits scratch.
-//   2. with the block maximum known, p = exp2(logit - max) is written back to LDS as bf16 pairs of
-//      the two keys a lane will multiply together, and summed in fp32.
-//   3. O += p V with v_dot2_f32_bf16 on (key A, key B) pairs: a lane owns 8 consecutive d of the
-//      rows it loads (16-byte loads, a wavefront covers whole contiguous rows), accumulates in fp32
-//      registers and the partial sums are reduced across lanes and wavefronts once at the end.
+// once, in one pass with both streams in flight: 8 or 16 lanes share a row (a lane owns 8 consecutive
+// d, 16-byte loads, a wavefront instruction covers whole contiguous rows of K or V), the G logits of
+// a row are v_dot2_f32_bf16 sums reduced over the row's lanes with DPP adds, and O += p V runs on
+// the same lanes with dot2 over pairs of rows. Every row group of a wavefront keeps its own running
+// maximum, sum and fp32 accumulator (the maximum moves lazily), so the loop has no barrier and no
+// cross-lane traffic beyond the row reduction; groups and wavefronts are merged once at the end.
+// The logits (log2 units) are gathered in LDS and leave for the fp32 scratch, [key][head], in bursts
+// of 32 KB: a write stream mixed into the reads costs HBM far more than its share of the bytes.
 // A merge kernel combines the splits and produces the base-2 log-sum-exp; a last streaming kernel
-// turns the stored logits into W = (1/G) sum_g exp2(logit_g - lse_g). No float atomics anywhere.
+// turns the stored logits into W = (1/G) sum_g exp2(logit_g - lse_g) and, in the fused H2O form, adds
+// W to the cumulative scores and finds each row's lowest-score slot in the same pass. K and V are
+// touched once: they are loaded non-temporally. No float atomics anywhere.
 #include "kvx_common.h"
 
 namespace kvx {
@@ -36,7 +37,7 @@ struct DecodeParams {
   uint16_t* o;
   float* lse_out;  // user (B, 1, Hq) or NULL
   float* w;        // user (B, Hkv, kv_len) or NULL
-  float* logits;   // (B, Hq, Tpad)
+  float* logits;   // (B, Hkv, Tpad, G)
   float* part_o;   // (B, Hq, S, D)
   float* part_ml;  // (B, Hq, S, 2)
   float* lse_ws;   // (B, Hq)
@@ -54,281 +55,408 @@ __device__ __forceinline__ u32x4_t dq8(uint32_t c0, uint32_t c1, int32_t zp, flo
   return r;
 }
 
+// Sum over the LPR lanes that share a row. Every lane of the group ends with the same bits: each
+// step adds two values that the partner lane adds in the other order.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+template <int LPR>
+__device__ __forceinline__ float row_group_sum(float x) {
+  static_assert(LPR == 16 || LPR == 8, "row groups of 8 or 16 lanes");
+  if constexpr (LPR == 16) {
+    x = dpp_add<0x128>(x);  // row_ror:8
+    x = dpp_add<0x124>(x);  // row_ror:4
+  } else {
+    x = dpp_add<0x141>(x);  // row_half_mirror
+  }
+  x = dpp_add<0x4E>(x);  // quad_perm [2,3,0,1]
+  x = dpp_add<0xB1>(x);  // quad_perm [1,0,3,2]
+  return x;
+}
+
+constexpr float kNegBig = -1.0e30f;  // running maximum before the first key (finite: no inf - inf)
+constexpr float kRescaleSlack = 8.0f;  // the running maximum moves only when a logit exceeds it by this
+
 template <int D, int G, bool U8>
 __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p) {
-  constexpr int KPB = 8192 / G;   // keys per block held in LDS
-  constexpr int LPR = D / 8;      // lanes per V row
-  constexpr int KPI = 64 / LPR;   // V rows per load instruction of a wavefront
-  constexpr int KS = D / 32;      // MFMA k-steps per key group
-  __shared__ float lg[KPB * G];          // logits [key][head], log2 units
-  __shared__ uint32_t pp[(KPB / 2) * G]; // bf16 pairs (p[key A], p[key B]) [pair][head]
-  __shared__ float smx[WAVES][G];        // per-wavefront maxima, later per-wavefront sums
+  constexpr int LPR = D / 8;     // lanes per row: a lane owns 8 consecutive d
+  constexpr int RPI = 64 / LPR;  // rows per load instruction of a wavefront
+  constexpr int U = 4;           // load instructions per step and tensor (even: rows pair up for dot2)
+  constexpr int CH = U * RPI;    // keys per wavefront and step, contiguous
+  constexpr int LGK = 8192 / G;  // keys whose logits are gathered in LDS before they go out in one burst
+  __shared__ __align__(16) float lgbuf[LGK * G];  // [key][head]
+  __shared__ float red[WAVES][G][D];
+  __shared__ float rml[WAVES][G][2];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int kk = lane / LPR, dc = lane % LPR;
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int k_begin = split * p.keys_per_split;
   const int k_end = min(k_begin + p.keys_per_split, p.kv_len);
 
-  // B operand: column nn = query head (zero beyond G), d = 32 j + 8 hq .. +8
-  const int nn = lane & 15, hq = lane >> 4;
-  bf16x8_t qf[KS];
+  uint32_t qv[G][4];  // bf16 pairs of q[head][8 dc .. 8 dc + 8]
 #pragma unroll
-  for (int j = 0; j < KS; ++j) {
-    u32x4_t t = {0, 0, 0, 0};
-    if (nn < G) t = *(const u32x4_t*)(p.q + b * p.q_sb + (int64_t)(kvh * G + nn) * p.q_sh + 32 * j + 8 * hq);
-    qf[j] = as_bf16x8(t);
+  for (int g = 0; g < G; ++g) {
+    const u32x4_t t = *(const u32x4_t*)(p.q + b * p.q_sb + (int64_t)(kvh * G + g) * p.q_sh + 8 * dc);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qv[g][e] = t[e];
   }
-
-  const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * (U8 ? 1 : 2);
-  const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * (U8 ? 1 : 2);
+  // Rows are addressed as a uniform base plus a 32-bit byte offset (the host checks the range).
+  constexpr int ES = U8 ? 1 : 2;
+  const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
+  const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * ES;
+  const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES, lane_off = 8 * dc * ES;
   const int64_t qs_off = b * p.qs_sb + kvh * p.qs_sh;
+  float* lgrow = p.logits ? p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G : nullptr;
+  int lg_base = k_begin;  // first key of the logits gathered in LDS
 
-  float acc[G][8];
+  // State of this lane's row group (rows kk, kk + RPI, ... of every chunk): identical in its lanes.
+  float acc[G][8], m_run[G], l_run[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g)
+  for (int g = 0; g < G; ++g) {
+    m_run[g] = kNegBig;
+    l_run[g] = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
-  float m_run[G], l_run[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m_run[g] = -INFINITY;
-    l_run[g] = 0.0f;
   }
 
-  for (int blk0 = k_begin; blk0 < k_end; blk0 += KPB) {
-    const int nk = min(KPB, k_end - blk0);
-    const int ngroups = (nk + 15) / 16;
-    // ---- phase 1: logits ----------------------------------------------------------------
-    float mloc = -INFINITY;  // lanes with nn < G: max over their keys for head nn
-    for (int gi = wave; gi < ngroups; gi += WAVES) {
-      const int key = blk0 + gi * 16 + nn;  // A operand row of this lane
-      const bool ok = key < k_end;
-      f32x4_t s = {0, 0, 0, 0};
+  struct Rows {
+    u32x4_t k[U], v[U];
+    float ks[U], vs[U];
+    int32_t kz[U], vz[U];
+  };
+  // Rows past the end re-read the last valid row; their logits become -inf below.
+  auto issue = [&](Rows& r, int chunk0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = min(chunk0 + u * RPI + kk, k_end - 1);
       if constexpr (!U8) {
-        const uint16_t* kp = (const uint16_t*)kbase + (int64_t)key * p.k_st + 8 * hq;
-        u32x4_t kr[KS];
-#pragma unroll
-        for (int j = 0; j < KS; ++j) kr[j] = ok ? *(const u32x4_t*)(kp + 32 * j) : u32x4_t{0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < KS; ++j) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kr[j]), qf[j], s, 0, 0, 0);
+        r.k[u] = __builtin_nontemporal_load((const u32x4_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
       } else {
-        const uint8_t* kp = kbase + (int64_t)key * p.k_st + 8 * hq;
-        u32x2_t kr[KS];
-#pragma unroll
-        for (int j = 0; j < KS; ++j) kr[j] = ok ? *(const u32x2_t*)(kp + 32 * j) : u32x2_t{0, 0};
-        const float sc = ok ? p.k_scale[qs_off + key] : 0.0f;
-        const int32_t zp = ok ? p.k_zp[qs_off + key] : 0;
-#pragma unroll
-        for (int j = 0; j < KS; ++j)
-          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dq8(kr[j][0], kr[j][1], zp, sc)), qf[j], s, 0, 0, 0);
-      }
-      // accumulator: column nn = head, rows 4 hq + i = keys of the group
-      if (nn < G) {
-        const int kl = gi * 16 + 4 * hq;  // local key of row i = 0
-        f32x4_t t;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          t[i] = (blk0 + kl + i < k_end) ? s[i] * p.c : -INFINITY;
-          mloc = fmaxf(mloc, t[i]);
-          lg[(kl + i) * G + nn] = t[i];
-        }
-        if (p.logits) *(f32x4_t*)(p.logits + ((int64_t)b * p.Hq + kvh * G + nn) * p.Tpad + blk0 + kl) = t;
+        const u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
+        r.k[u] = u32x4_t{c[0], c[1], 0, 0};
+        r.ks[u] = p.k_scale[qs_off + key];
+        r.kz[u] = p.k_zp[qs_off + key];
       }
     }
-    // keys of the last, partial pair group that phase 1 did not touch
-    for (int i = ngroups * 16 * G + tid; i < ((nk + 2 * KPI - 1) / (2 * KPI)) * (2 * KPI) * G; i += NTHREADS) lg[i] = -INFINITY;
-    // block maximum per head
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-    if (lane < G) smx[wave][lane] = mloc;
-    __syncthreads();
-    float m_new[G], alpha[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float mb = smx[0][g];
-#pragma unroll
-      for (int w = 1; w < WAVES; ++w) mb = fmaxf(mb, smx[w][g]);
-      m_new[g] = fmaxf(m_run[g], mb);  // finite: every block holds at least one key
-      alpha[g] = fast_exp2(m_run[g] - m_new[g]);
+    for (int u = 0; u < U; ++u) {
+      const int key = min(chunk0 + u * RPI + kk, k_end - 1);
+      if constexpr (!U8) {
+        r.v[u] = __builtin_nontemporal_load((const u32x4_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
+      } else {
+        const u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
+        r.v[u] = u32x4_t{c[0], c[1], 0, 0};
+        r.vs[u] = p.v_scale[qs_off + key];
+        r.vz[u] = p.v_zp[qs_off + key];
+      }
     }
-    // ---- phase 2: p = exp2(logit - max) as bf16 pairs (key, key + KPI) ---------------------
-    const int npairs = ((nk + 2 * KPI - 1) / (2 * KPI)) * KPI;
-    float lsum[G];
+  };
+  auto consume = [&](Rows& r, int chunk0) {
+    // logits (log2 units) of the U rows of this lane's group, all G heads
+    float s[U][G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) lsum[g] = 0.0f;
-    for (int pi = tid; pi < npairs; pi += NTHREADS) {
-      const int ka = (pi / KPI) * (2 * KPI) + (pi % KPI);
-      const int kb = ka + KPI;
+    for (int u = 0; u < U; ++u) {
+      u32x4_t kx = r.k[u];
+      if constexpr (U8) kx = dq8(kx[0], kx[1], r.kz[u], r.ks[u]);
+      const bool valid = chunk0 + u * RPI + kk < k_end;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const float pa = fast_exp2(lg[ka * G + g] - m_new[g]);
-        const float pb = fast_exp2(lg[kb * G + g] - m_new[g]);
-        lsum[g] += pa + pb;
-        pp[pi * G + g] = pack_bf16(pa, pb);
+        float a = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t kw = kx[e];  // a bit_cast applied to the vector element itself reads element 0
+          a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, kw), __builtin_bit_cast(bf16x2_t, qv[g][e]), a, false);
+        }
+        a = row_group_sum<LPR>(a) * p.c;
+        s[u][g] = valid ? a : -INFINITY;
       }
     }
-    __syncthreads();  // smx consumed, pp complete
-    // ---- phase 3: O += p V ------------------------------------------------------------------
+    if (lgrow && dc == 0 && chunk0 < k_end) {
+      float* dst = lgbuf + (chunk0 - lg_base + kk) * G;
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] *= alpha[g];
-    const int kk = lane / LPR, dc = lane % LPR;
-    const int niter = npairs / KPI;  // each iteration of a wavefront covers 2 KPI keys
-    for (int it = wave; it < niter; it += WAVES) {
-      const int ka = blk0 + it * 2 * KPI + kk;
-      const int kb = ka + KPI;
-      u32x4_t va, vb;
-      if constexpr (!U8) {
-        va = ka < k_end ? *(const u32x4_t*)((const uint16_t*)vbase + (int64_t)ka * p.v_st + 8 * dc) : u32x4_t{0, 0, 0, 0};
-        vb = kb < k_end ? *(const u32x4_t*)((const uint16_t*)vbase + (int64_t)kb * p.v_st + 8 * dc) : u32x4_t{0, 0, 0, 0};
-      } else {
-        const u32x2_t ca = ka < k_end ? *(const u32x2_t*)(vbase + (int64_t)ka * p.v_st + 8 * dc) : u32x2_t{0, 0};
-        const u32x2_t cb = kb < k_end ? *(const u32x2_t*)(vbase + (int64_t)kb * p.v_st + 8 * dc) : u32x2_t{0, 0};
-        va = dq8(ca[0], ca[1], ka < k_end ? p.v_zp[qs_off + ka] : 0, ka < k_end ? p.v_scale[qs_off + ka] : 0.0f);
-        vb = dq8(cb[0], cb[1], kb < k_end ? p.v_zp[qs_off + kb] : 0, kb < k_end ? p.v_scale[qs_off + kb] : 0.0f);
+        for (int g = 0; g < G; ++g) dst[u * RPI * G + g] = s[u][g];
+    }
+    // running maximum: moved only when some logit of the wavefront exceeds it by the slack
+    float smax[G];
+    bool need = false;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mx = s[0][g];
+#pragma unroll
+      for (int u = 1; u < U; ++u) mx = fmaxf(mx, s[u][g]);
+      smax[g] = mx;
+      need |= mx > m_run[g] + kRescaleSlack;
+    }
+    if (__any(need)) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float mn = fmaxf(m_run[g], smax[g]);
+        const float al = fast_exp2(m_run[g] - mn);
+        m_run[g] = mn;
+        l_run[g] *= al;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] *= al;
       }
-      uint32_t pr[G];
+    }
+    // O += p V, two rows per dot2
 #pragma unroll
-      for (int g = 0; g < G; ++g) pr[g] = pp[(it * KPI + kk) * G + g];
+    for (int u = 0; u < U; u += 2) {
+      u32x4_t xa = r.v[u], xb = r.v[u + 1];
+      if constexpr (U8) {
+        xa = dq8(xa[0], xa[1], r.vz[u], r.vs[u]);
+        xb = dq8(xb[0], xb[1], r.vz[u + 1], r.vs[u + 1]);
+      }
+      bf16x2_t pg[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float pa = fast_exp2(s[u][g] - m_run[g]);
+        const float pb = fast_exp2(s[u + 1][g] - m_run[g]);
+        l_run[g] += pa + pb;
+        pg[g] = __builtin_bit_cast(bf16x2_t, pack_bf16(pa, pb));
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bf16x2_t lo = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(vb[e], va[e], 0x05040100u));
-        const bf16x2_t hi = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(vb[e], va[e], 0x07060302u));
+        const bf16x2_t lo = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(xb[e], xa[e], 0x05040100u));
+        const bf16x2_t hi = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(xb[e], xa[e], 0x07060302u));
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-          const bf16x2_t pg = __builtin_bit_cast(bf16x2_t, pr[g]);
-          acc[g][2 * e] = __builtin_amdgcn_fdot2_f32_bf16(lo, pg, acc[g][2 * e], false);
-          acc[g][2 * e + 1] = __builtin_amdgcn_fdot2_f32_bf16(hi, pg, acc[g][2 * e + 1], false);
+          acc[g][2 * e] = __builtin_amdgcn_fdot2_f32_bf16(lo, pg[g], acc[g][2 * e], false);
+          acc[g][2 * e + 1] = __builtin_amdgcn_fdot2_f32_bf16(hi, pg[g], acc[g][2 * e + 1], false);
         }
       }
     }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      l_run[g] = l_run[g] * alpha[g] + lsum[g];  // per-thread share of the sum
-      m_run[g] = m_new[g];
+  };
+
+  // Two steps in flight per wavefront: the loads of step i + 1 are issued before step i is consumed.
+  const int nsteps = (k_end - k_begin + CH * WAVES - 1) / (CH * WAVES);
+  const int stride = CH * WAVES;
+  int chunk = k_begin + wave * CH;
+  constexpr int FLUSH_STEPS = LGK / (CH * WAVES);
+  static_assert(FLUSH_STEPS >= 2 && FLUSH_STEPS % 2 == 0, "the loop below advances two steps at a time");
+  Rows ra, rb;
+  issue(ra, chunk);
+  for (int i = 0; i < nsteps; i += 2) {
+    issue(rb, chunk + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(ra, chunk);
+    __builtin_amdgcn_sched_barrier(0);  // the loads below reuse the registers consumed above
+    issue(ra, chunk + 2 * stride);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(rb, chunk + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    chunk += 2 * stride;
+    if (lgrow && ((i + 2) % FLUSH_STEPS == 0 || i + 2 >= nsteps)) {
+      // the gathered logits leave as one contiguous burst (keys past the end of a chunk are -inf)
+      __syncthreads();
+      const int nkeys = min(LGK, (k_end - lg_base + CH - 1) / CH * CH);
+      f32x4_t* dst = (f32x4_t*)(lgrow + (int64_t)lg_base * G);
+      for (int j = tid; j < nkeys * G / 4; j += NTHREADS) {
+        dst[j] = ((const f32x4_t*)lgbuf)[j];
+      }
+      lg_base += LGK;
+      __syncthreads();
     }
-    __syncthreads();  // lg / pp are rewritten by the next block
   }
 
-  // ---- reduce the partial O over the lanes that share a d chunk, then over wavefronts ---------
+  // ---- merge the RPI row groups of the wavefront, then the wavefronts, into one partial -----------
 #pragma unroll
   for (int g = 0; g < G; ++g) {
+    float M = m_run[g];
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+    const float sc = fast_exp2(m_run[g] - M);
+    float l = l_run[g] * sc;
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      float x = acc[g][e];
+      float x = acc[g][e] * sc;
 #pragma unroll
       for (int off = LPR; off < 64; off <<= 1) x += __shfl_xor(x, off, 64);
-      acc[g][e] = x;
+      if (lane < LPR) red[wave][g][lane * 8 + e] = x;
     }
-    float s = l_run[g];
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
-    l_run[g] = s;
-  }
-  // lg is free now (the loop ended with a barrier): reuse it as red[wave][head][d]
-  float* red = lg;
-  if (lane < LPR) {
-#pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) red[(wave * G + g) * D + lane * 8 + e] = acc[g][e];
-  }
-  if (lane == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) smx[wave][g] = l_run[g];
+    if (lane == 0) {
+      rml[wave][g][0] = M;
+      rml[wave][g][1] = l;
+    }
   }
   __syncthreads();
   for (int i = tid; i < G * D; i += NTHREADS) {
     const int g = i / D, d = i % D;
-    float x = 0.0f;
+    float M = rml[0][g][0];
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) x += red[(w * G + g) * D + d];
-    p.part_o[(((int64_t)b * p.Hq + kvh * G + g) * p.num_splits + split) * D + d] = x;
-  }
-  if (tid == 0) {
+    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, rml[w][g][0]);
+    float x = 0.0f, l = 0.0f;
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float s = 0.0f;
-#pragma unroll
-      for (int w = 0; w < WAVES; ++w) s += smx[w][g];
-      const int64_t o = (((int64_t)b * p.Hq + kvh * G + g) * p.num_splits + split) * 2;
-      p.part_ml[o] = m_run[g];
-      p.part_ml[o + 1] = s;
+    for (int w = 0; w < WAVES; ++w) {
+      const float sc = fast_exp2(rml[w][g][0] - M);
+      x += red[w][g][d] * sc;
+      l += rml[w][g][1] * sc;
+    }
+    const int64_t o = ((int64_t)b * p.Hq + kvh * G + g) * p.num_splits + split;
+    p.part_o[o * D + d] = x;
+    if (d == 0) {
+      p.part_ml[o * 2] = M;
+      p.part_ml[o * 2 + 1] = l;
     }
   }
 }
 
-// One workgroup of D threads per (b, query head): combine the splits.
+// Combine the splits of one (b, query head): 4 groups of D threads each take a quarter of the
+// splits, then the groups are added through LDS. Also produces the base-2 log-sum-exp.
 template <int D>
-__global__ void decode_merge_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams p) {
+  __shared__ float red[4][D + 1];
+  __shared__ float sM;
   const int bh = blockIdx.x;
   const int b = bh / p.Hq, hqi = bh % p.Hq;
-  const int d = threadIdx.x;
+  const int d = threadIdx.x % D, grp = threadIdx.x / D;
   const float* ml = p.part_ml + (int64_t)bh * p.num_splits * 2;
-  float M = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, ml[2 * s]);
+  if (threadIdx.x < 64) {
+    float mloc = -INFINITY;
+    for (int s = threadIdx.x; s < p.num_splits; s += 64) mloc = fmaxf(mloc, ml[2 * s]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, off, 64));
+    if (threadIdx.x == 0) sM = mloc;
+  }
+  __syncthreads();
+  const float M = sM;
   float L = 0.0f, acc = 0.0f;
-  for (int s = 0; s < p.num_splits; ++s) {
+  for (int s = grp; s < p.num_splits; s += 4) {
     const float w = fast_exp2(ml[2 * s] - M);
     L += ml[2 * s + 1] * w;
     acc += p.part_o[((int64_t)bh * p.num_splits + s) * D + d] * w;
   }
-  const float r = acc / L;
-  const float other = __shfl_xor(r, 1, 64);
-  if ((d & 1) == 0) *(uint32_t*)(p.o + b * p.o_sb + hqi * p.o_sh + d) = pack_bf16(r, other);
-  if (d == 0) {
-    const float lse = M + fast_log2(L);
-    p.lse_ws[bh] = lse;
-    if (p.lse_out) p.lse_out[bh] = lse;
+  red[grp][d] = acc;
+  if (d == 0) red[grp][D] = L;
+  __syncthreads();
+  if (grp == 0) {
+    const float a4 = red[0][d] + red[1][d] + red[2][d] + red[3][d];
+    const float l4 = red[0][D] + red[1][D] + red[2][D] + red[3][D];
+    const float r = a4 / l4;
+    const float other = __shfl_xor(r, 1, 64);
+    if ((d & 1) == 0) *(uint32_t*)(p.o + b * p.o_sb + hqi * p.o_sh + d) = pack_bf16(r, other);
+    if (d == 0) {
+      const float lse = M + fast_log2(l4);
+      p.lse_ws[bh] = lse;
+      if (p.lse_out) p.lse_out[bh] = lse;
+    }
   }
 }
 
-// W[b, kvh, k] = (1/G) sum_g exp2(logit[b, kvh*G+g, k] - lse[b, kvh*G+g]); 4 keys per lane.
-template <int G>
-__global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams p) {
+// Monotone map float -> uint32 (a < b  <=>  key(a) < key(b)); -0.0 is folded onto +0.0.
+__device__ __forceinline__ uint32_t ordered_bits(float x) {
+  x += 0.0f;
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// W[b, kvh, k] = (1/G) sum_g exp2(logit[b, kvh, k, g] - lse[b, kvh*G+g]); one key per lane and pass,
+// 4096 keys per workgroup. With H2O set it also does the cache's score update and eviction choice
+// in the same pass (keys_values/kvcache/h2o.py:175-196, keys_values/kvcache/attn_weights.py:773-774
+// for one slot): scores += W, then the (value, slot) minimum of the row through an integer atomicMin.
+template <int G, bool H2O>
+__global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams p, const kvx_h2o_args hh, unsigned long long* best) {
+  typedef float fG __attribute__((ext_vector_type(G >= 4 ? 4 : (G == 2 ? 2 : 1))));
+  constexpr int NV = G >= 4 ? G / 4 : 1;
   const int kvh = blockIdx.y, b = blockIdx.z;
-  const int k0 = (blockIdx.x * 256 + threadIdx.x) * 4;
-  if (k0 >= p.kv_len) return;
-  f32x4_t acc = {0, 0, 0, 0};
+  float lse[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const int64_t bh = (int64_t)b * p.Hq + kvh * G + g;
-    const float lse = p.lse_ws[bh];
-    const f32x4_t t = *(const f32x4_t*)(p.logits + bh * p.Tpad + k0);
+  for (int g = 0; g < G; ++g) lse[g] = p.lse_ws[(int64_t)b * p.Hq + kvh * G + g];
+  const float* lgrow = p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G;
+  float* wr = p.w ? p.w + ((int64_t)b * p.Hkv + kvh) * p.kv_len : nullptr;
+  float* sc = H2O ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
+  const int32_t* tpr = (H2O && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
+  unsigned long long mine = ~0ull;
+  constexpr int PASSES = 16;
+  fG t[PASSES][NV];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] += fast_exp2(t[e] - lse);
+  for (int it = 0; it < PASSES; ++it) {
+    const int k = min(blockIdx.x * 4096 + it * 256 + (int)threadIdx.x, p.Tpad - 1);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) t[it][j] = *((const fG*)(lgrow + (int64_t)k * G) + j);
   }
-  acc *= 1.0f / (float)G;
-  float* wr = p.w + ((int64_t)b * p.Hkv + kvh) * p.kv_len;
-  if (k0 + 3 < p.kv_len && (p.kv_len & 3) == 0) {
-    *(f32x4_t*)(wr + k0) = acc;
-  } else {
-    for (int e = 0; e < 4 && k0 + e < p.kv_len; ++e) wr[k0 + e] = acc[e];
+#pragma unroll
+  for (int it = 0; it < PASSES; ++it) {
+    const int k = blockIdx.x * 4096 + it * 256 + threadIdx.x;
+    if (k >= p.kv_len) break;
+    float acc = 0.0f;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float x;
+      if constexpr (G >= 4) x = t[it][g / 4][g % 4];
+      else if constexpr (G == 2) x = t[it][0][g];
+      else x = t[it][0][0];
+      acc += fast_exp2(x - lse[g]);
+    }
+    acc *= 1.0f / (float)G;
+    if (wr) wr[k] = acc;
+    if constexpr (H2O) {
+      float val = sc[k] + acc;
+      sc[k] = val;
+      if (k < hh.limit) {
+        if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
+        const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
+        mine = key < mine ? key : mine;
+      }
+    }
   }
+  if constexpr (H2O) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const unsigned long long o = __shfl_xor(mine, off, 64);
+      mine = o < mine ? o : mine;
+    }
+    __shared__ unsigned long long wbest[4];
+    if ((threadIdx.x & 63) == 0) wbest[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long mn = wbest[0];
+      for (int i = 1; i < 4; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
+      if (mn != ~0ull) atomicMin(best + b * p.Hkv + kvh, mn);
+    }
+  }
+}
+
+__global__ void decode_argmin_init_kernel(unsigned long long* best, int rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) best[i] = ~0ull;
+}
+__global__ void decode_argmin_finish_kernel(const unsigned long long* best, int32_t* next_index, int rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) next_index[i] = (int32_t)(best[i] & 0xffffffffull);
 }
 
 struct Plan {
-  int G, kpb, num_splits, keys_per_split, Tpad;
+  int G, num_splits, keys_per_split, Tpad;
   size_t off_logits, off_part_o, off_part_ml, off_lse, total;
 };
 
-Plan make_plan(const kvx_sdpa_args& a) {
+Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
   pl.G = a.Hq / a.Hkv;
-  pl.kpb = 8192 / pl.G;
-  int splits = a.num_splits > 0 ? a.num_splits : (a.kv_len + pl.kpb - 1) / pl.kpb;
+  // About 16 workgroups per compute unit over the whole grid, each with at least 1024 keys.
+  int splits = a.num_splits;
+  if (splits <= 0) {
+    const int rows = a.B * a.Hkv;
+    splits = (16 * num_cus() + rows - 1) / rows;
+    splits = min(splits, (a.kv_len + 1023) / 1024);
+  }
   splits = max(1, min(splits, 512));
   int kps = (a.kv_len + splits - 1) / splits;
-  kps = ((kps + 63) / 64) * 64;  // keeps the 16-byte logits stores aligned
+  kps = ((kps + 63) / 64) * 64;  // keeps the chunks of a split aligned to the logits rows
   pl.keys_per_split = kps;
   pl.num_splits = (a.kv_len + kps - 1) / kps;
   pl.Tpad = ((a.kv_len + 63) / 64) * 64;
   size_t off = 0;
   pl.off_logits = off;
-  off += a.w ? (size_t)a.B * a.Hq * pl.Tpad * 4 : 0;
+  off += (a.w || fused_h2o) ? (size_t)a.B * a.Hq * pl.Tpad * 4 : 0;
   pl.off_part_o = off;
   off += (size_t)a.B * a.Hq * pl.num_splits * a.D * 4;
   pl.off_part_ml = off;
@@ -340,39 +468,56 @@ Plan make_plan(const kvx_sdpa_args& a) {
 }
 
 template <int D, int G>
-int launch_dg(const DecodeParams& p, bool u8, hipStream_t st) {
+int launch_dg(const DecodeParams& p, bool u8, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
+  unsigned long long* best = hh ? (unsigned long long*)hh->workspace : nullptr;
+  const int rows = p.B * p.Hkv;
+  if (hh) {
+    hipLaunchKernelGGL(decode_argmin_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, rows);
+    KVX_HIP(hipGetLastError());
+  }
   if (u8) hipLaunchKernelGGL((decode_split_kernel<D, G, true>), grid, dim3(NTHREADS), 0, st, p);
   else hipLaunchKernelGGL((decode_split_kernel<D, G, false>), grid, dim3(NTHREADS), 0, st, p);
   KVX_HIP(hipGetLastError());
-  hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(p.B * p.Hq), dim3(D), 0, st, p);
+  hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
   KVX_HIP(hipGetLastError());
-  if (p.w) {
-    hipLaunchKernelGGL((decode_weights_kernel<G>), dim3((p.kv_len + 1023) / 1024, p.Hkv, p.B), dim3(256), 0, st, p);
+  const dim3 wgrid((p.kv_len + 4095) / 4096, p.Hkv, p.B);
+  if (hh) {
+    hipLaunchKernelGGL((decode_weights_kernel<G, true>), wgrid, dim3(256), 0, st, p, *hh, best);
+    KVX_HIP(hipGetLastError());
+    hipLaunchKernelGGL(decode_argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, hh->next_index, rows);
+    KVX_HIP(hipGetLastError());
+  } else if (p.w) {
+    kvx_h2o_args none = {};
+    hipLaunchKernelGGL((decode_weights_kernel<G, false>), wgrid, dim3(256), 0, st, p, none, best);
     KVX_HIP(hipGetLastError());
   }
   return KVX_OK;
 }
 
 template <int D>
-int launch_d(const DecodeParams& p, int G, bool u8, hipStream_t st) {
+int launch_d(const DecodeParams& p, int G, bool u8, const kvx_h2o_args* hh, hipStream_t st) {
   switch (G) {
-    case 1: return launch_dg<D, 1>(p, u8, st);
-    case 2: return launch_dg<D, 2>(p, u8, st);
-    case 4: return launch_dg<D, 4>(p, u8, st);
-    case 8: return launch_dg<D, 8>(p, u8, st);
+    case 1: return launch_dg<D, 1>(p, u8, hh, st);
+    case 2: return launch_dg<D, 2>(p, u8, hh, st);
+    case 4: return launch_dg<D, 4>(p, u8, hh, st);
+    case 8: return launch_dg<D, 8>(p, u8, hh, st);
   }
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in {1, 2, 4, 8}", G);
 }
 
 }  // namespace
 
-size_t sdpa_decode_workspace(const kvx_sdpa_args& a) { return make_plan(a).total; }
+size_t sdpa_decode_workspace(const kvx_sdpa_args& a, bool fused_h2o) { return make_plan(a, fused_h2o).total; }
 
-int launch_sdpa_decode(const kvx_sdpa_args& a, hipStream_t st) {
-  const Plan pl = make_plan(a);
+int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream_t st) {
+  const Plan pl = make_plan(a, hh != nullptr);
   KVX_REQUIRE(a.workspace && a.workspace_bytes >= pl.total, KVX_ERR_WORKSPACE,
               "kvx_sdpa_decode: workspace of %zu bytes needed, %zu given", pl.total, a.workspace_bytes);
+  const int64_t es = a.kv_dtype == KVX_KV_U8 ? 1 : 2;
+  KVX_REQUIRE((int64_t)a.kv_len * a.k_stride_t * es < (1ll << 32) && (int64_t)a.kv_len * a.v_stride_t * es < (1ll << 32), KVX_ERR_UNSUPPORTED,
+              "kvx_sdpa_decode: one (batch, head) row set of K or V must span less than 4 GiB (kv_len %d, slot strides %lld / %lld)",
+              a.kv_len, (long long)a.k_stride_t, (long long)a.v_stride_t);
   DecodeParams p;
   char* ws = (char*)a.workspace;
   p.q = (const uint16_t*)a.q;
@@ -382,7 +527,7 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, hipStream_t st) {
   p.o = (uint16_t*)a.o;
   p.lse_out = a.lse;
   p.w = a.w;
-  p.logits = a.w ? (float*)(ws + pl.off_logits) : nullptr;
+  p.logits = (a.w || hh) ? (float*)(ws + pl.off_logits) : nullptr;
   p.part_o = (float*)(ws + pl.off_part_o);
   p.part_ml = (float*)(ws + pl.off_part_ml);
   p.lse_ws = (float*)(ws + pl.off_lse);
@@ -395,8 +540,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, hipStream_t st) {
   p.o_sb = a.o_stride_b; p.o_sh = a.o_stride_h;
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   const bool u8 = a.kv_dtype == KVX_KV_U8;
-  if (a.D == 128) return launch_d<128>(p, pl.G, u8, st);
-  if (a.D == 64) return launch_d<64>(p, pl.G, u8, st);
+  if (a.D == 128) return launch_d<128>(p, pl.G, u8, hh, st);
+  if (a.D == 64) return launch_d<64>(p, pl.G, u8, hh, st);
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128}", a.D);
 }
 

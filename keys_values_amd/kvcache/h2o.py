@@ -189,6 +189,10 @@ class H2OKVCache:
         kc, vc = self.k[:b, :, :T], self.v[:b, :, :T]
         tp = self.token_pos[:b, :, :T]
         quant = self._quant_state(T)
+        if num == 1 and T == self.cache_length:
+            # one token into a full cache: attention, score update and eviction choice in one call
+            out = self._decode_h2o_step(query, kc, vc, quant).unsqueeze(1)
+            return out.reshape(b, num, hq * d)
         if num == 1:
             out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
             out = out.unsqueeze(1)
@@ -254,6 +258,48 @@ class H2OKVCache:
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
 
+    def _h2o_args(self, full: bool) -> _lib.H2OArgs:
+        a = _lib.H2OArgs()
+        a.B, a.Hkv, a.kv_len = self.batch_size, self.n_query_groups, self.current_length
+        a.limit = self.current_length
+        a.k = self._select_k if full else 1
+        a.normalize = int(self.normalize_scores and full)
+        a.input_pos = self._input_pos
+        a.prefill_len = self.prefill_length
+        a.scores = self.scores.data_ptr()
+        a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
+        a.token_pos = self.token_pos.data_ptr()
+        a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
+        return a
+
+    def _decode_h2o_step(self, query, kc, vc, quant) -> torch.Tensor:
+        """``self.mha(...)`` and ``self._update(...)`` of keys_values/kvcache/base.py:583-595 for one new
+        token and a full cache, as the single fused call ``kvx_sdpa_decode_h2o`` (selection size 1)."""
+        if self._select_k != 1:
+            out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
+            self._update(w, 1)
+            return out
+        b, hq, _, d = query.shape
+        dev = self.device
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            out = torch.empty((b, hq, d), dtype=query.dtype, device=dev)
+            o_view = out.unsqueeze(2)
+            a = _lib.SdpaArgs()
+            ops._fill_common(a, query, kc, vc, self.scale_factor, self.current_length - 1, None, quant, 0)
+            a.o = o_view.data_ptr()
+            a.o_stride_b, a.o_stride_h, a.o_stride_t = o_view.stride(0), o_view.stride(1), o_view.stride(2)
+            h = self._h2o_args(True)
+            h.next_index = self._next_index.data_ptr()
+            nb_a = lib.kvx_sdpa_decode_h2o_workspace_bytes(ctypes.byref(a))
+            nb_h = (lib.kvx_h2o_workspace_bytes(ctypes.byref(h)) + 255) // 256 * 256
+            ws = _lib.workspace(dev, nb_a + nb_h)
+            h.workspace, h.workspace_bytes = ws.data_ptr(), nb_h
+            a.workspace, a.workspace_bytes = ws.data_ptr() + nb_h, ws.numel() - nb_h
+            _lib.check(lib.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), _lib.stream_ptr(dev)))
+        self._have_next = True
+        return out
+
     def _update(self, attn_weights: torch.Tensor, query_length: int):
         """keys_values/kvcache/attn_weights.py:721-783 with keys_values/kvcache/h2o.py:146-199."""
         if not isinstance(attn_weights, torch.Tensor):
@@ -268,18 +314,8 @@ class H2OKVCache:
         _lib.require_gpu(attn_weights)
         attn_weights = attn_weights.contiguous()
         full = self.current_length == self.cache_length
-        a = _lib.H2OArgs()
-        a.B, a.Hkv, a.kv_len = self.batch_size, self.n_query_groups, self.current_length
-        a.limit = self.current_length
-        a.k = self._select_k if full else 1
-        a.normalize = int(self.normalize_scores and full)
-        a.input_pos = self._input_pos
-        a.prefill_len = self.prefill_length
-        a.scores = self.scores.data_ptr()
-        a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
+        a = self._h2o_args(full)
         a.w = attn_weights.data_ptr()
-        a.token_pos = self.token_pos.data_ptr()
-        a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
         lib = _lib.load()
         with torch.cuda.device(self.device):
             if full:
