@@ -11,6 +11,8 @@ Inputs are resident in HBM before the timed region.
 `--workload decode`  : single-token decode over a bf16 cache with score-sums, H2O score update and
                        argmin (batch 8, 32/8 heads, 131072 positions), GB/s against HBM peak.
 `--workload quantize`: affine uint8 row quantiser on (1, 8, 65536, 128) K and V, GB/s.
+`--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
+                       launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
 Prints ONE JSON line (see the keys below). `roofline` describes the dominant kernel, timed with
 events on the launch stream inside the timed steps; `cpu_baseline` times the CPU oracle (the
@@ -31,13 +33,22 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# HBM bytes per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (KiB per dispatch, one counter per run, on these same workloads), each scaled by what the counter
+# reads for the `calib` launch of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+TRAFFIC_BYTES = {
+    "prefill": int((76989.8 * 2.000 + 66560.0) * 1024),    # sdpa_prefill_kernel<128,false>
+    "decode": int((2099047.6 * 2.000 + 139780.2) * 1024),  # decode_split_kernel<128,4,false>
+    "quantize": int((65576.8 * 2.000 + 69635.2) * 1024),   # quantize_rows_kernel<128>
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize"])
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--splits", type=int, default=0)
     return ap.parse_args()
@@ -162,7 +173,7 @@ def bench_prefill(args, torch, dev):
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": TRAFFIC_BYTES["prefill"],
         },
         "cpu_baseline": cpu,
     }
@@ -219,7 +230,7 @@ def bench_quantize(args, torch, dev):
         "config": {"workload": "BASELINE.json configs[2] quantiser: K and V (1, 8, 65536, 128) bf16 -> uint8 + fp32 scale + int32 zero point, seed 2",
                    "bytes_algorithmic_per_tensor": bytes_alg},
         "roofline": {"bound": "hbm", "kernel": "quantize_rows_kernel<128>", "achieved": round(kgbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(kgbs / PEAK_HBM_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(kgbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["quantize"]},
         "cpu_baseline": cpu,
     }
 
@@ -259,16 +270,30 @@ def bench_decode(args, torch, dev):
     ms_gpu = e0.elapsed_time(e1) / args.steps
     bytes_alg = 2 * B * Hkv * L * D * 2 + 2 * B * Hkv * L * 4  # K + V once, scores read-modify-write
     gbs = bytes_alg / (ms_step * 1e-3) / 1e9
+    # the dominant launch alone: the fused attention + score update + argmin call (split attention,
+    # merge, weights kernels), events on the launch stream around each call
+    launch, _ = cache._decode_h2o_prepare(qs[0], cache.k, cache.v, None)
+    launch()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a0, a1 in evs:
+        a0.record()
+        launch()
+        a1.record()
+    torch.cuda.synchronize()
+    ms_call = sum(a0.elapsed_time(a1) for a0, a1 in evs) / args.steps
     cpu = None
     if not args.no_cpu_baseline:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
-        kc, vc = cache.k[:1, :2].cpu(), cache.v[:1, :2].cpu()
+        nb = 2  # batch rows 0-1 of 8, all KV heads: a quarter of one step's attention
+        kc, vc = cache.k[:nb].cpu(), cache.v[:nb].cpu()
+        qc = qs[0, :nb].cpu()
         t_c0 = time.perf_counter()
-        O.sdpa_in_blocks(qs[0, :1, :8].cpu(), kc, vc, D ** -0.5, L, None)
+        O.sdpa_in_blocks(qc, kc, vc, D ** -0.5, L, None)
         t_c = time.perf_counter() - t_c0
-        frac = (1 * 2) / (B * Hkv)
+        frac = nb / B
         cpu = {"value": round(bytes_alg * frac / t_c / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": f"attention part of one step for batch 0, KV heads 0-1 (1/32 of a step), {t_c:.1f} s"}
+               "sample": f"attention + score-sums of one step for batch rows 0-{nb - 1} of {B} ({frac:.2f} of a step), {t_c:.1f} s"}
     return {
         "metric": "decode + H2O step GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
@@ -276,11 +301,32 @@ def bench_decode(args, torch, dev):
         "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3",
                    "bytes_algorithmic_per_step": bytes_alg, "ms_per_step_gpu_events": round(ms_gpu, 4),
                    "decode_tokens_per_s": round(B / (ms_step * 1e-3), 1)},
-        "roofline": {"bound": "hbm", "kernel": "whole decode step (cache write, split attention, merge, weights, score update + argmin)",
-                     "achieved": round(bytes_alg / (ms_gpu * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(bytes_alg / (ms_gpu * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,false> + merge + weights/score update/argmin",
+                     "achieved": round(bytes_alg / (ms_call * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(bytes_alg / (ms_call * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "ms_per_launch": round(ms_call, 4),
+                     "traffic": TRAFFIC_BYTES["decode"]},
         "cpu_baseline": cpu,
     }
+
+
+def bench_calib(args, torch, dev):
+    n = 1 << 29  # bf16 elements: 1 GiB in, 1 GiB out
+    src = torch.ones(n, dtype=torch.bfloat16, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        torch.neg(src, out=dst)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        torch.neg(src, out=dst)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    return {"metric": "calibration copy GB/s", "value": round(2 * n * 2 / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "elementwise negate, 1 GiB read + 1 GiB written per launch", "bytes_read": 2 * n, "bytes_written": 2 * n}}
 
 
 def main():
@@ -296,7 +342,7 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode}[args.workload]
+    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "calib": bench_calib}[args.workload]
     res = fn(args, torch, dev)
     print(json.dumps(res), flush=True)
 

@@ -279,6 +279,14 @@ class H2OKVCache:
             out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
             self._update(w, 1)
             return out
+        launch, out = self._decode_h2o_prepare(query, kc, vc, quant)
+        launch()
+        self._have_next = True
+        return out
+
+    def _decode_h2o_prepare(self, query, kc, vc, quant):
+        """Argument blocks and workspace of one ``kvx_sdpa_decode_h2o`` call; returns the launcher (it
+        may be called repeatedly: every call is one more update of the scores) and the output."""
         b, hq, _, d = query.shape
         dev = self.device
         lib = _lib.load()
@@ -296,9 +304,14 @@ class H2OKVCache:
             ws = _lib.workspace(dev, nb_a + nb_h)
             h.workspace, h.workspace_bytes = ws.data_ptr(), nb_h
             a.workspace, a.workspace_bytes = ws.data_ptr() + nb_h, ws.numel() - nb_h
-            _lib.check(lib.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), _lib.stream_ptr(dev)))
-        self._have_next = True
-        return out
+            stream = _lib.stream_ptr(dev)
+
+        def launch():
+            with torch.cuda.device(dev):
+                _lib.check(lib.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), stream))
+
+        launch.keepalive = (query, kc, vc, quant, out, ws)
+        return launch, out
 
     def _update(self, attn_weights: torch.Tensor, query_length: int):
         """keys_values/kvcache/attn_weights.py:721-783 with keys_values/kvcache/h2o.py:146-199."""
