@@ -76,7 +76,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t*
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
-    raw[i] = r < rows ? *(const u32x4_t*)(x + r * x_row_stride + col * 8) : u32x4_t{0, 0, 0, 0};
+    raw[i] = r < rows ? __builtin_nontemporal_load((const u32x4_t*)(x + r * x_row_stride + col * 8)) : u32x4_t{0, 0, 0, 0};
   }
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {

@@ -326,3 +326,64 @@ def test_attention_over_uint8_cache(kvx, gpu):
     torch.cuda.synchronize()
     assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
     torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,D,limit,normalize,quantized", [
+    (2, 8, 2, 1000, 128, 1000, False, False),
+    (1, 4, 4, 777, 64, 700, True, False),
+    (2, 8, 1, 4096 + 33, 128, 4096, True, True),
+    (1, 2, 1, 17, 64, 17, False, True),
+])
+def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, B, Hq, Hkv, T, D, limit, normalize, quantized):
+    """kvx_sdpa_decode_h2o == kvx_sdpa_decode (with weights) followed by kvx_h2o_update_select(k=1),
+    and both match the oracle."""
+    q, k, v, _ = make_qkv(50 + T, B, Hq, Hkv, 1, T, D)
+    gen = torch.Generator().manual_seed(T)
+    scores = torch.rand(B, Hkv, T, generator=gen) * 2
+    tp = torch.stack([torch.randperm(3 * T, generator=gen)[:T] for _ in range(B * Hkv)]).view(B, Hkv, T).to(torch.int32)
+    input_pos, prefill_len = 3 * T + 5, T // 2
+    scale = 1.0 / math.sqrt(D)
+    quant = None
+    kg, vg = k.to(gpu), v.to(gpu)
+    if quantized:
+        kc, ks, kz = O.quantize_rows(k.reshape(-1, D))
+        vc, vs, vz = O.quantize_rows(v.reshape(-1, D))
+        k = O.dequantize_rows(kc, ks, kz).view(B, Hkv, T, D)
+        v = O.dequantize_rows(vc, vs, vz).view(B, Hkv, T, D)
+        kg, vg = kc.view(B, Hkv, T, D).to(gpu), vc.view(B, Hkv, T, D).to(gpu)
+        quant = ops.QuantState(ks.view(B, Hkv, T).to(gpu), kz.view(B, Hkv, T).to(gpu), vs.view(B, Hkv, T).to(gpu), vz.view(B, Hkv, T).to(gpu))
+    # separate calls
+    out_a, w_a, _ = ops.decode_core(q.to(gpu), kg, vg, scale, return_weights=True, quant=quant)
+    s_a, n_a = gpu_h2o(kvx, gpu, scores, w_a.cpu(), T, limit, 1, normalize, tp, input_pos, prefill_len)
+    # fused call
+    qg = q.to(gpu)
+    out_b = torch.empty((B, Hq, D), dtype=torch.bfloat16, device=gpu)
+    ov = out_b.unsqueeze(2)
+    sc_g, tp_g = scores.to(gpu), tp.to(gpu)
+    nxt = torch.full((B, Hkv, 1), -1, dtype=torch.int32, device=gpu)
+    a = _lib.SdpaArgs()
+    ops._fill_common(a, qg, kg, vg, scale, T - 1, None, quant, 0)
+    a.o, a.o_stride_b, a.o_stride_h, a.o_stride_t = ov.data_ptr(), ov.stride(0), ov.stride(1), ov.stride(2)
+    h = _lib.H2OArgs()
+    h.B, h.Hkv, h.kv_len, h.limit, h.k = B, Hkv, T, limit, 1
+    h.normalize, h.input_pos, h.prefill_len = int(normalize), input_pos, prefill_len
+    h.scores, h.sc_stride_b, h.sc_stride_h = sc_g.data_ptr(), sc_g.stride(0), sc_g.stride(1)
+    h.token_pos, h.tp_stride_b, h.tp_stride_h = tp_g.data_ptr(), tp_g.stride(0), tp_g.stride(1)
+    h.next_index = nxt.data_ptr()
+    nb_h = (kvx.kvx_h2o_workspace_bytes(ctypes.byref(h)) + 255) // 256 * 256
+    nb_a = kvx.kvx_sdpa_decode_h2o_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(nb_h + nb_a + 256, dtype=torch.uint8, device=gpu)
+    h.workspace, h.workspace_bytes = ws.data_ptr(), nb_h
+    a.workspace, a.workspace_bytes = ws.data_ptr() + nb_h, nb_a
+    _lib.check(kvx.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    assert torch.equal(out_b, out_a)
+    assert torch.equal(sc_g.cpu(), s_a)
+    assert torch.equal(nxt.cpu(), n_a)
+    # oracle
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, T - 1, None)
+    assert rel_err(out_b.float().cpu().unsqueeze(2), o_ref.float()) < 2e-2
+    s_ref = scores.clone()
+    n_ref = O.h2o_update_select(s_ref, w_ref, T, limit, 1, normalize=normalize, token_pos=tp, input_pos=input_pos, prefill_len=prefill_len)
+    torch.testing.assert_close(sc_g.cpu(), s_ref, rtol=1e-3, atol=1e-6)
+    _sets_equal_away_from_ties(nxt.cpu().long(), n_ref, (s_ref[..., :limit] / (input_pos - torch.maximum(tp, torch.tensor(prefill_len - 1)))[..., :limit].float()) if normalize else s_ref[..., :limit], 1)
