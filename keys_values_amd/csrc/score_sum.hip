@@ -11,6 +11,8 @@
 // double-buffered, shared by the four wavefronts of the workgroup (256 keys per workgroup).
 // S = Q K^T is computed with rows along M, so a lane owns one key column: the sum over queries is a
 // per-lane running sum and the two halves of the wavefront are added once at the end.
+#include <type_traits>
+
 #include "kvx_common.h"
 
 namespace kvx {
@@ -39,8 +41,8 @@ template <int D>
 struct alignas(16) Smem {
   static constexpr int QCH16 = D / 8 + 1;  // 16-byte chunks per row incl. pad (conflict-free ds_read_b128)
   u32x4_t q[2][BQ][QCH16];
-  float lse[2][BQ];
-  int32_t qpos[2][BQ];
+  float lse[3][BQ];   // read one phase later than q, hence one more buffer
+  int32_t qpos[3][BQ];
 };
 
 template <int D>
@@ -66,6 +68,8 @@ struct QLoader {
   int qi[QCH], g[QCH];    // row of chunk i in the current tile
   int lqi, lg;            // row of the lse / position this thread stages (tid < BQ)
   int dq, dg;             // BQ / G, BQ % G
+  const uint16_t* src[QCH];  // dg == 0: address of chunk i in the current tile
+  int64_t step;              // dg == 0: elements between consecutive tiles
 
   __device__ __forceinline__ void init(const ScoreParams& p, int b, int kvh, int tid) {
     col = tid % CPR;
@@ -80,24 +84,36 @@ struct QLoader {
       const int r = row_in + i * RPI;
       qi[i] = r / G;
       g[i] = r % G;
+      src[i] = qbase + (int64_t)g[i] * q_sh + (int64_t)qi[i] * q_st + col * 8;
     }
+    step = (int64_t)dq * q_st;
     lqi = tid / G;
     lg = tid % G;
   }
 
   // fetch the tile whose first row is row0, then step the row bookkeeping to the next tile
   __device__ __forceinline__ void fetch(QStage<D>& s, int row0, int tid) {
+    if (dg == 0) {
+      // G divides the tile height: every row keeps its head and moves by BQ / G queries per tile.
+      // Rows past the end read row 0 (finite data); their lse = +inf makes their weight zero.
 #pragma unroll
-    for (int i = 0; i < QCH; ++i) {
-      const bool ok = row0 + row_in + i * RPI < R;
-      const uint16_t* src = qbase + (int64_t)g[i] * q_sh + (int64_t)(ok ? qi[i] : 0) * q_st + col * 8;
-      const u32x4_t v = *(const u32x4_t*)(ok ? src : qbase);
-      s.qr[i] = ok ? v : u32x4_t{0, 0, 0, 0};
-      qi[i] += dq;
-      g[i] += dg;
-      if (g[i] >= G) {
-        g[i] -= G;
-        qi[i] += 1;
+      for (int i = 0; i < QCH; ++i) {
+        const bool ok = row0 + row_in + i * RPI < R;
+        s.qr[i] = *(const u32x4_t*)(ok ? src[i] : qbase);
+        src[i] += step;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < QCH; ++i) {
+        const bool ok = row0 + row_in + i * RPI < R;
+        const uint16_t* ptr = qbase + (int64_t)g[i] * q_sh + (int64_t)(ok ? qi[i] : 0) * q_st + col * 8;
+        s.qr[i] = *(const u32x4_t*)(ok ? ptr : qbase);
+        qi[i] += dq;
+        g[i] += dg;
+        if (g[i] >= G) {
+          g[i] -= G;
+          qi[i] += 1;
+        }
       }
     }
     if (tid < BQ) {
@@ -114,12 +130,12 @@ struct QLoader {
     }
   }
 
-  __device__ __forceinline__ void commit(const QStage<D>& s, Smem<D>& sm, int buf, int tid) const {
+  __device__ __forceinline__ void commit(const QStage<D>& s, Smem<D>& sm, int buf, int buf3, int tid) const {
 #pragma unroll
     for (int i = 0; i < QCH; ++i) sm.q[buf][row_in + i * RPI][col] = s.qr[i];
     if (tid < BQ) {
-      sm.lse[buf][tid] = s.lse;
-      sm.qpos[buf][tid] = s.qpos;
+      sm.lse[buf3][tid] = s.lse;
+      sm.qpos[buf3][tid] = s.qpos;
     }
   }
 };
@@ -173,70 +189,108 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
   int tpmax = max(tpk[0], tpk[1]);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) tpmax = max(tpmax, __shfl_xor(tpmax, off, 64));
+  tpmax = __builtin_amdgcn_readfirstlane(tpmax);
 
   float wacc[2] = {0.0f, 0.0f};
   const int num_qt = (p.R + BQ - 1) / BQ;
   QLoader<D> ld;
   ld.init(p, b, kvh, tid);
   QStage<D> st;
-  ld.fetch(st, 0, tid);
-  ld.commit(st, sm, 0, tid);
-  if (num_qt > 1) ld.fetch(st, BQ, tid);
-  __syncthreads();
 
-  for (int t = 0; t < num_qt; ++t) {
-    const int buf = t & 1;
-    const int qpos_tile_min = p.input_pos + (t * BQ) / p.G;
-    const bool need_mask = tpmax > qpos_tile_min;
+  // S block = 32 query rows x 64 keys: Q rows come from LDS (A operand), K sits in registers.
+  auto mfma_block = [&](f32x16_t (&s)[2], int buf, int mt) {
 #pragma unroll
-    for (int mt = 0; mt < BQ / 32; ++mt) {
-      f32x16_t s[2];
+    for (int j = 0; j < D / 16; ++j) {
+      const u32x4_t qq = sm.q[buf][mt * 32 + n][2 * j + h];
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
-#pragma unroll
-      for (int j = 0; j < D / 16; ++j) {
-        const u32x4_t qq = sm.q[buf][mt * 32 + n][2 * j + h];
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], s[nt], 0, 0, 0);
-      }
-      // rows of the accumulator: 8 a + 4 h + (0..3)
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const f32x4_t ls = *(const f32x4_t*)&sm.lse[buf][mt * 32 + 8 * a + 4 * h];
-        if (need_mask) {
-          const int4 qp = *(const int4*)&sm.qpos[buf][mt * 32 + 8 * a + 4 * h];
-#pragma unroll
-          for (int nt = 0; nt < 2; ++nt) {
-            float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
-            float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
-            float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
-            float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
-            e0 = tpk[nt] > qp.x ? 0.0f : e0;
-            e1 = tpk[nt] > qp.y ? 0.0f : e1;
-            e2 = tpk[nt] > qp.z ? 0.0f : e2;
-            e3 = tpk[nt] > qp.w ? 0.0f : e3;
-            wacc[nt] += (e0 + e1) + (e2 + e3);
-          }
+      for (int nt = 0; nt < 2; ++nt) {
+        if (j == 0) {
+          const f32x16_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], zero, 0, 0, 0);
         } else {
-#pragma unroll
-          for (int nt = 0; nt < 2; ++nt) {
-            const float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
-            const float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
-            const float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
-            const float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
-            wacc[nt] += (e0 + e1) + (e2 + e3);
-          }
+          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], s[nt], 0, 0, 0);
         }
       }
     }
-    if (t + 1 < num_qt) {
-      ld.commit(st, sm, buf ^ 1, tid);
+  };
+  // p = exp2(c S - lse) summed over the block's rows; accumulator rows are 8 a + 4 h + (0..3)
+  auto valu_block = [&](auto mask_tag, const f32x16_t (&s)[2], int buf3, int mt) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const f32x4_t ls = *(const f32x4_t*)&sm.lse[buf3][mt * 32 + 8 * a + 4 * h];
+      int4 qp = {0, 0, 0, 0};
+      if constexpr (MASK) qp = *(const int4*)&sm.qpos[buf3][mt * 32 + 8 * a + 4 * h];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
+        float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
+        float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
+        float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
+        if constexpr (MASK) {
+          e0 = tpk[nt] > qp.x ? 0.0f : e0;
+          e1 = tpk[nt] > qp.y ? 0.0f : e1;
+          e2 = tpk[nt] > qp.z ? 0.0f : e2;
+          e3 = tpk[nt] > qp.w ? 0.0f : e3;
+        }
+        wacc[nt] += (e0 + e1) + (e2 + e3);
+      }
+    }
+  };
+  // one matrix instruction, its share of the LDS reads, then its share of the other block's
+  // vector work (6 or 10 instructions per matrix instruction, 2 of them transcendental)
+  auto interleave = [&](auto mask_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+#pragma unroll
+    for (int i = 0; i < 2 * (D / 16); ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, MASK ? 8 * 16 / (2 * (D / 16)) : 4 * 16 / (2 * (D / 16)), 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2 * 16 / (2 * (D / 16)), 0);
+    }
+  };
+
+  ld.fetch(st, 0, tid);
+  ld.commit(st, sm, 0, 0, tid);
+  if (num_qt > 1) ld.fetch(st, BQ, tid);
+  __syncthreads();
+  f32x16_t sa[2], sb[2];  // blocks 0 and 1 of the current tile
+  mfma_block(sa, 0, 0);
+
+  // Software pipeline: the matrix work of one block runs under the vector work of the block before.
+  // Tile t + 1 is committed at the start of iteration t and first read after the barrier inside it.
+  for (int t = 0; t < num_qt; ++t) {
+    const int buf = t & 1, buf3 = t % 3;
+    const bool more = t + 1 < num_qt;
+    if (more) {
+      ld.commit(st, sm, buf ^ 1, (t + 1) % 3, tid);
       if (t + 2 < num_qt) ld.fetch(st, (t + 2) * BQ, tid);
     }
+    const bool need_mask = tpmax > p.input_pos + (t * BQ) / p.G;
+    if (need_mask) {
+      mfma_block(sb, buf, 1);
+      valu_block(std::true_type{}, sa, buf3, 0);
+      interleave(std::true_type{});
+    } else {
+      mfma_block(sb, buf, 1);
+      valu_block(std::false_type{}, sa, buf3, 0);
+      interleave(std::false_type{});
+    }
     __syncthreads();
+    if (more) {
+      if (need_mask) {
+        mfma_block(sa, buf ^ 1, 0);
+        valu_block(std::true_type{}, sb, buf3, 1);
+        interleave(std::true_type{});
+      } else {
+        mfma_block(sa, buf ^ 1, 0);
+        valu_block(std::false_type{}, sb, buf3, 1);
+        interleave(std::false_type{});
+      }
+    } else {
+      if (need_mask) valu_block(std::true_type{}, sb, buf3, 1);
+      else valu_block(std::false_type{}, sb, buf3, 1);
+    }
   }
 
 #pragma unroll
