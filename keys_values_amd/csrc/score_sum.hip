@@ -241,6 +241,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
   // vector work (6 or 10 instructions per matrix instruction, 2 of them transcendental)
   auto interleave = [&](auto mask_tag) {
     constexpr bool MASK = decltype(mask_tag)::value;
+    // the first LDS reads go out ahead of the first matrix instruction, so that every operand has
+    // been on its way for several steps when its (in-order) consumer is reached
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
     for (int i = 0; i < 2 * (D / 16); ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);

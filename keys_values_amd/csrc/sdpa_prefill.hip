@@ -78,7 +78,8 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
 // ds_read_b64_tr_b16: within each group of 16 lanes, lane i (a = i % 4, r = i / 4) supplies the
 // address of 4 consecutive bf16 of "row r, columns 4a..4a+3"; it receives column i of rows 0..3.
-__device__ __forceinline__ u32x2_t lds_read_tr16(const void* p) {
+typedef char __attribute__((address_space(3))) * lds_ptr_t;
+__device__ __forceinline__ u32x2_t lds_read_tr16(lds_ptr_t p) {
   const s16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(p));
   return __builtin_bit_cast(u32x2_t, t);
 }
@@ -338,7 +339,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
 
   // second product for one tile: O^T += V^T P^T with V from v[buf]
   auto pv = [&](const uint32_t (&pb)[2][8], int buf) {
-    const char* vl = (const char*)&sm.v[buf][0][0];
+    // one LDS pointer per d tile; every read below is that pointer plus a compile-time offset
+    lds_ptr_t vl[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vl[dt] = (lds_ptr_t)((const char*)&sm.v[buf][0][0] + va[dt]);
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -347,8 +351,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
         const int rb = (32 * mt + 16 * j) * CPR * 16;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const u32x2_t lo = lds_read_tr16(vl + rb + va[dt]);
-          const u32x2_t hi = lds_read_tr16(vl + rb + va[dt] + 8 * CPR * 16);
+          const u32x2_t lo = lds_read_tr16(vl[dt] + rb);
+          const u32x2_t hi = lds_read_tr16(vl[dt] + rb + 8 * CPR * 16);
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
         }
       }
@@ -412,6 +416,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
       // interleave in the instruction stream: each matrix instruction of the second product is
       // followed by the two LDS reads of the next one and by its share of the softmax arithmetic,
       // so the vector ALU works in the shadow of the matrix core instead of after it
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // operands of the first two go out ahead
 #pragma unroll
       for (int i = 0; i < 4 * DT; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
