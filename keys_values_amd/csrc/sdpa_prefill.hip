@@ -136,6 +136,7 @@ struct Loader {
   int64_t k_tile_bytes, v_tile_bytes, k_st, v_st;
   int64_t k_step, v_step;       // bytes between this wavefront's consecutive row groups (NWAVES RPW rows)
   int wave, lane, kv_len, rl, cgk, cgv;
+  uint32_t lds_k, lds_v;        // LDS addresses of the K and V buffers (wavefront-uniform)
   // uint8 path staging registers
   u32x2_t kc[NI], vc[NI];
   float ksr[NI], vsr[NI];
@@ -143,8 +144,10 @@ struct Loader {
 
   __device__ __forceinline__ int row_of(int i) const { return (NWAVES * i + wave) * RPW + rl; }
 
-  __device__ __forceinline__ void init(const PrefillParams& p, int b, int kvh, int tid) {
-    wave = tid >> 6;
+  __device__ __forceinline__ void init(const PrefillParams& p, Smem<D>& sm, int b, int kvh, int tid) {
+    lds_k = __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.k[0][0][0]));
+    lds_v = __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.v[0][0][0]));
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform: keeps the LDS targets in scalar registers
     lane = tid & 63;
     rl = lane / CPR;  // row inside the group
     kv_len = p.kv_len;
@@ -183,8 +186,8 @@ struct Loader {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         if constexpr (!U8) {
-          const uint32_t dst = lds_addr_of(IS_K ? &sm.k[buf][(NWAVES * i + wave) * RPW][0] : &sm.v[buf][(NWAVES * i + wave) * RPW][0]);
-          dma16(tb + i * step, off0, __builtin_amdgcn_readfirstlane(dst));
+          const uint32_t dst = (IS_K ? lds_k : lds_v) + (uint32_t)((buf * BN + (NWAVES * i + wave) * RPW) * CPR * 16);
+          dma16(tb + i * step, off0, dst);
         } else {
           const int key = key0 + row_of(i);
           const u32x2_t c = *(const u32x2_t*)(tb + i * step + off0);
@@ -200,8 +203,8 @@ struct Loader {
         const int key = min(key0 + row_of(i), kv_len - 1);
         const uint32_t off = (uint32_t)(((int64_t)(key - key0) * st + (IS_K ? cgk : cgv) * 8) * ESZ);
         if constexpr (!U8) {
-          const uint32_t dst = lds_addr_of(IS_K ? &sm.k[buf][(NWAVES * i + wave) * RPW][0] : &sm.v[buf][(NWAVES * i + wave) * RPW][0]);
-          dma16(tb, off, __builtin_amdgcn_readfirstlane(dst));
+          const uint32_t dst = (IS_K ? lds_k : lds_v) + (uint32_t)((buf * BN + (NWAVES * i + wave) * RPW) * CPR * 16);
+          dma16(tb, off, dst);
         } else {
           const u32x2_t c = *(const u32x2_t*)(tb + off);
           if (IS_K) { kc[i] = c; ksr[i] = ks[key]; kzr[i] = kz[key]; }
@@ -363,7 +366,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const Prefill
   // K(t+1) and V(t) are in flight to the other buffers and are published by the barrier that ends
   // the iteration.
   Loader<D, U8> ld;
-  ld.init(p, b, kvh, tid);
+  ld.init(p, sm, b, kvh, tid);
   uint32_t pb_prev[2][8];
   // every split owns at least one tile (the host sizes the splits that way)
   ld.template issue_one<true>(sm, tile_begin, 0, tid);
