@@ -41,6 +41,7 @@ struct DecodeParams {
   float* part_o;   // (B, Hq, S, D)
   float* part_ml;  // (B, Hq, S, 2)
   float* lse_ws;   // (B, Hq)
+  unsigned long long* best;  // fused H2O form: (value, slot) minimum per (b, kvh) row, else NULL
   int32_t B, Hq, Hkv, kv_len, Tpad, num_splits, keys_per_split;
   float c;
   int64_t q_sb, q_sh, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, qs_sb, qs_sh;
@@ -346,6 +347,10 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
       const float lse = M + fast_log2(l4);
       p.lse_ws[bh] = lse;
       if (p.lse_out) p.lse_out[bh] = lse;
+      // fused H2O form: reset the running minimum of the KV head's row for the weights kernel
+      if (p.best && hqi % (p.Hq / p.Hkv) == 0) {
+        p.best[b * p.Hkv + hqi / (p.Hq / p.Hkv)] = ~0ull;
+      }
     }
   }
 }
@@ -362,7 +367,7 @@ __device__ __forceinline__ uint32_t ordered_bits(float x) {
 // in the same pass (keys_values/kvcache/h2o.py:175-196, keys_values/kvcache/attn_weights.py:773-774
 // for one slot): scores += W, then the (value, slot) minimum of the row through an integer atomicMin.
 template <int G, bool H2O>
-__global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams p, const kvx_h2o_args hh, unsigned long long* best) {
+__global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams p, const kvx_h2o_args hh) {
   typedef float fG __attribute__((ext_vector_type(G >= 4 ? 4 : (G == 2 ? 2 : 1))));
   constexpr int NV = G >= 4 ? G / 4 : 1;
   const int kvh = blockIdx.y, b = blockIdx.z;
@@ -419,15 +424,14 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams 
     if (threadIdx.x == 0) {
       unsigned long long mn = wbest[0];
       for (int i = 1; i < 4; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
-      if (mn != ~0ull) atomicMin(best + b * p.Hkv + kvh, mn);
+      if (mn != ~0ull) atomicMin(p.best + b * p.Hkv + kvh, mn);
     }
   }
 }
 
-__global__ void decode_argmin_init_kernel(unsigned long long* best, int rows) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < rows) best[i] = ~0ull;
-}
+// Publishes the slot of each row's minimum. A separate launch: doing it in the last workgroup of the
+// weights kernel needs a device-scope fence per workgroup, which on this multi-die part writes back L2
+// and more than doubles that kernel's time.
 __global__ void decode_argmin_finish_kernel(const unsigned long long* best, int32_t* next_index, int rows) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < rows) next_index[i] = (int32_t)(best[i] & 0xffffffffull);
@@ -435,7 +439,7 @@ __global__ void decode_argmin_finish_kernel(const unsigned long long* best, int3
 
 struct Plan {
   int G, num_splits, keys_per_split, Tpad;
-  size_t off_logits, off_part_o, off_part_ml, off_lse, total;
+  size_t off_logits, off_part_o, off_part_ml, off_lse, off_best, total;
 };
 
 Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
@@ -463,6 +467,9 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   off += (size_t)a.B * a.Hq * pl.num_splits * 2 * 4;
   pl.off_lse = off;
   off += (size_t)a.B * a.Hq * 4;
+  off = (off + 7) & ~(size_t)7;
+  pl.off_best = off;
+  off += fused_h2o ? (size_t)a.B * a.Hkv * 8 : 0;
   pl.total = (off + 255) & ~(size_t)255;
   return pl;
 }
@@ -470,12 +477,6 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
 template <int D, int G>
 int launch_dg(const DecodeParams& p, bool u8, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
-  unsigned long long* best = hh ? (unsigned long long*)hh->workspace : nullptr;
-  const int rows = p.B * p.Hkv;
-  if (hh) {
-    hipLaunchKernelGGL(decode_argmin_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, rows);
-    KVX_HIP(hipGetLastError());
-  }
   if (u8) hipLaunchKernelGGL((decode_split_kernel<D, G, true>), grid, dim3(NTHREADS), 0, st, p);
   else hipLaunchKernelGGL((decode_split_kernel<D, G, false>), grid, dim3(NTHREADS), 0, st, p);
   KVX_HIP(hipGetLastError());
@@ -483,13 +484,14 @@ int launch_dg(const DecodeParams& p, bool u8, const kvx_h2o_args* hh, hipStream_
   KVX_HIP(hipGetLastError());
   const dim3 wgrid((p.kv_len + 4095) / 4096, p.Hkv, p.B);
   if (hh) {
-    hipLaunchKernelGGL((decode_weights_kernel<G, true>), wgrid, dim3(256), 0, st, p, *hh, best);
+    hipLaunchKernelGGL((decode_weights_kernel<G, true>), wgrid, dim3(256), 0, st, p, *hh);
     KVX_HIP(hipGetLastError());
-    hipLaunchKernelGGL(decode_argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, hh->next_index, rows);
+    const int rows = p.B * p.Hkv;
+    hipLaunchKernelGGL(decode_argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.best, hh->next_index, rows);
     KVX_HIP(hipGetLastError());
   } else if (p.w) {
     kvx_h2o_args none = {};
-    hipLaunchKernelGGL((decode_weights_kernel<G, false>), wgrid, dim3(256), 0, st, p, none, best);
+    hipLaunchKernelGGL((decode_weights_kernel<G, false>), wgrid, dim3(256), 0, st, p, none);
     KVX_HIP(hipGetLastError());
   }
   return KVX_OK;
@@ -531,6 +533,7 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.part_o = (float*)(ws + pl.off_part_o);
   p.part_ml = (float*)(ws + pl.off_part_ml);
   p.lse_ws = (float*)(ws + pl.off_lse);
+  p.best = hh ? (unsigned long long*)(ws + pl.off_best) : nullptr;
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
   p.num_splits = pl.num_splits; p.keys_per_split = pl.keys_per_split;
   p.c = a.sm_scale * kLog2e;
