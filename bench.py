@@ -51,12 +51,16 @@ def parse():
     ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8"],
+                    help="cache storage for the prefill / decode workloads; uint8 = BASELINE.json configs[2]: codes + per-row "
+                         "scale and zero point, dequantised inside the attention kernels")
     return ap.parse_args()
 
 
-def rope_inputs(torch, O, dev):
-    B, Hq, Hkv, q_len, T, D, input_pos = 1, 32, 8, 1024, 32768, 128, 31744
-    gen = torch.Generator().manual_seed(1)
+def rope_inputs(torch, O, dev, T=32768, seed=1):
+    B, Hq, Hkv, q_len, D = 1, 32, 8, 1024, 128
+    input_pos = T - q_len
+    gen = torch.Generator().manual_seed(seed)
     q = torch.randn(B, Hq, q_len, D, generator=gen)
     k = torch.randn(B, Hkv, T, D, generator=gen)
     v = torch.randn(B, Hkv, T, D, generator=gen).to(torch.bfloat16)
@@ -71,15 +75,31 @@ def bench_prefill(args, torch, dev):
     from oracle import kvx_oracle as O
 
     lib = _lib.load()
-    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev)
+    u8 = args.kv == "uint8"
+    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev, 65536 if u8 else 32768, 2 if u8 else 1)
     scale = D ** -0.5
     q, k, v = q_c.to(dev), k_c.to(dev), v_c.to(dev)
+    quant = None
+    if u8:
+        # quantise with the library's own kernel; the CPU sample below attends over the dequantised rows
+        def quantise(x):
+            c = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+            sc = torch.empty(x.shape[:-1], dtype=torch.float32, device=dev)
+            zp = torch.empty(x.shape[:-1], dtype=torch.int32, device=dev)
+            _lib.check(lib.kvx_quantize_rows(x.data_ptr(), D, x.numel() // D, D, c.data_ptr(), sc.data_ptr(), zp.data_ptr(), _lib.stream_ptr(dev)))
+            return c, sc, zp
+        k, ksc, kzp = quantise(k)
+        v, vsc, vzp = quantise(v)
+        quant = ops.QuantState(ksc, kzp, vsc, vzp)
+        torch.cuda.synchronize()
+        k_c = O.dequantize_rows(k.cpu(), ksc.cpu(), kzp.cpu())
+        v_c = O.dequantize_rows(v.cpu(), vsc.cpu(), vzp.cpu())
     out = torch.empty((B, q_len, Hq, D), dtype=torch.bfloat16, device=dev)
     o_view = out.permute(0, 2, 1, 3)
     lse = torch.empty((B, q_len, Hq), dtype=torch.float32, device=dev)
     w = torch.empty((B, Hkv, T), dtype=torch.float32, device=dev)
     a = _lib.SdpaArgs()
-    ops._fill_common(a, q, k, v, scale, input_pos, None, None, args.splits)
+    ops._fill_common(a, q, k, v, scale, input_pos, None, quant, args.splits)
     a.o = o_view.data_ptr()
     a.o_stride_b, a.o_stride_h, a.o_stride_t = o_view.stride(0), o_view.stride(1), o_view.stride(2)
     a.lse, a.w = lse.data_ptr(), w.data_ptr()
@@ -136,7 +156,7 @@ def bench_prefill(args, torch, dev):
             "unit": "TFLOP/s",
             "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"KV head 0 of {Hkv} (4 query heads x 1024 queries x 32768 keys), one pass, {t_c:.1f} s",
+            "sample": f"KV head 0 of {Hkv} (4 query heads x 1024 queries x {T} keys), one pass, {t_c:.1f} s",
         }
         # the sample doubles as an end-to-end check of the timed outputs
         err = ((out.permute(0, 2, 1, 3)[:, : 4 * hs].float().cpu() - o_ref.float()).norm() / o_ref.float().norm()).item()
@@ -157,7 +177,9 @@ def bench_prefill(args, torch, dev):
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE.json configs[1]: chunked prefill attention + score-sum, B1 Hq32 Hkv8 D128 T32768 q1024, RoPE theta 1e6, seed 1",
+            "workload": ("BASELINE.json configs[2]: attention + score-sum over the uint8 cache (dequantised in the kernels), B1 Hq32 Hkv8 D128 T65536 q1024, seed 2"
+                         if u8 else
+                         "BASELINE.json configs[1]: chunked prefill attention + score-sum, B1 Hq32 Hkv8 D128 T32768 q1024, RoPE theta 1e6, seed 1"),
             "flops_algorithmic": flops_alg,
             "flops_issued": flops_issued,
             "pct_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
@@ -168,12 +190,12 @@ def bench_prefill(args, torch, dev):
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "sdpa_prefill_kernel<128,false> (+ split merge)",
+            "kernel": "sdpa_prefill_kernel<128,%s> (+ split merge)" % ("true" if u8 else "false"),
             "achieved": round(attn_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": TRAFFIC_BYTES["prefill"],
+            "traffic": None if u8 else TRAFFIC_BYTES["prefill"],
         },
         "cpu_baseline": cpu,
     }
@@ -242,10 +264,20 @@ def bench_decode(args, torch, dev):
 
     B, Hq, Hkv, L, D = 8, 32, 8, 131072, 128
     gen = torch.Generator(device=dev).manual_seed(3)
-    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, device=dev)
+    u8 = args.kv == "uint8"
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, quantized=u8, device=dev)
     # state as after a prefill that filled the cache (the prefill itself is not part of this workload)
-    cache.k.copy_(torch.randn(cache.k.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
-    cache.v.copy_(torch.randn(cache.v.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
+    if u8:
+        lib = _lib.load()
+        for codes, sc, zp in ((cache.k, cache.k_scale, cache.k_zp), (cache.v, cache.v_scale, cache.v_zp)):
+            for bi in range(B):  # one batch row at a time keeps the bf16 temporaries small
+                x = torch.randn(codes[bi].shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                _lib.check(lib.kvx_quantize_rows(x.data_ptr(), D, x.numel() // D, D, codes[bi].data_ptr(), sc[bi].data_ptr(),
+                                                 zp[bi].data_ptr(), _lib.stream_ptr(dev)))
+            torch.cuda.synchronize()
+    else:
+        cache.k.copy_(torch.randn(cache.k.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
+        cache.v.copy_(torch.randn(cache.v.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
     cache.token_pos.copy_(torch.arange(L, dtype=torch.int32, device=dev).view(1, 1, L).expand(B, Hkv, L))
     cache.batch_size, cache.current_length, cache.prefill_length = B, L, L
     cache._input_pos = L
@@ -268,11 +300,12 @@ def bench_decode(args, torch, dev):
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     ms_gpu = e0.elapsed_time(e1) / args.steps
-    bytes_alg = 2 * B * Hkv * L * D * 2 + 2 * B * Hkv * L * 4  # K + V once, scores read-modify-write
+    # K + V once (bf16 rows, or codes + 8 bytes of row state), scores read-modify-write
+    bytes_alg = 2 * B * Hkv * L * (D + 8 if u8 else 2 * D) + 2 * B * Hkv * L * 4
     gbs = bytes_alg / (ms_step * 1e-3) / 1e9
     # the dominant launch alone: the fused attention + score update + argmin call (split attention,
     # merge, weights kernels), events on the launch stream around each call
-    launch, _ = cache._decode_h2o_prepare(qs[0], cache.k, cache.v, None)
+    launch, _ = cache._decode_h2o_prepare(qs[0], cache.k, cache.v, cache._quant_state(L))
     launch()
     torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
@@ -286,7 +319,11 @@ def bench_decode(args, torch, dev):
     if not args.no_cpu_baseline:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         nb = 2  # batch rows 0-1 of 8, all KV heads: a quarter of one step's attention
-        kc, vc = cache.k[:nb].cpu(), cache.v[:nb].cpu()
+        if u8:
+            kc = O.dequantize_rows(cache.k[:nb].cpu(), cache.k_scale[:nb].cpu(), cache.k_zp[:nb].cpu())
+            vc = O.dequantize_rows(cache.v[:nb].cpu(), cache.v_scale[:nb].cpu(), cache.v_zp[:nb].cpu())
+        else:
+            kc, vc = cache.k[:nb].cpu(), cache.v[:nb].cpu()
         qc = qs[0, :nb].cpu()
         t_c0 = time.perf_counter()
         O.sdpa_in_blocks(qc, kc, vc, D ** -0.5, L, None)
@@ -298,13 +335,13 @@ def bench_decode(args, torch, dev):
         "metric": "decode + H2O step GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3",
+        "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3" + (", uint8 cache" if u8 else ""),
                    "bytes_algorithmic_per_step": bytes_alg, "ms_per_step_gpu_events": round(ms_gpu, 4),
                    "decode_tokens_per_s": round(B / (ms_step * 1e-3), 1)},
-        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,false> + merge + weights/score update/argmin",
+        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + merge + weights/score update/argmin" % ("true" if u8 else "false"),
                      "achieved": round(bytes_alg / (ms_call * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(bytes_alg / (ms_call * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "ms_per_launch": round(ms_call, 4),
-                     "traffic": TRAFFIC_BYTES["decode"]},
+                     "traffic": None if u8 else TRAFFIC_BYTES["decode"]},
         "cpu_baseline": cpu,
     }
 

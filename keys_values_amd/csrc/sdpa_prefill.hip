@@ -7,7 +7,7 @@
 // Work decomposition
 //   The G query heads that share a KV head are packed into the row dimension: row r of a
 //   (batch, KV head) pair is (query r / G, head r % G), R = q_len * G rows in all. A workgroup of
-//   four wavefronts owns 128 consecutive rows (32 per wavefront) and walks the key tiles of its KV
+//   four (uint8 cache: eight) wavefronts owns 32 consecutive rows per wavefront and walks the key tiles of its KV
 //   split, 64 keys at a time, so a K/V tile staged once in LDS serves all G heads.
 //   Scores are produced TRANSPOSED, S^T = K Q^T (32x32x16 bf16 MFMA, keys along M, rows along N):
 //   every lane then owns one row's statistics (running max and sum) and only the other half of the
@@ -28,10 +28,11 @@ namespace {
 
 constexpr float kSlackLog2 = 8.0f;  // see the running-maximum update in the kernel
 
-constexpr int NWAVES = 4;        // wavefronts per workgroup, 32 rows each
-constexpr int BM = 32 * NWAVES;  // rows per workgroup
+// Wavefronts per workgroup, 32 rows each. The uint8 cache takes 8: a tile is dequantised once per
+// workgroup, so twice the rows halve that vector work per row (-13 % kernel time); for bf16 tiles the
+// two sizes run alike and the smaller one leaves more workgroups for short chunks.
+constexpr int nwaves(bool u8) { return u8 ? 8 : 4; }
 constexpr int BN = 64;   // keys per tile
-constexpr int NTHREADS = 64 * NWAVES;
 
 struct PrefillParams {
   const uint16_t* q;
@@ -123,6 +124,8 @@ template <int D, bool U8>
 struct Loader {
   static constexpr int CPR = D / 8;
   static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
+  static constexpr int NWAVES = nwaves(U8);
+  static constexpr int NTHREADS = 64 * NWAVES;
   static constexpr int NI = BN / RPW / NWAVES;     // instructions per wavefront per operand: 4 / 2
   static constexpr int ESZ = U8 ? 1 : 2;
   const char* kbase;
@@ -241,7 +244,8 @@ struct Loader {
 };
 
 template <int D, bool U8>
-__global__ __launch_bounds__(NTHREADS, 2) void sdpa_prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(64 * nwaves(U8), U8 ? 1 : 2) void sdpa_prefill_kernel(const PrefillParams p) {
+  constexpr int BM = 32 * nwaves(U8);  // rows per workgroup
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;  // k-steps of the first product
   constexpr int DT = D / 32;  // d tiles of the second product
@@ -555,7 +559,8 @@ void fill_params(PrefillParams& p, const kvx_sdpa_args& a) {
   p.R = a.q_len * p.G;
   p.input_pos = a.input_pos;
   p.num_tiles = (a.kv_len + BN - 1) / BN;
-  p.m_blocks = (p.R + BM - 1) / BM;
+  const int bm = 32 * nwaves(a.kv_dtype == KVX_KV_U8);
+  p.m_blocks = (p.R + bm - 1) / bm;
   p.num_splits = pick_splits(a, p.m_blocks, p.num_tiles);
   p.tiles_per_split = (p.num_tiles + p.num_splits - 1) / p.num_splits;
   p.num_splits = (p.num_tiles + p.tiles_per_split - 1) / p.tiles_per_split;
@@ -579,7 +584,7 @@ size_t partial_bytes(const PrefillParams& p, int D) {
 template <int D, bool U8>
 int launch_t(PrefillParams& p, hipStream_t st) {
   dim3 grid(p.B * p.Hkv, p.m_blocks, p.num_splits);
-  hipLaunchKernelGGL((sdpa_prefill_kernel<D, U8>), grid, dim3(NTHREADS), 0, st, p);
+  hipLaunchKernelGGL((sdpa_prefill_kernel<D, U8>), grid, dim3(64 * nwaves(U8)), 0, st, p);
   KVX_HIP(hipGetLastError());
   if (p.num_splits > 1) {
     constexpr int ROWS = 256 / (D / 4);
