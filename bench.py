@@ -37,9 +37,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (KiB per dispatch, one counter per run, on these same workloads), each scaled by what the counter
 # reads for the `calib` launch of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
 TRAFFIC_BYTES = {
-    "prefill": int((76989.8 * 2.000 + 66560.0) * 1024),    # sdpa_prefill_kernel<128,false>
-    "decode": int((2099047.6 * 2.000 + 139780.2) * 1024),  # decode_split_kernel<128,4,false>
-    "quantize": int((65576.8 * 2.000 + 69635.2) * 1024),   # quantize_rows_kernel<128>
+    "prefill": int((76748.7 * 2.000 + 66560.0) * 1024),    # sdpa_prefill_kernel<128,false>
+    "decode": int((2099026.5 * 2.000 + 139780.3) * 1024),  # decode_split_kernel<128,4,false>
+    "quantize": int((65576.8 * 2.000 + 69632.1) * 1024),   # quantize_rows_kernel<128>
 }
 
 
