@@ -143,10 +143,10 @@ def bench_prefill(args, torch, dev):
 
     cpu = None
     if not args.no_cpu_baseline:
-        # bounded sample: KV head 0 with its 4 query heads = 1/8 of the workload, same op sequence
-        # as the reference's eager path (fp32 upcast, <= 3 GB score slices, mask, softmax, mean/sum)
+        # bounded sample: the first KV heads with their query heads, same op sequence as the
+        # reference's eager path (fp32 upcast, <= 3 GB score slices, mask, softmax, mean/sum)
         torch.set_num_threads(min(16, os.cpu_count() or 1))
-        hs = 1
+        hs = Hkv  # the whole workload: a second or two on the host's cores
         qs, ks, vs = q_c[:, : 4 * hs], k_c[:, :hs], v_c[:, :hs]
         t_c0 = time.perf_counter()
         o_ref, w_ref = O.sdpa_in_blocks(qs, ks, vs, scale, input_pos, None)
@@ -156,7 +156,7 @@ def bench_prefill(args, torch, dev):
             "unit": "TFLOP/s",
             "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"KV head 0 of {Hkv} (4 query heads x 1024 queries x {T} keys), one pass, {t_c:.1f} s",
+            "sample": f"KV heads 0-{hs - 1} of {Hkv} ({4 * hs} query heads x 1024 queries x {T} keys), one pass, {t_c:.1f} s",
         }
         # the sample doubles as an end-to-end check of the timed outputs
         err = ((out.permute(0, 2, 1, 3)[:, : 4 * hs].float().cpu() - o_ref.float()).norm() / o_ref.float().norm()).item()
@@ -318,7 +318,7 @@ def bench_decode(args, torch, dev):
     cpu = None
     if not args.no_cpu_baseline:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
-        nb = 2  # batch rows 0-1 of 8, all KV heads: a quarter of one step's attention
+        nb = B  # the attention of one whole step
         if u8:
             kc = O.dequantize_rows(cache.k[:nb].cpu(), cache.k_scale[:nb].cpu(), cache.k_zp[:nb].cpu())
             vc = O.dequantize_rows(cache.v[:nb].cpu(), cache.v_scale[:nb].cpu(), cache.v_zp[:nb].cpu())
