@@ -141,6 +141,34 @@ def bench_prefill(args, torch, dev):
     rows = w.sum(-1).cpu()
     assert torch.allclose(rows, torch.full_like(rows, float(q_len)), rtol=1e-4, atol=5e-2), rows
 
+    # The same chunk through the cache object (keys_values/kvcache/base.py:554-595): write the 1024 new
+    # rows into the slots chosen by the step before, attend, score-sum, scores += W, choose the next
+    # 1024 lowest-score slots. Steady state: after the first step the positions are scattered.
+    h2o_ms = None
+    if not u8:
+        from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
+        cache = H2OKVCache(KVCacheParams(B, Hkv, T, D, Hq), max_chunk_size=q_len, device=dev)
+        cache.k.copy_(k)
+        cache.v.copy_(v)
+        cache.token_pos.copy_(torch.arange(T, dtype=torch.int32, device=dev).view(1, 1, T).expand(B, Hkv, T))
+        cache.scores.copy_(torch.rand((B, Hkv, T), device=dev))
+        cache.batch_size, cache.current_length, cache.prefill_length = B, T, T
+        cache._input_pos = T
+        cache._use_initial_rule = False
+        cache._next_index.copy_(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
+        cache._have_next = True
+        kn, vn = k[:, :, -q_len:].contiguous(), v[:, :, -q_len:].contiguous()
+        for _ in range(3):
+            cache.forward(q, kn, vn)
+        torch.cuda.synchronize()
+        h0, h1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        h0.record()
+        for _ in range(10):
+            cache.forward(q, kn, vn)
+        h1.record()
+        torch.cuda.synchronize()
+        h2o_ms = h0.elapsed_time(h1) / 10
+
     cpu = None
     if not args.no_cpu_baseline:
         # bounded sample: the first KV heads with their query heads, same op sequence as the
@@ -187,6 +215,8 @@ def bench_prefill(args, torch, dev):
             "ms_attention_kernel": round(ms_attn, 4),
             "ms_score_sum_kernel": round(ms_score, 4),
             "score_sum_tflops": round(2.0 * B * Hq * q_len * T * D / (ms_score * 1e-3) / 1e12, 2),
+            "h2o_cache_chunk_ms": None if h2o_ms is None else round(h2o_ms, 4),
+            "h2o_cache_chunk_tokens_per_s": None if h2o_ms is None else round(q_len / (h2o_ms * 1e-3), 1),
         },
         "roofline": {
             "bound": "mfma",

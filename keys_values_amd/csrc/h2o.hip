@@ -8,10 +8,11 @@
 //   k == 1 (single-token decode): a streaming pass over all rows with many workgroups; each folds
 //          its slice into one 64-bit key (ordered value bits << 32 | slot) and publishes it with
 //          an integer atomicMin, which is order independent and therefore deterministic.
-//   k  > 1 (chunked prefill): one workgroup per (batch, head) row. A 4-pass 8-bit radix select over
-//          the ordered value bits finds the k-th smallest value; elements below it, plus the
-//          lowest-slot elements equal to it, are gathered into LDS and bitonic-sorted as 64-bit
-//          (value, slot) keys.
+//   k  > 1 (chunked prefill): one workgroup per (batch, head) row. The first pass adds the weights and
+//          leaves the row's ordered value bits in LDS (rows of up to ~36K slots; longer rows are
+//          re-read from global memory). A 4-pass 8-bit radix select finds the k-th smallest value;
+//          elements below it, plus the lowest-slot elements equal to it, are gathered and
+//          bitonic-sorted as 64-bit (value, slot) keys.
 #include "kvx_common.h"
 
 namespace kvx {
@@ -106,11 +107,17 @@ __global__ void argmin_finish_kernel(const unsigned long long* best, int32_t* ne
 
 // ---- k > 1 ----------------------------------------------------------------------------------
 
-__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a) {
-  __shared__ unsigned long long cand[MAX_K];
+// CACHED: the row's ordered keys live in LDS after the first pass (rows of up to ~36K slots), so the
+// radix passes and the gather never go back to global memory.
+template <bool CACHED>
+__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a, int kpad) {
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  unsigned long long* cand = (unsigned long long*)dyn_lds;    // kpad entries
+  uint32_t* keys = (uint32_t*)(dyn_lds + (size_t)kpad * 8);   // a.limit entries (CACHED only)
   __shared__ uint32_t hist[256];
   __shared__ uint32_t wave_cnt[SEL_THREADS / 64];
-  __shared__ uint32_t sh_prefix, sh_krem, sh_nless, sh_eqbase;
+  __shared__ uint32_t sh_prefix, sh_krem, sh_nless, sh_diff;
+  __shared__ int sh_hi;
 
   const int tid = threadIdx.x;
   const int row = blockIdx.x;
@@ -119,82 +126,151 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   const float* w = a.w ? a.w + (int64_t)row * a.kv_len : nullptr;
   const int32_t* tpr = a.token_pos ? a.token_pos + b * a.tp_stride_b + hh * a.tp_stride_h : nullptr;
 
-  // pass 0: scores += w. Every later pass of this thread touches the same slots it wrote here.
-  if (w)
-    for (int i = tid; i < a.kv_len; i += SEL_THREADS) sc[i] += w[i];
+  // pass 0: scores += w (every later pass of this thread touches the slots it wrote here) and the keys
+  // One workgroup walks the whole row: batches of 8 loads per array are issued before anything is
+  // stored, otherwise the stores to sc (which may alias w for all the compiler knows) serialise the
+  // loads and the pass costs one memory round trip per element of a thread.
+  const int n0 = max(a.kv_len, a.limit);
+  constexpr int PB = 8;
+  for (int i0 = tid; i0 < n0; i0 += PB * SEL_THREADS) {
+    float sv[PB], wv[PB];
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+      const int i = i0 + j * SEL_THREADS;
+      sv[j] = i < n0 ? sc[i] : 0.0f;
+      wv[j] = (w && i < a.kv_len) ? w[i] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+      const int i = i0 + j * SEL_THREADS;
+      if (i >= n0) break;
+      float v = sv[j];
+      if (w && i < a.kv_len) {
+        v += wv[j];
+        sc[i] = v;
+      }
+      if (CACHED && i < a.limit) keys[i] = ordered_bits(select_value(v, a, tpr, i));
+    }
+  }
+  auto key_of = [&](int i) -> uint32_t {
+    if constexpr (CACHED) return keys[i];
+    else return ordered_bits(select_value(sc[i], a, tpr, i));
+  };
 
-  int kpad = 1;
-  while (kpad < a.k) kpad <<= 1;
   for (int i = tid; i < kpad; i += SEL_THREADS) cand[i] = ~0ull;
   if (tid == 0) {
     sh_prefix = 0;
     sh_krem = (uint32_t)a.k;
     sh_nless = 0;
-    sh_eqbase = 0;
+    sh_diff = 0;
   }
   __syncthreads();
 
-  // radix select: after the pass for digit `dg`, sh_prefix holds the digits dg..3 of the k-th
-  // smallest key and sh_krem its rank among the keys sharing them.
-  for (int dg = 3; dg >= 0; --dg) {
+  // Bits that all keys of the row share need no pass, and skipping them matters: scores of one row
+  // share their sign and most of their exponent, so a first digit taken from bit 31 down would send
+  // nearly every key to the same few LDS counters (same-address atomics serialise).
+  {
+    const uint32_t key0 = key_of(0);
+    uint32_t diff = 0;
+    for (int i = tid; i < a.limit; i += SEL_THREADS) diff |= key_of(i) ^ key0;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) diff |= __shfl_xor(diff, off, 64);
+    if ((tid & 63) == 0 && diff) atomicOr(&sh_diff, diff);
+    __syncthreads();
+    if (tid == 0) {
+      const int top = sh_diff ? 32 - __clz(sh_diff) : 0;  // bits [0, top) differ somewhere
+      sh_hi = top;
+      sh_prefix = top >= 32 ? 0u : (key0 >> top) << top;
+    }
+    __syncthreads();
+  }
+  // radix select over the remaining bits, 8 at a time from the top: after a pass sh_prefix holds the
+  // bits [lo, 32) of the k-th smallest key and sh_krem its rank among the keys sharing them.
+  for (int hi = sh_hi; hi > 0;) {
+    const int lo = max(hi - 8, 0);
     if (tid < 256) hist[tid] = 0;
     __syncthreads();
     const uint32_t prefix = sh_prefix;
-    const uint32_t himask = dg == 3 ? 0u : (0xffffffffu << (8 * (dg + 1)));
+    const uint32_t himask = hi >= 32 ? 0u : (0xffffffffu << hi);
+    const uint32_t dmask = (1u << (hi - lo)) - 1u;
     for (int i = tid; i < a.limit; i += SEL_THREADS) {
-      const uint32_t u = ordered_bits(select_value(sc[i], a, tpr, i));
-      if ((u & himask) == prefix) atomicAdd(&hist[(u >> (8 * dg)) & 255u], 1u);
+      const uint32_t u = key_of(i);
+      if ((u & himask) == prefix) atomicAdd(&hist[(u >> lo) & dmask], 1u);
     }
     __syncthreads();
-    if (tid == 0) {
-      uint32_t krem = sh_krem, cum = 0;
-      int d = 0;
-      for (; d < 256; ++d) {
-        if (cum + hist[d] >= krem) break;
-        cum += hist[d];
+    if (tid < 64) {
+      // the digit where the running count reaches the rank: 4 bins per lane, wavefront prefix sum
+      const uint32_t krem = sh_krem;
+      uint32_t h4[4], tot = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        h4[j] = hist[4 * tid + j];
+        tot += h4[j];
       }
-      sh_prefix = prefix | ((uint32_t)d << (8 * dg));
-      sh_krem = krem - cum;
+      uint32_t incl = tot;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t o = __shfl_up(incl, off, 64);
+        if (tid >= off) incl += o;
+      }
+      uint32_t cum = incl - tot;  // keys in the bins before this lane's
+      if (cum < krem && incl >= krem) {
+        int j = 0;
+        for (; j < 3; ++j) {
+          if (cum + h4[j] >= krem) break;
+          cum += h4[j];
+        }
+        sh_prefix = prefix | ((uint32_t)(4 * tid + j) << lo);
+        sh_krem = krem - cum;
+      }
     }
     __syncthreads();
+    hi = lo;
   }
   const uint32_t ustar = sh_prefix;   // k-th smallest value
   const uint32_t need_eq = sh_krem;   // how many slots equal to it are taken (lowest slots first)
   const uint32_t nless = (uint32_t)a.k - need_eq;
 
-  // gather: slots below ustar in any order, slots equal to it by ascending slot
+  // gather: slots below ustar in any order; slots equal to it by ascending slot. Every wavefront
+  // owns a contiguous stretch of the row, so slot order is (wavefront, step, lane) order and the
+  // ties need two barriers in all: count per wavefront, prefix, place.
   const int lane = tid & 63, wave = tid >> 6;
-  for (int i0 = 0; i0 < a.limit; i0 += SEL_THREADS) {
-    const int i = i0 + tid;
-    uint32_t u = 0xffffffffu;
-    bool less = false, eq = false;
-    if (i < a.limit) {
-      u = ordered_bits(select_value(sc[i], a, tpr, i));
-      less = u < ustar;
-      eq = u == ustar;
+  constexpr int NWV = SEL_THREADS / 64;
+  const int chunk = ((a.limit + NWV - 1) / NWV + 63) / 64 * 64;
+  const int c_begin = wave * chunk, c_end = min(c_begin + chunk, a.limit);
+  uint32_t my_eq = 0;
+  for (int i0 = c_begin; i0 < c_end; i0 += 64) {
+    const int i = i0 + lane;
+    const uint32_t u = i < c_end ? key_of(i) : 0xffffffffu;
+    const bool less = i < c_end && u < ustar;
+    const unsigned long long lm = __ballot(less);
+    if (lm) {
+      uint32_t base = 0;
+      if (lane == 0) base = atomicAdd(&sh_nless, (uint32_t)__popcll(lm));
+      base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+      if (less) cand[base + (uint32_t)__popcll(lm & ((1ull << lane) - 1ull))] = ((unsigned long long)u << 32) | (unsigned)i;
     }
-    if (less) {
-      const uint32_t pos = atomicAdd(&sh_nless, 1u);
-      cand[pos] = ((unsigned long long)u << 32) | (unsigned)i;
-    }
-    const unsigned long long eqm = __ballot(eq);
-    if (lane == 0) wave_cnt[wave] = (uint32_t)__popcll(eqm);
-    __syncthreads();
-    if (eq) {
-      uint32_t rank = sh_eqbase + (uint32_t)__popcll(eqm & ((1ull << lane) - 1ull));
-      for (int ww = 0; ww < wave; ++ww) rank += wave_cnt[ww];
-      if (rank < need_eq) cand[nless + rank] = ((unsigned long long)u << 32) | (unsigned)i;
-    }
-    __syncthreads();
-    if (tid == 0) {
-      uint32_t t = 0;
-      for (int ww = 0; ww < SEL_THREADS / 64; ++ww) t += wave_cnt[ww];
-      sh_eqbase += t;
-    }
-    __syncthreads();
+    my_eq += (uint32_t)__popcll(__ballot(i < c_end && u == ustar));
   }
+  if (lane == 0) wave_cnt[wave] = my_eq;
+  __syncthreads();
+  uint32_t rank = 0;  // ties in the wavefronts before this one
+  for (int ww = 0; ww < wave; ++ww) rank += wave_cnt[ww];
+  if (rank < need_eq && my_eq) {
+    for (int i0 = c_begin; i0 < c_end; i0 += 64) {
+      const int i = i0 + lane;
+      const bool eq = i < c_end && key_of(i) == ustar;
+      const unsigned long long eqm = __ballot(eq);
+      const uint32_t r = rank + (uint32_t)__popcll(eqm & ((1ull << lane) - 1ull));
+      if (eq && r < need_eq) cand[nless + r] = ((unsigned long long)ustar << 32) | (unsigned)i;
+      rank += (uint32_t)__popcll(eqm);
+    }
+  }
+  __syncthreads();
 
-  // bitonic sort of kpad 64-bit keys
+  // bitonic sort of kpad 64-bit keys. Comparator t of a stage with stride <= 64 only touches the 128
+  // keys of its own wavefront's stretch, and a wavefront's LDS accesses execute in order: those
+  // stages need no workgroup barrier.
   for (int size = 2; size <= kpad; size <<= 1)
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
       for (int t = tid; t < kpad / 2; t += SEL_THREADS) {
@@ -207,8 +283,10 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
           cand[hi] = x;
         }
       }
-      __syncthreads();
+      if (stride > 64 || (stride == 1 && 2 * size > 128)) __syncthreads();
+      else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     }
+  __syncthreads();
   for (int j = tid; j < a.k; j += SEL_THREADS) a.next_index[(int64_t)row * a.k + j] = (int32_t)(cand[j] & 0xffffffffull);
 }
 
@@ -231,7 +309,18 @@ int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st) {
     KVX_HIP(hipGetLastError());
     return KVX_OK;
   }
-  hipLaunchKernelGGL(update_select_kernel, dim3(rows), dim3(SEL_THREADS), 0, st, a);
+  int kpad = 1;
+  while (kpad < a.k) kpad <<= 1;
+  // keys in LDS when the row fits beside the candidates (144 KB of the 160 KB of a compute unit)
+  constexpr size_t kDynLimit = 144 * 1024;
+  const size_t cached_bytes = (size_t)kpad * 8 + (size_t)a.limit * 4;
+  if (cached_bytes <= kDynLimit) {
+    if (cached_bytes > 48 * 1024)  // beyond the default dynamic LDS allowance (the setting is per device and kernel)
+      KVX_HIP(hipFuncSetAttribute((const void*)update_select_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLimit));
+    hipLaunchKernelGGL(update_select_kernel<true>, dim3(rows), dim3(SEL_THREADS), cached_bytes, st, a, kpad);
+  } else {
+    hipLaunchKernelGGL(update_select_kernel<false>, dim3(rows), dim3(SEL_THREADS), (size_t)kpad * 8, st, a, kpad);
+  }
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
