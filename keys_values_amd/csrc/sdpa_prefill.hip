@@ -531,9 +531,10 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(const PrefillPa
 
 int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
   if (a.num_splits > 0) return min(a.num_splits, num_tiles);
-  // Aim for about four workgroups per compute unit, at least 8 key tiles per split.
+  // Aim for one resident round of workgroups (2 per compute unit, 1 with the uint8 cache): more
+  // splits only add partials to write, merge and re-read. At least 8 key tiles per split.
   const int64_t base = (int64_t)a.B * a.Hkv * m_blocks;
-  const int target = 4 * num_cus();
+  const int target = (a.kv_dtype == KVX_KV_U8 ? 1 : 2) * num_cus();
   int s = (int)((target + base - 1) / base);
   s = max(1, min(s, num_tiles / 8));
   return max(1, min(s, 64));
