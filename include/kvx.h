@@ -236,6 +236,29 @@ typedef struct kvx_h2o_args {
 int kvx_h2o_update_select(const kvx_h2o_args* args, void* stream);
 size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* args);
 
+/* ---- callers of the path: normalisation and rotary encoding of the new tokens ---------------- */
+
+/* RMS normalisation of `rows` rows of `dim` bf16 values: out = (x / (|x|_2 / sqrt(dim) + eps)) * weight,
+ * computed in fp32 with eps added to the norm, as RMSNorm.forward (keys_values/model.py:870-878).
+ * weight: fp32 (dim). dim a multiple of 8, at most 8192. In place is allowed (out == x). */
+int kvx_rmsnorm_rows(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride,
+                     const float* weight, int64_t rows, int32_t dim, float eps, void* stream);
+
+/* Per-head normalisation of the new queries and keys followed by the rotary position encoding, in
+ * place on the output of the QKV projection: what CausalSelfAttention.forward does between the
+ * projection and the cache (keys_values/model.py:733-775: norm_q / norm_k, then
+ * mha.pos_encoding -> apply_rope, keys_values/pos_encoding.py:34-44,201-238).
+ * qkv: bf16 (B, num, (Hq + 2 Hkv) * D) by strides (elements), a token's heads stored as
+ *      Hq query heads, Hkv key heads, Hkv value heads; the value heads are not touched.
+ * q_weight / k_weight: fp32 (D) norm weights, or both NULL for no normalisation.
+ * cos / sin: fp32 tables (table_rows, D / 2), row p = cos / sin of p * theta_j (half-split
+ *      convention: element d is paired with d +- D/2). Token t of the chunk sits at input_pos + t.
+ * D in {64, 128}. */
+int kvx_qk_norm_rope(void* qkv, int64_t stride_b, int64_t stride_t, int32_t B, int32_t num, int32_t Hq,
+                     int32_t Hkv, int32_t D, const float* q_weight, const float* k_weight, float eps,
+                     const float* cos, const float* sin, int32_t table_rows, int32_t input_pos,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif

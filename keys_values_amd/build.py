@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libkvx.so")
-SOURCES = ["kvx_api.hip", "sdpa_prefill.hip", "score_sum.hip", "sdpa_decode.hip", "quantize.hip", "h2o.hip"]
+SOURCES = ["kvx_api.hip", "sdpa_prefill.hip", "score_sum.hip", "sdpa_decode.hip", "quantize.hip", "h2o.hip", "norm_rope.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -41,7 +41,7 @@ def _compile(src: str) -> str:
 
 
 def build(verbose: bool = True) -> str:
-    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+    with ThreadPoolExecutor(max_workers=min(7, os.cpu_count() or 1)) as ex:
         objs = list(ex.map(_compile, SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -237,4 +237,33 @@ int kvx_sdpa_decode_h2o(const kvx_sdpa_args* a, const kvx_h2o_args* h, void* str
   return launch_sdpa_decode(*a, h, (hipStream_t)stream);
 }
 
+int kvx_rmsnorm_rows(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride, const float* weight, int64_t rows,
+                     int32_t dim, float eps, void* stream) {
+  KVX_REQUIRE(rows >= 0 && dim > 0, KVX_ERR_INVALID, "kvx_rmsnorm_rows: rows=%lld, dim=%d", (long long)rows, dim);
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(x && out && weight, KVX_ERR_INVALID, "kvx_rmsnorm_rows: NULL pointer");
+  KVX_REQUIRE(dim % 8 == 0 && dim <= 8192, KVX_ERR_UNSUPPORTED, "kvx_rmsnorm_rows: dim=%d must be a multiple of 8, at most 8192", dim);
+  KVX_REQUIRE(aligned16(x) && aligned16(out) && aligned16(weight) && mult8(x_row_stride) && mult8(out_row_stride), KVX_ERR_INVALID,
+              "kvx_rmsnorm_rows: rows must be 16-byte aligned");
+  return launch_rmsnorm_rows(x, x_row_stride, out, out_row_stride, weight, rows, dim, eps, (hipStream_t)stream);
+}
+
+int kvx_qk_norm_rope(void* qkv, int64_t stride_b, int64_t stride_t, int32_t B, int32_t num, int32_t Hq, int32_t Hkv, int32_t D,
+                     const float* q_weight, const float* k_weight, float eps, const float* cos, const float* sin, int32_t table_rows,
+                     int32_t input_pos, void* stream) {
+  KVX_REQUIRE(B >= 0 && num >= 0 && Hq > 0 && Hkv > 0, KVX_ERR_INVALID, "kvx_qk_norm_rope: B=%d num=%d Hq=%d Hkv=%d", B, num, Hq, Hkv);
+  if (B == 0 || num == 0) return KVX_OK;
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_qk_norm_rope: head size %d not in {64, 128}", D);
+  KVX_REQUIRE(qkv && cos && sin, KVX_ERR_INVALID, "kvx_qk_norm_rope: NULL pointer");
+  KVX_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), KVX_ERR_INVALID, "kvx_qk_norm_rope: give both norm weights or none");
+  KVX_REQUIRE(input_pos >= 0 && (int64_t)input_pos + num <= table_rows, KVX_ERR_INVALID,
+              "kvx_qk_norm_rope: positions %d..%lld exceed the %d rows of the cos/sin tables", input_pos, (long long)input_pos + num - 1, table_rows);
+  KVX_REQUIRE(stride_t >= (int64_t)(Hq + Hkv) * D, KVX_ERR_INVALID, "kvx_qk_norm_rope: token stride %lld shorter than the query and key heads",
+              (long long)stride_t);
+  KVX_REQUIRE(aligned16(qkv) && aligned16(cos) && aligned16(sin) && mult8(stride_b) && mult8(stride_t) &&
+                  (!q_weight || (aligned16(q_weight) && aligned16(k_weight))),
+              KVX_ERR_INVALID, "kvx_qk_norm_rope: pointers and strides must keep 16-byte alignment");
+  return launch_qk_norm_rope(qkv, stride_b, stride_t, B, num, Hq, Hkv, D, q_weight, k_weight, eps, cos, sin, input_pos, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -296,11 +296,14 @@ class H2OCacheOracle:
         self.use_initial_rule = False
         self.scale = 1.0 / math.sqrt(D)
 
-    def prefill(self, query, key, value):
+    def prefill(self, query, key, value, store_key=None, store_value=None):
+        """The first chunk attends over key / value as given (keys_values/kvcache/base.py:567-571);
+        store_key / store_value are what the buffers hold afterwards when they differ (a quantised
+        store holds the dequantised rows)."""
         n = key.shape[2]
         assert n <= self.L
-        self.k[:, :, :n] = key.to(self.k.dtype)
-        self.v[:, :, :n] = value.to(self.v.dtype)
+        self.k[:, :, :n] = (key if store_key is None else store_key).to(self.k.dtype)
+        self.v[:, :, :n] = (value if store_value is None else store_value).to(self.v.dtype)
         self.token_pos[:, :, :n] = torch.arange(n, dtype=torch.int32)
         self.scores.zero_()
         self.current_length = n
