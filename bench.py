@@ -11,6 +11,10 @@ Inputs are resident in HBM before the timed region.
 `--workload decode`  : single-token decode over a bf16 cache with score-sums, H2O score update and
                        argmin (batch 8, 32/8 heads, 131072 positions), GB/s against HBM peak.
 `--workload quantize`: affine uint8 row quantiser on (1, 8, 65536, 128) K and V, GB/s.
+`--workload longctx` : BASELINE.json configs[4]: random-init Qwen3-4B-shaped stack (36 layers), 131072 random
+                       tokens in chunks of 1024 after a 16384-token first chunk, uint8 H2O caches of 16384
+                       slots per layer; end-to-end prefill tokens/s. One step = one whole sequence.
+                       `--layers N --tokens T` shrink it (stated in the output).
 `--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
                        launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
@@ -48,9 +52,11 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "calib"])
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
+    ap.add_argument("--tokens", type=int, default=131072, help="longctx: prompt length")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8"],
                     help="cache storage for the prefill / decode workloads; uint8 = BASELINE.json configs[2]: codes + per-row "
                          "scale and zero point, dequantised inside the attention kernels")
@@ -376,6 +382,76 @@ def bench_decode(args, torch, dev):
     }
 
 
+def bench_longctx(args, torch, dev):
+    import dataclasses
+
+    from keys_values_amd.longctx.model import QWEN3_4B, LongContextPrefillModel
+
+    cfg = dataclasses.replace(QWEN3_4B, n_layer=args.layers)
+    L, chunk, seq = 16384, 1024, args.tokens
+    model = LongContextPrefillModel(cfg, cache_length=L, chunk_size=chunk, max_batch_size=1, quantized=True, max_context=max(seq, L), seed=4,
+                                    device=dev)
+    ids = torch.randint(0, cfg.vocab_size, (1, seq), generator=torch.Generator().manual_seed(4))
+    sizes = model.chunk_sizes(seq)
+    steps = max(1, min(args.steps, 3))
+    warm = 1 if args.warmup > 0 else 0
+    for _ in range(warm):
+        model.prefill(ids)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        h = model.prefill(ids)
+    e1.record()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    ms_gpu = e0.elapsed_time(e1) / steps
+    assert torch.isfinite(h.float()).all()
+    # algorithmic FLOP: attention + score-sums per chunk and layer, causal first chunk, dense layers
+    Hq, D = cfg.n_head, cfg.head_size
+    attn = 0.0
+    for i, n in enumerate(sizes):
+        T = min(sum(sizes[: i + 1]), L)
+        attn += (2.0 * Hq * n * n * D) if i == 0 else (4.0 * Hq * n * T * D)
+    attn *= cfg.n_layer
+    per_tok = 2.0 * cfg.n_layer * (cfg.n_embd * (Hq + 2 * cfg.n_query_groups) * D + Hq * D * cfg.n_embd + 3 * cfg.n_embd * cfg.intermediate_size)
+    dense = per_tok * seq
+    cpu = None
+    if not args.no_cpu_baseline:
+        # bounded sample: one layer, the first chunk shortened to 2048 tokens plus two 1024-token chunks on a
+        # 2048-slot cache, through the CPU oracle of the same stack (same op sequence as the reference's eager path)
+        from oracle import longctx_oracle as LO
+
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        c1 = dataclasses.replace(cfg, n_layer=1)
+        layer = model.layers[0]
+        weights = [{k: getattr(layer, k).cpu() for k in ("qkv", "proj", "fc_1", "fc_2", "mlp_proj", "norm_1", "norm_2", "norm_q", "norm_k")}]
+        ref = LO.PrefillOracle(c1, model.wte.cpu(), weights, model.ln_f.cpu(), 2048, chunk, 1, True, 4096)
+        t_c0 = time.perf_counter()
+        ref.forward_chunk(ids[:, :2048])
+        ref.forward_chunk(ids[:, 2048:3072])
+        ref.forward_chunk(ids[:, 3072:4096])
+        t_c = time.perf_counter() - t_c0
+        cpu = {"value": round(4096 / t_c / cfg.n_layer, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"one layer over 4096 tokens (2048-token first chunk, two 1024-token chunks, 2048-slot cache) in {t_c:.1f} s, "
+                         f"scaled to {cfg.n_layer} layers"}
+    tps = seq / (ms_step * 1e-3)
+    return {
+        "metric": "H2O long-context prefill tokens/s, Qwen3-4B shape", "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": warm, "ms_per_step": round(ms_step, 2), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"BASELINE.json configs[4]: random-init Qwen3-4B-shaped stack, {cfg.n_layer} layers, {seq} random tokens, "
+                               f"chunks {sizes[0]} + {len(sizes) - 1} x {chunk}, uint8 H2O caches of {L} slots, seed 4",
+                   "ms_per_step_gpu_events": round(ms_gpu, 2), "flops_attention_score_sums": attn, "flops_dense_layers": dense,
+                   "tflops_total": round((attn + dense) / (ms_step * 1e-3) / 1e12, 1)},
+        "roofline": {"bound": "mfma", "kernel": "whole prefill (attention + score-sum kernels and library GEMMs)",
+                     "achieved": round((attn + dense) / (ms_gpu * 1e-3) / 1e12, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round((attn + dense) / (ms_gpu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+
 def bench_calib(args, torch, dev):
     n = 1 << 29  # bf16 elements: 1 GiB in, 1 GiB out
     src = torch.ones(n, dtype=torch.bfloat16, device=dev)
@@ -409,7 +485,7 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "calib": bench_calib}[args.workload]
+    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "calib": bench_calib}[args.workload]
     res = fn(args, torch, dev)
     print(json.dumps(res), flush=True)
 

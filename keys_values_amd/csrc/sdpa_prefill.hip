@@ -301,7 +301,29 @@ __global__ __launch_bounds__(64 * nwaves(U8), U8 ? 1 : 2) void sdpa_prefill_kern
   }
 
   const int tile_begin = split * p.tiles_per_split;
-  const int tile_end = min(tile_begin + p.tiles_per_split, p.num_tiles);
+  int tile_end = min(tile_begin + p.tiles_per_split, p.num_tiles);
+  if (!p.tp) {
+    // slots hold positions 0, 1, 2, ...: tiles past the last position any row of this workgroup may
+    // see are masked out completely (the upper triangle of a causal first chunk) and are skipped
+    const int qpos_max = p.input_pos + min(mblk * BM + BM - 1, p.R - 1) / p.G;
+    tile_end = min(tile_end, qpos_max / BN + 1);
+    if (tile_end <= tile_begin) {  // whole split invisible: an empty partial (only with num_splits > 1)
+      if (row_ok) {
+        const int64_t prow = ((int64_t)split * p.B * p.Hkv + group) * p.R + row;
+        float* po = p.part_o + prow * D;
+        const f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) *(f32x4_t*)(po + dt * 32 + 8 * a + 4 * h) = z;
+        if (h == 0) {
+          p.part_ml[prow * 2] = -INFINITY;
+          p.part_ml[prow * 2 + 1] = 0.0f;
+        }
+      }
+      return;
+    }
+  }
 
   f32x16_t o[DT];
 #pragma unroll
