@@ -15,6 +15,9 @@ Inputs are resident in HBM before the timed region.
                        tokens in chunks of 1024 after a 16384-token first chunk, uint8 H2O caches of 16384
                        slots per layer; end-to-end prefill tokens/s. One step = one whole sequence.
                        `--layers N --tokens T` shrink it (stated in the output).
+`--workload policy`  : the same 1024-token chunk through the cache object (write with the ring move, attention,
+                       score-sum, score update, choice of the next 1024 slots) for each eviction-policy variant
+                       (grace period, normalised scores, V-norm weighting, Q-Hitter); ms per chunk step.
 `--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
                        launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
@@ -52,7 +55,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "calib"])
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
@@ -452,6 +455,92 @@ def bench_longctx(args, torch, dev):
     }
 
 
+def bench_policy(args, torch, dev):
+    """One 1024-token chunk into a full 32768-slot cache, per policy variant, through the cache object."""
+    from keys_values_amd.kvcache.h2o import KVCacheParams, create_kv_cache
+    from oracle import kvx_oracle as O
+
+    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev)
+    q, k, v = q_c.to(dev), k_c.to(dev), v_c.to(dev)
+    kn, vn = k[:, :, -q_len:].contiguous(), v[:, :, -q_len:].contiguous()
+    variants = [
+        ("h2o-default", dict()),
+        ("h2o-default", dict(grace_period=256)),
+        ("h2o-default", dict(grace_period=256, normalize_scores=True)),
+        ("h2o-vlen-default", dict(grace_period=256)),
+        ("h2o-torch-quantized8", dict(grace_period=256)),
+        ("qh2o-torch-quantized8", dict(grace_period=256)),
+        ("qh2o-vlen-torch-quantized8", dict(grace_period=256, normalize_scores=True)),
+    ]
+    table = {}
+    for name, kw in variants:
+        cache = create_kv_cache(name, KVCacheParams(B, Hkv, T, D, Hq), max_chunk_size=q_len, device=dev, **kw)
+        # prime: all T rows through the write kernel (it quantises and fills v_norm / q_errors), then the
+        # bookkeeping of a cache that has been full for a while
+        cache.batch_size, cache.current_length, cache.prefill_length = B, T, T
+        idx = torch.arange(T, dtype=torch.int32, device=dev).view(1, 1, T).expand(B, Hkv, T).contiguous()
+        cache._write(idx, k, v, 0)
+        cache.scores.copy_(torch.rand((B, Hkv, T), device=dev))
+        cache._input_pos = T
+        cache._use_initial_rule = False
+        cache.next_grace_pos = T - cache.grace_period if cache.grace_period else None
+        cache._next_index.copy_(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
+        cache._have_next = True
+        for _ in range(max(args.warmup, 2)):
+            cache.forward(q, kn, vn)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            cache.forward(q, kn, vn)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / args.steps
+        # cheap invariants of the final state
+        tp = cache.token_positions()
+        assert int(tp.max()) == cache.input_pos - 1
+        if cache.grace_period:
+            last = cache.input_pos - 1
+            ring = tp[0, 0, T - cache.grace_period:].sort().values.cpu()
+            assert torch.equal(ring, torch.arange(last - cache.grace_period + 1, last + 1, dtype=ring.dtype)), "ring lost a recent token"
+            assert int(cache._next_index.max()) < T - cache.grace_period
+        label = name + "".join(f"+{a}={b}" for a, b in kw.items())
+        table[label] = round(ms, 4)
+        del cache
+    heavy = "qh2o-vlen-torch-quantized8+grace_period=256+normalize_scores=True"
+    base = table["h2o-default"]
+    flops_alg = 4.0 * B * Hq * q_len * T * D
+    return {
+        "metric": "H2O cache chunk step with eviction-policy variants, tokens/s of the heaviest variant",
+        "value": round(q_len / (table[heavy] * 1e-3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": table[heavy],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE.json configs[1] shapes (B1 Hq32 Hkv8 D128, 32768 slots, 1024-token chunk) through the cache object, per policy",
+            "ms_per_chunk_step": table,
+            "overhead_vs_plain_h2o_ms": {kk: round(vv - base, 4) for kk, vv in table.items()},
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "whole chunk step of the heaviest variant (attention + score-sum dominate)",
+            "achieved": round(flops_alg / (table[heavy] * 1e-3) / 1e12, 2),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(flops_alg / (table[heavy] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "traffic": None,
+        },
+        "cpu_baseline": None,
+    }
+
+
 def bench_calib(args, torch, dev):
     n = 1 << 29  # bf16 elements: 1 GiB in, 1 GiB out
     src = torch.ones(n, dtype=torch.bfloat16, device=dev)
@@ -485,7 +574,7 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "calib": bench_calib}[args.workload]
+    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib}[args.workload]
     res = fn(args, torch, dev)
     print(json.dumps(res), flush=True)
 

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define KVX_VERSION 100 /* major*10000 + minor*100 + patch */
+#define KVX_VERSION 101 /* major*10000 + minor*100 + patch */
 
 enum kvx_status {
   KVX_OK = 0,
@@ -175,15 +175,33 @@ int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t*
 
 /* Write `num` new tokens into the slots chosen by the previous selection, and do the bookkeeping
  * that AttnWeightsKVCache._forward_internal does around it
- * (keys_values/kvcache/attn_weights.py:510-635 without grace period; update_token_positions
- * :214-317; DefaultKVCacheBuffers.set_slots, keys_values/kvcache/buffers.py:498-519;
- * _update_score_buffers_in_forward :679-681):
+ * (keys_values/kvcache/attn_weights.py:510-635; update_token_positions :214-317;
+ * DefaultKVCacheBuffers.set_slots, keys_values/kvcache/buffers.py:498-519;
+ * _update_score_buffers_in_forward :636-681):
  *   slot = index[b,h,j];  token_pos[b,h,slot] = input_pos + j;  scores[b,h,slot] = 0;
  *   K[b,h,slot,:] = key[b,h,j,:];  V likewise.
  * With kv_dtype == KVX_KV_U8 the rows are quantised on the way in (same arithmetic as
  * kvx_quantize_rows) into codes + k_scale/k_zp/v_scale/v_zp.
  * index: int32 (B, Hkv, index_stride_h >= num) with index_stride_b / _h in elements.
- * key/value: bf16 (B, Hkv, num, D) by strides. scores may be NULL (no score buffer). */
+ * key/value: bf16 (B, Hkv, num, D) by strides. scores may be NULL (no score buffer).
+ *
+ * Grace period (grace_num = num2 > 0; the cache is full and its last grace_period slots are a ring
+ * of the most recent tokens, keys_values/kvcache/attn_weights.py:267-303,565-606). With
+ * num1 = num - num2 and ring = grace_slots[j] (oldest ring slot first), job j does
+ *   j <  num2: everything slot `ring` holds (K/V row, quantiser state, token position
+ *              input_pos - grace_period + j, scores, v_norm, q_errors) moves to index[b,h,j];
+ *              then the new token num1 + j goes into `ring` (position input_pos + num1 + j);
+ *   j >= num2: the new token j - num2 goes into index[b,h,j] (position input_pos + j - num2).
+ * A moved row of a uint8 cache keeps its codes, scale and zero point (the reference dequantises and
+ * re-quantises it, which is not the identity). Slots in index must lie outside the ring.
+ *
+ * Further score buffers, same layout and strides as scores, NULL if the policy has none:
+ *   v_norm   |value row|_2 in fp32 (VLengthInstantScoreMixin._initial_scores_in_forward,
+ *            keys_values/kvcache/h2o.py:316-341);
+ *   q_errors |k - dq(q(k))|_2 + |v - dq(q(v))|_2 of the new row, differences rounded to bf16 and
+ *            norms in fp32 (QuantizedH2OKVCache._compute_quantization_errors,
+ *            keys_values/kvcache/qh2o.py:130-176; keys_values/kvcache/quantize/pytorch.py:530-548).
+ *            Needs KVX_KV_U8. */
 typedef struct kvx_cache_write_args {
   int32_t B, Hkv, num, D, cache_len;
   int32_t input_pos;
@@ -207,6 +225,11 @@ typedef struct kvx_cache_write_args {
   int64_t tp_stride_b, tp_stride_h;
   float* scores; /* (B, Hkv, cache_len) or NULL */
   int64_t sc_stride_b, sc_stride_h;
+  int32_t grace_num;          /* num2 <= min(num, grace_period); 0 = no ring move */
+  int32_t grace_period;
+  const int32_t* grace_slots; /* (grace_num) ring slots, shared by all (b, h) */
+  float* v_norm;              /* (B, Hkv, cache_len) by sc_stride_*, or NULL */
+  float* q_errors;            /* (B, Hkv, cache_len) by sc_stride_*, or NULL */
 } kvx_cache_write_args;
 int kvx_cache_write(const kvx_cache_write_args* args, void* stream);
 
@@ -216,11 +239,22 @@ int kvx_cache_write(const kvx_cache_write_args* args, void* stream);
  *   next_index[b,h,0..k) = the k slots of scores[b,h,:limit] with the smallest value,
  *                          in ascending (value, slot) order, ties to the lower slot.
  * This is scores.argsort(-1)[..., :k]; the reference's topk(k, largest=False, sorted=False) returns
- * the same set in unspecified order. With normalize != 0 the value compared is
+ * the same set in unspecified order. limit = cache_length - grace_period: the ring is never evicted.
+ * With normalize != 0 the value compared is
  * scores / (input_pos - max(token_pos, prefill_len - 1)) (keys_values/kvcache/h2o.py:183-196);
  * token_pos then must be given. 1 <= k <= min(limit, 4096); limit <= kv_len.
  * scores rows at scores + b*sc_stride_b + h*sc_stride_h; w contiguous (B, Hkv, kv_len).
- * next_index: int32 (B, Hkv, k) contiguous. */
+ * next_index: int32 (B, Hkv, k) contiguous.
+ *
+ * Policy variants (all pointers NULL / zero for plain H2O):
+ *   v_norm   (same layout as scores): the amount added is (v_norm*w / sum_k(v_norm*w)) * q_len in
+ *            place of w (VLengthInstantScoreMixin._instantaneous_score, keys_values/kvcache/h2o.py:297-314).
+ *   q_errors (same layout as scores): the value compared becomes
+ *            c*mm(value) + ((c-1)/2)*mm(q_errors) + (1-c), c = combination, where mm is the min-max
+ *            normalisation over all (head, slot < limit) entries of one batch element
+ *            (QuantizedH2OKVCache._modify_scores, keys_values/kvcache/qh2o.py:178-210).
+ * With a variant the workspace also holds per-row statistics (kvx_h2o_workspace_bytes accounts for
+ * them) and kvx_sdpa_decode_h2o is not available. */
 typedef struct kvx_h2o_args {
   int32_t B, Hkv, kv_len, limit, k;
   int32_t normalize, input_pos, prefill_len;
@@ -232,6 +266,10 @@ typedef struct kvx_h2o_args {
   int32_t* next_index;
   void* workspace;
   size_t workspace_bytes;
+  const float* v_norm;   /* or NULL */
+  const float* q_errors; /* or NULL */
+  int32_t q_len;         /* queries behind w (v_norm only) */
+  double combination;    /* c in [0, 1] (q_errors only); a double, as the reference's Python float */
 } kvx_h2o_args;
 int kvx_h2o_update_select(const kvx_h2o_args* args, void* stream);
 size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* args);

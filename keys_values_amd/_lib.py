@@ -45,6 +45,8 @@ class CacheWriteArgs(ctypes.Structure):
         ("qs_stride_b", c_int64), ("qs_stride_h", c_int64),
         ("token_pos", c_void_p), ("tp_stride_b", c_int64), ("tp_stride_h", c_int64),
         ("scores", c_void_p), ("sc_stride_b", c_int64), ("sc_stride_h", c_int64),
+        ("grace_num", c_int32), ("grace_period", c_int32), ("grace_slots", c_void_p),
+        ("v_norm", c_void_p), ("q_errors", c_void_p),
     ]
 
 
@@ -59,6 +61,7 @@ class H2OArgs(ctypes.Structure):
         ("token_pos", c_void_p), ("tp_stride_b", c_int64), ("tp_stride_h", c_int64),
         ("next_index", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("v_norm", c_void_p), ("q_errors", c_void_p), ("q_len", c_int32), ("combination", ctypes.c_double),
     ]
 
 

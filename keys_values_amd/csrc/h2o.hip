@@ -18,8 +18,6 @@
 namespace kvx {
 namespace {
 
-constexpr int SEL_THREADS = 1024;
-constexpr int MAX_K = 4096;
 
 // Monotone map float -> uint32 (a < b  <=>  key(a) < key(b)); -0.0 is folded onto +0.0 first, as
 // comparisons treat them as equal.
@@ -31,10 +29,135 @@ __device__ __forceinline__ uint32_t ordered_bits(float x) {
 
 // Value the selection compares: the score, or the score divided by the slot's residency
 // (keys_values/kvcache/h2o.py:183-196).
-__device__ __forceinline__ float select_value(float score, const kvx_h2o_args& a, const int32_t* tp_row, int idx) {
+__device__ __forceinline__ float residency_value(float score, const kvx_h2o_args& a, const int32_t* tp_row, int idx) {
   if (!a.normalize) return score;
   const int t = max(tp_row[idx], a.prefill_len - 1);
   return score / (float)(a.input_pos - t);
+}
+
+// Q-Hitter combination (keys_values/kvcache/qh2o.py:178-210): both terms are min-max normalised over
+// all (head, slot < limit) entries of the batch element, then c*s + ((c-1)/2)*q + (1-c). Each
+// product and sum is rounded on its own, as the reference's tensor expression is.
+struct Modify {
+  const float* qe;  // q_errors row, or nullptr: no modification
+  float smin, sden, qmin, qden;
+  float c, c2, c3;
+};
+
+// stats: 4 floats per (batch, head) row = min / max of the compared value and of q_errors.
+__device__ __forceinline__ Modify load_modify(const kvx_h2o_args& a, const float* stats, int b, int hh) {
+  Modify m;
+  m.qe = nullptr;
+  if (!stats) return m;
+  m.qe = a.q_errors + b * a.sc_stride_b + hh * a.sc_stride_h;
+  float smin = INFINITY, smax = -INFINITY, qmin = INFINITY, qmax = -INFINITY;
+  for (int h = 0; h < a.Hkv; ++h) {
+    const f32x4_t st = *(const f32x4_t*)(stats + ((int64_t)b * a.Hkv + h) * 4);
+    smin = fminf(smin, st[0]);
+    smax = fmaxf(smax, st[1]);
+    qmin = fminf(qmin, st[2]);
+    qmax = fmaxf(qmax, st[3]);
+  }
+  m.smin = smin;
+  m.sden = smax - smin;
+  m.qmin = qmin;
+  m.qden = qmax - qmin;
+  m.c = (float)a.combination;
+  m.c2 = (float)((a.combination - 1.0) / 2.0);
+  m.c3 = (float)(1.0 - a.combination);
+  return m;
+}
+
+__device__ __forceinline__ float select_value(float score, const kvx_h2o_args& a, const int32_t* tp_row, int idx, const Modify& m) {
+  float v = residency_value(score, a, tp_row, idx);
+  if (m.qe) {
+    const float s = (v - m.smin) / m.sden;
+    const float q = (m.qe[idx] - m.qmin) / m.qden;
+    v = __fadd_rn(__fadd_rn(__fmul_rn(m.c, s), __fmul_rn(m.c2, q)), m.c3);
+  }
+  return v;
+}
+
+// ---- policy variants: the accumulation pass ---------------------------------------------------
+
+constexpr int SEL_THREADS = 1024;
+
+// Deterministic workgroup reductions (wavefront butterfly, then the 16 partials in a fixed order).
+template <typename Op>
+__device__ __forceinline__ float block_reduce(float v, float* red, Op op) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+  __syncthreads();  // red may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < SEL_THREADS / 64; ++i) r = op(r, red[i]);
+  return r;
+}
+
+// One workgroup per (batch, head) row: scores += instantaneous score, where the latter is w or,
+// with v_norm, (v_norm*w / sum(v_norm*w)) * q_len (keys_values/kvcache/h2o.py:297-314); and the row's
+// min / max of the compared value and of q_errors over the slots below limit, for the combination.
+__global__ __launch_bounds__(SEL_THREADS) void accumulate_kernel(const kvx_h2o_args a, float* __restrict__ stats) {
+  __shared__ float red[SEL_THREADS / 64];
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x;
+  const int b = row / a.Hkv, hh = row % a.Hkv;
+  const int64_t off = b * a.sc_stride_b + hh * a.sc_stride_h;
+  float* sc = a.scores + off;
+  const float* w = a.w ? a.w + (int64_t)row * a.kv_len : nullptr;
+  const float* vn = a.v_norm ? a.v_norm + off : nullptr;
+  const float* qe = a.q_errors ? a.q_errors + off : nullptr;
+  const int32_t* tpr = a.token_pos ? a.token_pos + b * a.tp_stride_b + hh * a.tp_stride_h : nullptr;
+  float z = 1.0f;
+  if (w && vn) {
+    float part = 0.0f;
+    for (int i = tid; i < a.kv_len; i += SEL_THREADS) part += vn[i] * w[i];
+    z = block_reduce(part, red, [](float x, float y) { return x + y; });
+  }
+  const float ql = (float)a.q_len;
+  float smin = INFINITY, smax = -INFINITY, qmin = INFINITY, qmax = -INFINITY;
+  constexpr int PB = 4;
+  for (int i0 = tid; i0 < a.kv_len; i0 += PB * SEL_THREADS) {
+    float sv[PB], wv[PB], nv[PB], qv[PB];
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {  // all loads of the batch before the first store (sc may alias for all the compiler knows)
+      const int i = i0 + j * SEL_THREADS;
+      const bool in = i < a.kv_len;
+      sv[j] = in ? sc[i] : 0.0f;
+      wv[j] = (in && w) ? w[i] : 0.0f;
+      nv[j] = (in && w && vn) ? vn[i] : 0.0f;
+      qv[j] = (qe && i < a.limit) ? qe[i] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+      const int i = i0 + j * SEL_THREADS;
+      if (i >= a.kv_len) break;
+      float v = sv[j];
+      if (w) {
+        float inst = wv[j];
+        if (vn) inst = __fmul_rn(__fmul_rn(nv[j], wv[j]) / z, ql);
+        v = __fadd_rn(v, inst);
+        sc[i] = v;
+      }
+      if (qe && i < a.limit) {
+        const float cv = residency_value(v, a, tpr, i);
+        smin = fminf(smin, cv);
+        smax = fmaxf(smax, cv);
+        qmin = fminf(qmin, qv[j]);
+        qmax = fmaxf(qmax, qv[j]);
+      }
+    }
+  }
+  if (qe) {
+    auto mn = [](float x, float y) { return fminf(x, y); };
+    auto mx = [](float x, float y) { return fmaxf(x, y); };
+    smin = block_reduce(smin, red, mn);
+    smax = block_reduce(smax, red, mx);
+    qmin = block_reduce(qmin, red, mn);
+    qmax = block_reduce(qmax, red, mx);
+    if (tid == 0) *(f32x4_t*)(stats + (int64_t)row * 4) = f32x4_t{smin, smax, qmin, qmax};
+  }
 }
 
 // ---- k == 1 ---------------------------------------------------------------------------------
@@ -44,9 +167,10 @@ __global__ void argmin_init_kernel(unsigned long long* best, int rows) {
   if (i < rows) best[i] = ~0ull;
 }
 
-__global__ __launch_bounds__(256) void update_argmin_kernel(const kvx_h2o_args a, unsigned long long* best) {
+__global__ __launch_bounds__(256) void update_argmin_kernel(const kvx_h2o_args a, unsigned long long* best, const float* stats) {
   const int row = blockIdx.y;
   const int b = row / a.Hkv, hh = row % a.Hkv;
+  const Modify md = load_modify(a, stats, b, hh);
   float* sc = a.scores + b * a.sc_stride_b + hh * a.sc_stride_h;
   const float* w = a.w ? a.w + (int64_t)row * a.kv_len : nullptr;
   const int32_t* tpr = a.token_pos ? a.token_pos + b * a.tp_stride_b + hh * a.tp_stride_h : nullptr;
@@ -66,7 +190,7 @@ __global__ __launch_bounds__(256) void update_argmin_kernel(const kvx_h2o_args a
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (i0 + e < a.limit) {
-          const unsigned long long key = ((unsigned long long)ordered_bits(select_value(s[e], a, tpr, i0 + e)) << 32) | (unsigned)(i0 + e);
+          const unsigned long long key = ((unsigned long long)ordered_bits(select_value(s[e], a, tpr, i0 + e, md)) << 32) | (unsigned)(i0 + e);
           mine = key < mine ? key : mine;
         }
     } else {
@@ -79,7 +203,7 @@ __global__ __launch_bounds__(256) void update_argmin_kernel(const kvx_h2o_args a
           sc[i] = s;
         }
         if (i < a.limit) {
-          const unsigned long long key = ((unsigned long long)ordered_bits(select_value(s, a, tpr, i)) << 32) | (unsigned)i;
+          const unsigned long long key = ((unsigned long long)ordered_bits(select_value(s, a, tpr, i, md)) << 32) | (unsigned)i;
           mine = key < mine ? key : mine;
         }
       }
@@ -110,7 +234,7 @@ __global__ void argmin_finish_kernel(const unsigned long long* best, int32_t* ne
 // CACHED: the row's ordered keys live in LDS after the first pass (rows of up to ~36K slots), so the
 // radix passes and the gather never go back to global memory.
 template <bool CACHED>
-__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a, int kpad) {
+__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a, int kpad, const float* stats) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   unsigned long long* cand = (unsigned long long*)dyn_lds;    // kpad entries
   uint32_t* keys = (uint32_t*)(dyn_lds + (size_t)kpad * 8);   // a.limit entries (CACHED only)
@@ -125,6 +249,7 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   float* sc = a.scores + b * a.sc_stride_b + hh * a.sc_stride_h;
   const float* w = a.w ? a.w + (int64_t)row * a.kv_len : nullptr;
   const int32_t* tpr = a.token_pos ? a.token_pos + b * a.tp_stride_b + hh * a.tp_stride_h : nullptr;
+  const Modify md = load_modify(a, stats, b, hh);
 
   // pass 0: scores += w (every later pass of this thread touches the slots it wrote here) and the keys
   // One workgroup walks the whole row: batches of 8 loads per array are issued before anything is
@@ -149,12 +274,12 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
         v += wv[j];
         sc[i] = v;
       }
-      if (CACHED && i < a.limit) keys[i] = ordered_bits(select_value(v, a, tpr, i));
+      if (CACHED && i < a.limit) keys[i] = ordered_bits(select_value(v, a, tpr, i, md));
     }
   }
   auto key_of = [&](int i) -> uint32_t {
     if constexpr (CACHED) return keys[i];
-    else return ordered_bits(select_value(sc[i], a, tpr, i));
+    else return ordered_bits(select_value(sc[i], a, tpr, i, md));
   };
 
   for (int i = tid; i < kpad; i += SEL_THREADS) cand[i] = ~0ull;
@@ -292,18 +417,32 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
 
 }  // namespace
 
-size_t h2o_workspace(const kvx_h2o_args& a) { return a.k == 1 ? (size_t)a.B * a.Hkv * sizeof(unsigned long long) : 0; }
+static bool is_variant(const kvx_h2o_args& a) { return a.v_norm != nullptr || a.q_errors != nullptr; }
+static size_t best_bytes(const kvx_h2o_args& a) { return a.k == 1 ? ((size_t)a.B * a.Hkv * sizeof(unsigned long long) + 15) / 16 * 16 : 0; }
 
-int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st) {
+size_t h2o_workspace(const kvx_h2o_args& a) { return best_bytes(a) + (a.q_errors ? (size_t)a.B * a.Hkv * 4 * sizeof(float) : 0); }
+
+int launch_h2o_update_select(const kvx_h2o_args& a_in, hipStream_t st) {
+  kvx_h2o_args a = a_in;
   const int rows = a.B * a.Hkv;
   if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(h2o_workspace(a) == 0 || (a.workspace && a.workspace_bytes >= h2o_workspace(a)), KVX_ERR_WORKSPACE,
+              "kvx_h2o_update_select: workspace of %zu bytes needed", h2o_workspace(a));
+  float* stats = nullptr;
+  if (is_variant(a)) {
+    // the accumulation (and the batch statistics of the combination) first; what follows only selects
+    if (a.q_errors) stats = (float*)((char*)a.workspace + best_bytes(a));
+    if (a.w || stats) {
+      hipLaunchKernelGGL(accumulate_kernel, dim3(rows), dim3(SEL_THREADS), 0, st, a, stats);
+      KVX_HIP(hipGetLastError());
+    }
+    a.w = nullptr;
+  }
   if (a.k == 1) {
-    KVX_REQUIRE(a.workspace && a.workspace_bytes >= h2o_workspace(a), KVX_ERR_WORKSPACE,
-                "kvx_h2o_update_select: workspace of %zu bytes needed", h2o_workspace(a));
     unsigned long long* best = (unsigned long long*)a.workspace;
     hipLaunchKernelGGL(argmin_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, rows);
     KVX_HIP(hipGetLastError());
-    hipLaunchKernelGGL(update_argmin_kernel, dim3((a.kv_len + 4095) / 4096, rows), dim3(256), 0, st, a, best);
+    hipLaunchKernelGGL(update_argmin_kernel, dim3((a.kv_len + 4095) / 4096, rows), dim3(256), 0, st, a, best, (const float*)stats);
     KVX_HIP(hipGetLastError());
     hipLaunchKernelGGL(argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, best, a.next_index, rows);
     KVX_HIP(hipGetLastError());
@@ -317,9 +456,9 @@ int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st) {
   if (cached_bytes <= kDynLimit) {
     if (cached_bytes > 48 * 1024)  // beyond the default dynamic LDS allowance (the setting is per device and kernel)
       KVX_HIP(hipFuncSetAttribute((const void*)update_select_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLimit));
-    hipLaunchKernelGGL(update_select_kernel<true>, dim3(rows), dim3(SEL_THREADS), cached_bytes, st, a, kpad);
+    hipLaunchKernelGGL(update_select_kernel<true>, dim3(rows), dim3(SEL_THREADS), cached_bytes, st, a, kpad, (const float*)stats);
   } else {
-    hipLaunchKernelGGL(update_select_kernel<false>, dim3(rows), dim3(SEL_THREADS), (size_t)kpad * 8, st, a, kpad);
+    hipLaunchKernelGGL(update_select_kernel<false>, dim3(rows), dim3(SEL_THREADS), (size_t)kpad * 8, st, a, kpad, (const float*)stats);
   }
   KVX_HIP(hipGetLastError());
   return KVX_OK;

@@ -201,6 +201,14 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   if (a->kv_dtype == KVX_KV_U8)
     KVX_REQUIRE(a->k_scale && a->k_zp && a->v_scale && a->v_zp, KVX_ERR_INVALID, "kvx_cache_write: uint8 cache needs scale / zero-point arrays");
   KVX_REQUIRE((int64_t)a->input_pos + a->num < INT32_MAX && a->input_pos >= 0, KVX_ERR_INVALID, "kvx_cache_write: bad input_pos");
+  KVX_REQUIRE(a->grace_num >= 0 && a->grace_num <= a->num, KVX_ERR_INVALID, "kvx_cache_write: grace_num=%d must be in [0, num=%d]", a->grace_num, a->num);
+  if (a->grace_num > 0) {
+    KVX_REQUIRE(a->grace_slots, KVX_ERR_INVALID, "kvx_cache_write: grace_num > 0 needs grace_slots");
+    KVX_REQUIRE(a->grace_num <= a->grace_period && a->grace_period < a->cache_len && a->input_pos >= a->grace_period, KVX_ERR_INVALID,
+                "kvx_cache_write: need grace_num=%d <= grace_period=%d < cache_len=%d and input_pos=%d >= grace_period", a->grace_num,
+                a->grace_period, a->cache_len, a->input_pos);
+  }
+  KVX_REQUIRE(!a->q_errors || a->kv_dtype == KVX_KV_U8, KVX_ERR_INVALID, "kvx_cache_write: q_errors needs the uint8 cache");
   return launch_cache_write(*a, (hipStream_t)stream);
 }
 
@@ -213,6 +221,9 @@ static int check_h2o(const kvx_h2o_args* a, const char* who) {
   KVX_REQUIRE(a->k >= 1 && a->k <= a->limit && a->k <= 4096, KVX_ERR_INVALID, "%s: k=%d must be in [1, min(limit, 4096)]", who, a->k);
   KVX_REQUIRE(a->scores && a->next_index, KVX_ERR_INVALID, "%s: NULL pointer", who);
   KVX_REQUIRE(!a->normalize || a->token_pos, KVX_ERR_INVALID, "%s: normalize needs token_pos", who);
+  KVX_REQUIRE(!(a->v_norm && a->w) || a->q_len > 0, KVX_ERR_INVALID, "%s: v_norm needs q_len > 0", who);
+  KVX_REQUIRE(!a->q_errors || (a->combination >= 0.0 && a->combination <= 1.0), KVX_ERR_INVALID,
+              "%s: combination = %g, must be in [0, 1]", who, a->combination);
   return KVX_OK;
 }
 
@@ -230,6 +241,8 @@ int kvx_sdpa_decode_h2o(const kvx_sdpa_args* a, const kvx_h2o_args* h, void* str
   KVX_REQUIRE(a->q_len == 1, KVX_ERR_INVALID, "kvx_sdpa_decode_h2o: q_len must be 1, got %d", a->q_len);
   const int G = a->Hq / a->Hkv;
   KVX_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode_h2o: group size %d not in {1, 2, 4, 8}", G);
+  KVX_REQUIRE(!h->v_norm && !h->q_errors, KVX_ERR_UNSUPPORTED,
+              "kvx_sdpa_decode_h2o: v_norm / q_errors policies take kvx_sdpa_decode + kvx_h2o_update_select");
   KVX_REQUIRE(h->k == 1 && h->kv_len == a->kv_len && h->B == a->B && h->Hkv == a->Hkv, KVX_ERR_INVALID,
               "kvx_sdpa_decode_h2o: needs k == 1 and the cache shape of the attention call");
   KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_decode_h2o: workspace must be 16-byte aligned");

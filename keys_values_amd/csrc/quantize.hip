@@ -127,7 +127,52 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t
   }
 }
 
-// One lane per 8 elements of one new (b, h, j) row, for K and V.
+// Sum over the LPR adjacent lanes holding one row; every lane gets the result.
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+  if constexpr (LPR == 16)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+  return v;
+}
+
+// |row|_2 of a bf16 row spread over LPR lanes, accumulated in fp32.
+template <int LPR>
+__device__ __forceinline__ float row_norm(u32x4_t raw) {
+  float ss = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float a = bf16_lo(raw[e]), b = bf16_hi(raw[e]);
+    ss += a * a;
+    ss += b * b;
+  }
+  return sqrtf(row_sum<LPR>(ss));
+}
+
+// |x - dq(q(x))|_2 of a row: the dequantised value and the difference are rounded to bf16, the norm
+// accumulates in fp32 (keys_values/kvcache/quantize/pytorch.py:530-548).
+template <int LPR>
+__device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, float scale, int32_t zp) {
+  float ss = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t cw = codes[e >> 1];
+    const int sh = (e & 1) * 16;
+    const uint32_t dq = dequant_pair((cw >> sh) & 0xff, (cw >> (sh + 8)) & 0xff, zp, scale);
+    const uint32_t diff = pack_bf16(bf16_lo(raw[e]) - bf16_lo(dq), bf16_hi(raw[e]) - bf16_hi(dq));
+    const float a = bf16_lo(diff), b = bf16_hi(diff);
+    ss += a * a;
+    ss += b * b;
+  }
+  return sqrtf(row_sum<LPR>(ss));
+}
+
+// One lane per 8 elements of one job (b, h, j), for K and V. Without a ring move job j writes new
+// token j into index[b,h,j]. With one (j < grace_num) the lane first carries its 8 elements of ring
+// slot grace_slots[j] over to index[b,h,j], then writes new token num - grace_num + j into the ring
+// slot: the read and the write of that slot are issued by the same lane, in this order.
 template <int D, bool U8>
 __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
   constexpr int LPR = D / 8;
@@ -141,36 +186,75 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   const int hh = (int)((ridc / a.num) % a.Hkv);
   const int b = (int)(ridc / ((int64_t)a.num * a.Hkv));
   const int slot = a.index[b * a.index_stride_b + hh * a.index_stride_h + j];
-  const bool ok = live && slot >= 0 && slot < a.cache_len;  // a bad index is dropped, never written out of bounds
-  const uint16_t* ks = (const uint16_t*)a.key + b * a.key_stride_b + hh * a.key_stride_h + (int64_t)j * a.key_stride_t + col * 8;
-  const uint16_t* vs = (const uint16_t*)a.value + b * a.value_stride_b + hh * a.value_stride_h + (int64_t)j * a.value_stride_t + col * 8;
+  const bool moves = j < a.grace_num;
+  const int ring = moves ? a.grace_slots[j] : -1;
+  const int src = moves ? a.num - a.grace_num + j : j - a.grace_num;  // new token this job stores
+  // a bad index is dropped, never written out of bounds
+  const bool ok = live && slot >= 0 && slot < a.cache_len && (!moves || (ring >= 0 && ring < a.cache_len && ring != slot));
+  const int wslot = moves ? ring : slot;  // where the new token goes
+  const uint16_t* ks = (const uint16_t*)a.key + b * a.key_stride_b + hh * a.key_stride_h + (int64_t)src * a.key_stride_t + col * 8;
+  const uint16_t* vs = (const uint16_t*)a.value + b * a.value_stride_b + hh * a.value_stride_h + (int64_t)src * a.value_stride_t + col * 8;
   const u32x4_t kr = live ? *(const u32x4_t*)ks : u32x4_t{0, 0, 0, 0};
   const u32x4_t vr = live ? *(const u32x4_t*)vs : u32x4_t{0, 0, 0, 0};
+  const int64_t tp_row = b * a.tp_stride_b + hh * a.tp_stride_h;
+  const int64_t sc_row = b * a.sc_stride_b + hh * a.sc_stride_h;
+  const int64_t qs_row = b * a.qs_stride_b + hh * a.qs_stride_h;
+  constexpr int ES = U8 ? 1 : 2;  // bytes per cache element
+  uint8_t* kc_row = (uint8_t*)a.k_cache + (b * a.kc_stride_b + hh * a.kc_stride_h) * ES + col * 8 * ES;
+  uint8_t* vc_row = (uint8_t*)a.v_cache + (b * a.vc_stride_b + hh * a.vc_stride_h) * ES + col * 8 * ES;
+
+  if (ok && moves) {
+    if constexpr (!U8) {
+      *(u32x4_t*)(kc_row + (int64_t)slot * a.kc_stride_t * ES) = *(const u32x4_t*)(kc_row + (int64_t)ring * a.kc_stride_t * ES);
+      *(u32x4_t*)(vc_row + (int64_t)slot * a.vc_stride_t * ES) = *(const u32x4_t*)(vc_row + (int64_t)ring * a.vc_stride_t * ES);
+    } else {
+      *(u32x2_t*)(kc_row + (int64_t)slot * a.kc_stride_t) = *(const u32x2_t*)(kc_row + (int64_t)ring * a.kc_stride_t);
+      *(u32x2_t*)(vc_row + (int64_t)slot * a.vc_stride_t) = *(const u32x2_t*)(vc_row + (int64_t)ring * a.vc_stride_t);
+      if (col == 0) {
+        a.k_scale[qs_row + slot] = a.k_scale[qs_row + ring];
+        a.k_zp[qs_row + slot] = a.k_zp[qs_row + ring];
+        a.v_scale[qs_row + slot] = a.v_scale[qs_row + ring];
+        a.v_zp[qs_row + slot] = a.v_zp[qs_row + ring];
+      }
+    }
+    if (col == 0) {
+      a.token_pos[tp_row + slot] = a.input_pos - a.grace_period + j;
+      if (a.scores) a.scores[sc_row + slot] = a.scores[sc_row + ring];
+      if (a.v_norm) a.v_norm[sc_row + slot] = a.v_norm[sc_row + ring];
+      if (a.q_errors) a.q_errors[sc_row + slot] = a.q_errors[sc_row + ring];
+    }
+  }
+
+  float qerr = 0.0f;
   if constexpr (!U8) {
     if (ok) {
-      *(u32x4_t*)((uint16_t*)a.k_cache + b * a.kc_stride_b + hh * a.kc_stride_h + (int64_t)slot * a.kc_stride_t + col * 8) = kr;
-      *(u32x4_t*)((uint16_t*)a.v_cache + b * a.vc_stride_b + hh * a.vc_stride_h + (int64_t)slot * a.vc_stride_t + col * 8) = vr;
+      *(u32x4_t*)(kc_row + (int64_t)wslot * a.kc_stride_t * ES) = kr;
+      *(u32x4_t*)(vc_row + (int64_t)wslot * a.vc_stride_t * ES) = vr;
     }
   } else {
     float s1, s2;
     int32_t z1, z2;
     const u32x2_t kc = quantize8<LPR>(kr, s1, z1);
     const u32x2_t vc = quantize8<LPR>(vr, s2, z2);
+    if (a.q_errors) qerr = row_quant_error<LPR>(kr, kc, s1, z1) + row_quant_error<LPR>(vr, vc, s2, z2);  // uniform branch
     if (ok) {
-      *(u32x2_t*)((uint8_t*)a.k_cache + b * a.kc_stride_b + hh * a.kc_stride_h + (int64_t)slot * a.kc_stride_t + col * 8) = kc;
-      *(u32x2_t*)((uint8_t*)a.v_cache + b * a.vc_stride_b + hh * a.vc_stride_h + (int64_t)slot * a.vc_stride_t + col * 8) = vc;
+      *(u32x2_t*)(kc_row + (int64_t)wslot * a.kc_stride_t) = kc;
+      *(u32x2_t*)(vc_row + (int64_t)wslot * a.vc_stride_t) = vc;
       if (col == 0) {
-        const int64_t so = b * a.qs_stride_b + hh * a.qs_stride_h + slot;
-        a.k_scale[so] = s1;
-        a.k_zp[so] = z1;
-        a.v_scale[so] = s2;
-        a.v_zp[so] = z2;
+        a.k_scale[qs_row + wslot] = s1;
+        a.k_zp[qs_row + wslot] = z1;
+        a.v_scale[qs_row + wslot] = s2;
+        a.v_zp[qs_row + wslot] = z2;
       }
     }
   }
+  float vnorm = 0.0f;
+  if (a.v_norm) vnorm = row_norm<LPR>(vr);  // uniform branch: every lane takes part in the reduction
   if (ok && col == 0) {
-    a.token_pos[b * a.tp_stride_b + hh * a.tp_stride_h + slot] = a.input_pos + j;
-    if (a.scores) a.scores[b * a.sc_stride_b + hh * a.sc_stride_h + slot] = 0.0f;
+    a.token_pos[tp_row + wslot] = a.input_pos + src;
+    if (a.scores) a.scores[sc_row + wslot] = 0.0f;
+    if (a.v_norm) a.v_norm[sc_row + wslot] = vnorm;
+    if (a.q_errors) a.q_errors[sc_row + wslot] = qerr;
   }
 }
 

@@ -16,7 +16,14 @@ resident and the attention kernels dequantise them on load; the reference instea
 whole cache into a bf16 working buffer per layer and re-quantises it afterwards
 (keys_values/kvcache/quant_buffers.py:473-503,732-804).
 
-Not covered (raises): grace period, replay log, fp16/fp32 caches.
+Policy variants on the same kernels: a grace period (the last ``grace_period`` slots are a ring of
+the most recent tokens, never evicted; keys_values/kvcache/attn_weights.py:267-303,565-606), the
+V-norm weighted instantaneous score (``VLengthH2OKVCache``, keys_values/kvcache/h2o.py:266-420) and
+the Q-Hitter combination with the quantisation error (``QuantizedH2OKVCache`` /
+``QuantizedVLengthH2OKVCache``, keys_values/kvcache/qh2o.py). ``create_kv_cache`` takes the names of
+keys_values/kvcache/factory.py:50-66.
+
+Not covered (raises): replay log, fp16/fp32 caches, 4-bit and bitsandbytes stores.
 """
 import ctypes
 from dataclasses import dataclass
@@ -28,6 +35,7 @@ from .. import _lib
 from ..attention import ops
 
 DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
+DEFAULT_COMBINATION_CONSTANT = 0.5  # keys_values/kvcache/qh2o.py:25
 MAX_SELECT = 4096  # largest k of kvx_h2o_update_select
 
 
@@ -53,9 +61,16 @@ class H2OKVCache:
         quantized: bool = False,
         keep_initial_fraction: float = DEFAULT_KEEP_INITIAL_FRACTION,
         device: Optional[torch.device] = None,
+        v_length: bool = False,
+        q_hitter: bool = False,
+        combination_constant: float = DEFAULT_COMBINATION_CONSTANT,
     ):
-        if grace_period != 0:
-            raise NotImplementedError("grace_period > 0 is not implemented")
+        if not (0 <= grace_period < params.cache_length):  # keys_values/kvcache/attn_weights.py:440-444
+            raise ValueError(f"grace_period = {grace_period}, must be in [0, {params.cache_length})")
+        if q_hitter and not quantized:  # keys_values/kvcache/qh2o.py:95-96
+            raise TypeError("the quantisation-error policy needs the quantised store")
+        if not (0 <= combination_constant <= 1):  # keys_values/kvcache/qh2o.py:97-100
+            raise ValueError(f"combination_constant = {combination_constant}, must be in [0, 1]")
         if params.dtype not in (None, torch.bfloat16):
             raise NotImplementedError(f"cache dtype {params.dtype}: the kernels take bfloat16")
         if params.head_size not in (64, 128):
@@ -69,14 +84,19 @@ class H2OKVCache:
         self.cache_length = params.cache_length
         self.head_size = params.head_size
         self.dtype = torch.bfloat16
-        self.grace_period = 0
+        self.grace_period = grace_period
+        self.next_grace_pos = None
+        self.v_length = v_length
+        self.q_hitter = q_hitter
+        self.combination_constant = combination_constant
         self.normalize_scores = normalize_scores
         self.quantized = quantized
         # keys_values/kvcache/attn_weights.py:458-462: silently disabled when too large
         if max_chunk_size is not None and max_chunk_size > self.cache_length // 2:
             max_chunk_size = None
         self.max_chunk_size = max_chunk_size
-        self._select_k = min(self.cache_length, MAX_SELECT) if max_chunk_size is None else min(max_chunk_size, MAX_SELECT)
+        limit = self.cache_length - grace_period
+        self._select_k = min(limit, MAX_SELECT) if max_chunk_size is None else min(max_chunk_size, limit, MAX_SELECT)
         self._keep_initial_fraction = keep_initial_fraction
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         if self.device.type != "cuda":
@@ -92,6 +112,12 @@ class H2OKVCache:
             self.v_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
         self.token_pos = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)  # attn_weights.py:466-470
         self.scores = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)  # h2o.py:85-91
+        # further score buffers, moved and initialised with the slots (h2o.py:405-413, qh2o.py:107-113)
+        self.v_norm = torch.zeros((b, h, length), dtype=torch.float32, device=self.device) if v_length else None
+        self.q_errors = torch.zeros((b, h, length), dtype=torch.float32, device=self.device) if q_hitter else None
+        if grace_period > 0:  # the ring twice over: any wrap-around run of up to grace_period slots is one view of it
+            ring = torch.arange(length - grace_period, length, dtype=torch.int32, device=self.device)
+            self._ring_twice = torch.cat((ring, ring))
         self._next_index = torch.zeros((b, h, self._select_k), dtype=torch.int32, device=self.device)
         self._have_next = False
         self._use_initial_rule = None
@@ -114,7 +140,7 @@ class H2OKVCache:
     def max_forward_length(self) -> int:
         """keys_values/kvcache/attn_weights.py:501-508."""
         diff = self.cache_length - self.current_length
-        result = self.cache_length
+        result = self.cache_length - self.grace_period
         if diff > 0:
             result = min(result, diff)
         if self.max_chunk_size is not None:
@@ -215,8 +241,13 @@ class H2OKVCache:
         self.batch_size = b
         index = torch.arange(num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, self.n_query_groups, -1).contiguous()
         self.scores.zero_()
+        for extra in (self.v_norm, self.q_errors):
+            if extra is not None:
+                extra.zero_()
         self.current_length = num
         self._write(index, key, value, 0)
+        if self.grace_period > 0:  # first slot to move out once the cache is full, attn_weights.py:861-863
+            self.next_grace_pos = self.cache_length - self.grace_period
         self.prefill_length = num
         self._use_initial_rule = num == self.cache_length
         self._have_next = False
@@ -255,13 +286,26 @@ class H2OKVCache:
         a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
         a.scores = self.scores.data_ptr()
         a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
+        a.v_norm, a.q_errors = _lib.ptr(self.v_norm), _lib.ptr(self.q_errors)
+        ring = None
+        if self.grace_period > 0 and input_pos >= self.cache_length:
+            # keys_values/kvcache/attn_weights.py:267-303: the num2 oldest ring slots move out to
+            # `index` and take the last num2 new tokens; wrap-around run starting at next_grace_pos
+            gp = self.grace_period
+            prefix = self.cache_length - gp
+            num2 = min(num, gp)
+            start = self.next_grace_pos - prefix
+            ring = self._ring_twice[start : start + num2]
+            a.grace_num, a.grace_period, a.grace_slots = num2, gp, ring.data_ptr()
+            if num <= gp:  # attn_weights.py:601-606
+                self.next_grace_pos = (self.next_grace_pos - prefix + num) % gp + prefix
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
 
     def _h2o_args(self, full: bool) -> _lib.H2OArgs:
         a = _lib.H2OArgs()
         a.B, a.Hkv, a.kv_len = self.batch_size, self.n_query_groups, self.current_length
-        a.limit = self.current_length
+        a.limit = self.cache_length - self.grace_period if full else self.current_length
         a.k = self._select_k if full else 1
         a.normalize = int(self.normalize_scores and full)
         a.input_pos = self._input_pos
@@ -270,12 +314,15 @@ class H2OKVCache:
         a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
         a.token_pos = self.token_pos.data_ptr()
         a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
+        a.v_norm = _lib.ptr(self.v_norm)
+        a.q_errors = _lib.ptr(self.q_errors) if full else None  # only the selection reads them
+        a.combination = self.combination_constant
         return a
 
     def _decode_h2o_step(self, query, kc, vc, quant) -> torch.Tensor:
         """``self.mha(...)`` and ``self._update(...)`` of keys_values/kvcache/base.py:583-595 for one new
         token and a full cache, as the single fused call ``kvx_sdpa_decode_h2o`` (selection size 1)."""
-        if self._select_k != 1:
+        if self._select_k != 1 or self.v_length or self.q_hitter:
             out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
             self._update(w, 1)
             return out
@@ -329,6 +376,7 @@ class H2OKVCache:
         full = self.current_length == self.cache_length
         a = self._h2o_args(full)
         a.w = attn_weights.data_ptr()
+        a.q_len = query_length
         lib = _lib.load()
         with torch.cuda.device(self.device):
             if full:
@@ -342,3 +390,45 @@ class H2OKVCache:
             a.workspace_bytes = 0 if ws is None else ws.numel()
             _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
         self._have_next = full
+
+
+class VLengthH2OKVCache(H2OKVCache):
+    """keys_values/kvcache/h2o.py:344-420: the instantaneous score is the attention weight times the
+    norm of the slot's V row, normalised to sum to the number of queries."""
+
+    def __init__(self, params: KVCacheParams, **kwargs):
+        super().__init__(params, v_length=True, **kwargs)
+
+
+class QuantizedH2OKVCache(H2OKVCache):
+    """keys_values/kvcache/qh2o.py:31-230: H2O scores and quantisation errors, both min-max
+    normalised per batch element, in a convex combination. Quantised store only."""
+
+    def __init__(self, params: KVCacheParams, **kwargs):
+        kwargs.setdefault("quantized", True)
+        super().__init__(params, q_hitter=True, **kwargs)
+
+
+class QuantizedVLengthH2OKVCache(H2OKVCache):
+    """keys_values/kvcache/qh2o.py:233-330."""
+
+    def __init__(self, params: KVCacheParams, **kwargs):
+        kwargs.setdefault("quantized", True)
+        super().__init__(params, q_hitter=True, v_length=True, **kwargs)
+
+
+_CACHE_TYPES = {"h2o": H2OKVCache, "h2o-vlen": VLengthH2OKVCache, "qh2o": QuantizedH2OKVCache, "qh2o-vlen": QuantizedVLengthH2OKVCache}
+_STORES = {"default": False, "torch-quantized8": True}
+
+
+def create_kv_cache(name: str, params: KVCacheParams, **kwargs) -> H2OKVCache:
+    """``<policy>-<store>`` as in keys_values/kvcache/factory.py:50-66 (``h2o-default``,
+    ``h2o-vlen-torch-quantized8``, ``qh2o-torch-quantized8`` ...). Policies other than the H2O family
+    and stores other than bf16 / 8-bit raise."""
+    for store, quantized in _STORES.items():
+        if name.endswith("-" + store):
+            policy = name[: -len(store) - 1]
+            if policy not in _CACHE_TYPES:
+                raise NotImplementedError(f"cache policy '{policy}' is not implemented; have {sorted(_CACHE_TYPES)}")
+            return _CACHE_TYPES[policy](params, quantized=quantized, **kwargs)
+    raise NotImplementedError(f"cache name '{name}': store must be one of {sorted(_STORES)}")

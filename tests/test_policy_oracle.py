@@ -1,0 +1,196 @@
+"""Pins of the policy-variant oracle (oracle/policy_oracle.py) on the CPU: an independent per-slot
+model for the grace period, closed forms and brute force for the V-norm weighting and the Q-Hitter
+combination. None of these retype the oracle's own expressions."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kvx_oracle as O
+from oracle import policy_oracle as P
+
+
+def _inputs(seed, B, Hq, Hkv, total, D):
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    return q, k, v
+
+
+def test_no_grace_no_variant_is_the_h2o_oracle():
+    B, Hq, Hkv, L, D, chunk = 2, 4, 2, 64, 16, 8
+    q, k, v = _inputs(0, B, Hq, Hkv, L + 5 * chunk, D)
+    a = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=chunk)
+    b = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk)
+    n0 = L - 3  # the cache fills up during the first step after the prefill
+    oa = a.prefill(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    ob = b.prefill(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    assert torch.equal(oa, ob)
+    pos = n0
+    for num in (3, chunk, 1, chunk, 5):
+        sl = slice(pos, pos + num)
+        ra = a.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        rb = b.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        for x, y in zip(ra, rb):
+            assert torch.equal(x, y)
+        assert torch.equal(a.token_pos, b.token_pos) and torch.equal(a.scores, b.scores)
+        assert torch.equal(a.k, b.k) and torch.equal(a.v, b.v)
+        assert torch.equal(a.next_index, b.next_index)
+        pos += num
+
+
+@pytest.mark.parametrize("gp,steps", [(5, (1, 1, 3, 5, 7, 2, 8, 1, 4, 6, 5, 1)), (1, (1, 2, 1, 4, 1)), (13, (1,) * 40)])
+def test_grace_period_against_a_per_slot_model(gp, steps):
+    """The model keeps, per (b, h), a dict token -> (key row, value row, score) and a list of the
+    last `gp` tokens; it never computes a slot index. After every step the oracle's buffers, read
+    back through its token positions, must hold exactly the model's content, the ring must hold the
+    most recent tokens oldest-first from next_grace_pos, and the invariants of
+    test/kvcache/test_h2o.py:87-106 must hold."""
+    B, Hq, Hkv, L, D = 2, 4, 2, 48, 8
+    total = L + sum(steps)
+    q, k, v = _inputs(gp, B, Hq, Hkv, total, D)
+    ora = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=8, grace_period=gp)
+    ora.prefill(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    model = [[{t: [k[b, h, t], v[b, h, t], 0.0] for t in range(L)} for h in range(Hkv)] for b in range(B)]
+    pos = L
+    for num in steps:
+        sl = slice(pos, pos + num)
+        before_tp = ora.token_pos.clone()
+        _, w, index = ora.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        assert int(index.max()) < L - gp, "evicted slots must lie outside the ring"
+        for b in range(B):
+            for h in range(Hkv):
+                m = model[b][h]
+                for t in before_tp[b, h, index[b, h]].tolist():  # tokens in the evicted slots
+                    del m[t]
+                for t in range(pos, pos + num):
+                    m[t] = [k[b, h, t], v[b, h, t], 0.0]
+                tp = ora.token_pos[b, h].tolist()
+                assert sorted(tp) == sorted(m.keys()), "token set differs"
+                for slot, t in enumerate(tp):
+                    m[t][2] += float(w[b, h, slot])
+                    assert torch.equal(ora.k[b, h, slot], m[t][0]) and torch.equal(ora.v[b, h, slot], m[t][1])
+                    assert abs(float(ora.scores[b, h, slot]) - m[t][2]) <= 1e-5 * max(1.0, abs(m[t][2]))
+                # the ring: last gp tokens, oldest first from next_grace_pos
+                prefix = L - gp
+                start = ora.next_grace_pos - prefix
+                ring = [tp[prefix + (start + i) % gp] for i in range(gp)]
+                last = pos + num - 1
+                assert ring == list(range(last - gp + 1, last + 1))
+                assert all(0 <= x <= last - gp for x in tp[:prefix])
+        pos += num
+
+
+def test_v_length_with_equal_norms_is_plain_h2o():
+    # sum_k W = q_len, so a constant |v| cancels: instantaneous score == W
+    B, Hq, Hkv, L, D, chunk = 1, 4, 2, 64, 16, 8
+    q, k, v = _inputs(5, B, Hq, Hkv, L + 4 * chunk, D)
+    v = (v.float() / torch.linalg.vector_norm(v.float(), dim=-1, keepdim=True)).to(torch.bfloat16)
+    plain = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk)
+    vlen = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, v_length=True)
+    plain.prefill(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    vlen.prefill(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    pos = L
+    for _ in range(4):
+        sl = slice(pos, pos + chunk)
+        if vlen.next_index is not None:
+            vlen.next_index = plain.next_index  # same evictions, so that the score buffers stay comparable
+        _, _, idx = plain.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        before = vlen.scores.clone()
+        before.scatter_(-1, idx, 0.0)
+        vlen.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        # bf16 rounding leaves the norms equal to within 2^-8
+        torch.testing.assert_close(vlen.scores, plain.scores, rtol=2e-2, atol=1e-4)
+        torch.testing.assert_close((vlen.scores - before).sum(-1), torch.full((B, Hkv), float(chunk)), rtol=1e-5, atol=1e-5)
+        pos += chunk
+
+
+def test_v_length_scores_by_brute_force():
+    # test/kvcache/test_h2o.py:109-225: no eviction, every token's score recomputed from full
+    # attention over the tokens so far, in float64 loops
+    B, Hq, Hkv, L, D, n0, total = 1, 4, 2, 40, 8, 20, 36
+    q, k, v = _inputs(9, B, Hq, Hkv, total, D)
+    ora = P.PolicyCacheOracle(B, Hq, Hkv, L, D, v_length=True)
+    ora.prefill(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    expect = np.zeros((B, Hkv, total))
+    vn = np.sqrt((v.double().numpy() ** 2).sum(-1))
+    for pos in range(n0, total):
+        ora.forward(q[:, :, pos : pos + 1], k[:, :, pos : pos + 1], v[:, :, pos : pos + 1])
+        _, W, _ = O.weights_bruteforce_f64(q[:, :, pos : pos + 1], k[:, :, : pos + 1], v[:, :, : pos + 1], 1 / math.sqrt(D), pos, None)
+        s = W * vn[:, :, : pos + 1]
+        expect[:, :, : pos + 1] += s / s.sum(-1, keepdims=True)
+    np.testing.assert_allclose(ora.scores[:, :, :total].double().numpy(), expect, rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(ora.buffers["v_norm"][:, :, :total].double().numpy(), vn, rtol=1e-6)
+
+
+def _bf16_round(x: np.ndarray) -> np.ndarray:
+    """float32 -> nearest-even bfloat16, as float32 (bit arithmetic, no torch)."""
+    u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def test_quantization_error_by_loops():
+    gen = torch.Generator().manual_seed(11)
+    x = (torch.randn(6, 64, generator=gen) * 3).to(torch.bfloat16)
+    got = O.quantization_error(x).numpy()
+    xs = x.float().numpy()
+    for r in range(xs.shape[0]):
+        row = xs[r]
+        mn, mx = np.float32(row.min()), np.float32(row.max())
+        scale = max(np.float32((mx - mn) / np.float32(255.0)), np.float32(1.1920929e-07))
+        zp = -int(np.rint(np.float32(mn / scale)))
+        acc = 0.0
+        for d in range(row.size):
+            code = min(max(int(np.rint(np.float32(row[d] * np.float32(np.float32(1.0) / scale)))) + zp, 0), 255)
+            dq = _bf16_round(np.array([np.float32(code - zp) * scale], dtype=np.float32))[0]
+            diff = _bf16_round(np.array([row[d] - dq], dtype=np.float32))[0]
+            acc += float(diff) ** 2
+        assert abs(got[r] - math.sqrt(acc)) <= 1e-5 * math.sqrt(acc) + 1e-9
+
+
+def _qh_pair(c, seed=21):
+    B, Hq, Hkv, L, D, chunk = 2, 4, 2, 64, 16, 8
+    q, k, v = _inputs(seed, B, Hq, Hkv, L + 3 * chunk, D)
+    gen = torch.Generator().manual_seed(seed + 1)
+    k = (k.float() * (1 + 4 * torch.rand(B, Hkv, k.shape[2], 1, generator=gen))).to(torch.bfloat16)  # spread the quantisation errors
+    plain = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, quantized=True)
+    qh = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, quantized=True, q_hitter=True, combination_constant=c)
+    for o in (plain, qh):
+        o.prefill(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+        o.forward(q[:, :, L : L + chunk], k[:, :, L : L + chunk], v[:, :, L : L + chunk])
+    return plain, qh, chunk
+
+
+def test_q_hitter_constant_one_is_plain_h2o():
+    plain, qh, chunk = _qh_pair(1.0)
+    assert torch.equal(qh.scores, plain.scores)
+    for b in range(2):
+        for h in range(2):
+            assert set(qh.next_index[b, h].tolist()) == set(plain.next_index[b, h].tolist())
+    assert float(qh.compared.min()) >= 0.0 and float(qh.compared.max()) <= 1.0
+
+
+def test_q_hitter_constant_zero_evicts_the_largest_errors():
+    _, qh, chunk = _qh_pair(0.0)
+    qe = qh.buffers["q_errors"]
+    for b in range(2):
+        for h in range(2):
+            want = set(torch.argsort(qe[b, h], descending=True, stable=True)[:chunk].tolist())
+            assert set(qh.next_index[b, h].tolist()) == want
+    assert float(qh.compared.min()) >= 0.5 - 1e-6 and float(qh.compared.max()) <= 1.0 + 1e-6
+
+
+def test_q_hitter_values_stay_in_range_and_errors_follow_the_slots():
+    _, qh, chunk = _qh_pair(0.3)
+    c = 0.3
+    assert float(qh.compared.min()) >= (1 - c) / 2 - 1e-6 and float(qh.compared.max()) <= 1.0 + 1e-6
+    # q_errors of a slot = error of the row it holds, recomputed from the stored token position
+    B, Hq, Hkv, L, D = qh.B, qh.Hq, qh.Hkv, qh.L, qh.D
+    q, k, v = _inputs(21, B, Hq, Hkv, L + 3 * chunk, D)
+    gen = torch.Generator().manual_seed(22)
+    k = (k.float() * (1 + 4 * torch.rand(B, Hkv, k.shape[2], 1, generator=gen))).to(torch.bfloat16)
+    err = O.quantization_error(k) + O.quantization_error(v)
+    torch.testing.assert_close(qh.buffers["q_errors"], err.gather(-1, qh.token_pos.long()), rtol=0, atol=0)
