@@ -171,6 +171,37 @@ int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t
 int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows,
                         int32_t D, void* out, int64_t out_row_stride, void* stream);
 
+/* The 4-bit store of the same quantiser (num_bits = 4, keys_values/kvcache/quantize/pytorch.py:191-196):
+ * scale = max((max - min) / 15, 1.1920929e-07), codes clamped to [0, 15], and two codes per byte,
+ * byte j = code[j] << 4 | code[j + D/2] for j < D/2 (_compress_internal / _uncompress_internal,
+ * keys_values/kvcache/quantize/pytorch.py:384-393,457-465). codes: rows * D/2 bytes, contiguous. */
+int kvx_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int32_t D,
+                       uint8_t* codes, float* scale, int32_t* zp, void* stream);
+int kvx_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows,
+                         int32_t D, void* out, int64_t out_row_stride, void* stream);
+
+/* General form: a quantisation block is `nseg` segments of D contiguous bf16 values, segment s of block
+ * (o, i) at x + o*x_stride_outer + i*x_stride_inner + s*x_stride_seg (strides in elements). With
+ * nseg = n_query_groups and the segment stride that of the head axis this is blocks_over_heads=True
+ * (one block per token over all heads, keys_values/kvcache/quantize/pytorch.py:235-245,333-336: the
+ * values are transposed to (batch, slot, head, head_size) before they are flattened); nseg = 1 is the
+ * row form above. bits is 8 or 4; with 4 bits byte j of a block holds code[j] << 4 | code[j + E/2],
+ * E = nseg * D. Block (o, i) goes to codes + o*codes_stride_outer + i*E*bits/8 (bytes) and its state
+ * to scale / zp [o*state_stride_outer + i]. E <= 8192, D a multiple of 16.
+ * kvx_dequantize_blocks is the inverse with the same argument block (x is then the output). */
+typedef struct kvx_block_quant_args {
+  void* x; /* bf16; input of quantize, output of dequantize */
+  int64_t x_stride_outer, x_stride_inner, x_stride_seg;
+  int32_t n_outer, n_inner, nseg, D, bits;
+  uint8_t* codes;
+  int64_t codes_stride_outer; /* bytes */
+  float* scale;
+  int32_t* zp;
+  int64_t state_stride_outer; /* elements */
+} kvx_block_quant_args;
+int kvx_quantize_blocks(const kvx_block_quant_args* args, void* stream);
+int kvx_dequantize_blocks(const kvx_block_quant_args* args, void* stream);
+
 /* ---- cache: write and H2O bookkeeping ------------------------------------------------------- */
 
 /* Write `num` new tokens into the slots chosen by the previous selection, and do the bookkeeping

@@ -65,6 +65,17 @@ class H2OArgs(ctypes.Structure):
     ]
 
 
+class BlockQuantArgs(ctypes.Structure):
+    """struct kvx_block_quant_args"""
+
+    _fields_ = [
+        ("x", c_void_p), ("x_stride_outer", c_int64), ("x_stride_inner", c_int64), ("x_stride_seg", c_int64),
+        ("n_outer", c_int32), ("n_inner", c_int32), ("nseg", c_int32), ("D", c_int32), ("bits", c_int32),
+        ("codes", c_void_p), ("codes_stride_outer", c_int64),
+        ("scale", c_void_p), ("zp", c_void_p), ("state_stride_outer", c_int64),
+    ]
+
+
 # every symbol include/kvx.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "kvx_version": (ctypes.c_int, []),
@@ -81,6 +92,10 @@ SYMBOLS = {
     "kvx_sdpa_decode_h2o_workspace_bytes": (c_size_t, [POINTER(SdpaArgs)]),
     "kvx_quantize_rows": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "kvx_dequantize_rows": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
+    "kvx_quantize_rows4": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "kvx_dequantize_rows4": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
+    "kvx_quantize_blocks": (ctypes.c_int, [POINTER(BlockQuantArgs), c_void_p]),
+    "kvx_dequantize_blocks": (ctypes.c_int, [POINTER(BlockQuantArgs), c_void_p]),
     "kvx_cache_write": (ctypes.c_int, [POINTER(CacheWriteArgs), c_void_p]),
     "kvx_h2o_update_select": (ctypes.c_int, [POINTER(H2OArgs), c_void_p]),
     "kvx_h2o_workspace_bytes": (c_size_t, [POINTER(H2OArgs)]),

@@ -185,6 +185,58 @@ int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t*
   return launch_dequantize_rows(codes, scale, zp, rows, D, out, out_row_stride, (hipStream_t)stream);
 }
 
+int kvx_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale, int32_t* zp,
+                       void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_quantize_rows4: row length %d not in {64, 128}", D);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_quantize_rows4: rows must be >= 0");
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(x && codes && scale && zp, KVX_ERR_INVALID, "kvx_quantize_rows4: NULL pointer");
+  KVX_REQUIRE(aligned16(x) && mult8(x_row_stride) && x_row_stride >= D, KVX_ERR_INVALID,
+              "kvx_quantize_rows4: x must be 16-byte aligned, row stride a multiple of 8 and >= D");
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_quantize_rows4: codes must be 8-byte aligned");
+  return launch_quantize_rows4(x, x_row_stride, rows, D, codes, scale, zp, (hipStream_t)stream);
+}
+
+int kvx_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out,
+                         int64_t out_row_stride, void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_dequantize_rows4: row length %d not in {64, 128}", D);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_dequantize_rows4: rows must be >= 0");
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(codes && scale && zp && out, KVX_ERR_INVALID, "kvx_dequantize_rows4: NULL pointer");
+  KVX_REQUIRE(aligned16(out) && mult8(out_row_stride) && out_row_stride >= D, KVX_ERR_INVALID,
+              "kvx_dequantize_rows4: out must be 16-byte aligned, row stride a multiple of 8 and >= D");
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_dequantize_rows4: codes must be 8-byte aligned");
+  return launch_dequantize_rows4(codes, scale, zp, rows, D, out, out_row_stride, (hipStream_t)stream);
+}
+
+static int check_blocks(const kvx_block_quant_args* a, const char* who) {
+  KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "%s: args is NULL", who);
+  KVX_REQUIRE(a->n_outer >= 0 && a->n_inner >= 0 && a->nseg > 0 && a->D > 0, KVX_ERR_INVALID, "%s: bad sizes", who);
+  KVX_REQUIRE(a->bits == 8 || a->bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, a->bits);
+  KVX_REQUIRE(a->D % 16 == 0 && (int64_t)a->nseg * a->D <= 8192, KVX_ERR_UNSUPPORTED,
+              "%s: D = %d must be a multiple of 16 and the block (nseg * D = %lld) at most 8192 values", who, a->D,
+              (long long)a->nseg * a->D);
+  if (a->n_outer == 0 || a->n_inner == 0) return KVX_OK;
+  KVX_REQUIRE(a->x && a->codes && a->scale && a->zp, KVX_ERR_INVALID, "%s: NULL pointer", who);
+  KVX_REQUIRE(aligned16(a->x) && mult8(a->x_stride_outer) && mult8(a->x_stride_inner) && mult8(a->x_stride_seg), KVX_ERR_INVALID,
+              "%s: x must be 16-byte aligned with strides that are multiples of 8", who);
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(a->codes) & 7) == 0 && (a->codes_stride_outer & 7) == 0, KVX_ERR_INVALID,
+              "%s: codes must be 8-byte aligned", who);
+  return KVX_OK;
+}
+
+int kvx_quantize_blocks(const kvx_block_quant_args* a, void* stream) {
+  int rc = check_blocks(a, "kvx_quantize_blocks");
+  if (rc != KVX_OK) return rc;
+  return launch_quantize_blocks(*a, (hipStream_t)stream);
+}
+
+int kvx_dequantize_blocks(const kvx_block_quant_args* a, void* stream) {
+  int rc = check_blocks(a, "kvx_dequantize_blocks");
+  if (rc != KVX_OK) return rc;
+  return launch_dequantize_blocks(*a, (hipStream_t)stream);
+}
+
 int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");

@@ -46,6 +46,12 @@ int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int 
                          int32_t* zp, hipStream_t st);
 int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
                            int64_t out_row_stride, hipStream_t st);
+int launch_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale, int32_t* zp,
+                          hipStream_t st);
+int launch_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
+                            int64_t out_row_stride, hipStream_t st);
+int launch_quantize_blocks(const kvx_block_quant_args& a, hipStream_t st);
+int launch_dequantize_blocks(const kvx_block_quant_args& a, hipStream_t st);
 int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st);
 int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st);
 size_t h2o_workspace(const kvx_h2o_args& a);
@@ -79,15 +85,16 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 
 // The affine 8-bit row quantiser, one element. `inv` = 1.0f / scale, `zf` = (float) zero point.
 // rint before the add, so the multiply can never fuse with it.
-__device__ __forceinline__ uint32_t quant_code(float x, float inv, float zf) {
+// `qmax` = 255 (8-bit) or 15 (4-bit codes).
+__device__ __forceinline__ uint32_t quant_code(float x, float inv, float zf, float qmax = 255.0f) {
   float c = __builtin_rintf(x * inv) + zf;
-  c = fminf(fmaxf(c, 0.0f), 255.0f);
+  c = fminf(fmaxf(c, 0.0f), qmax);
   return (uint32_t)c;
 }
 
 // scale and zero point of a row from its min and max (IEEE division, no fast-math).
-__device__ __forceinline__ void quant_params(float mn, float mx, float& scale, int32_t& zp) {
-  float s = (mx - mn) / 255.0f;
+__device__ __forceinline__ void quant_params(float mn, float mx, float& scale, int32_t& zp, float qmax = 255.0f) {
+  float s = (mx - mn) / qmax;
   s = fmaxf(s, 1.1920929e-07f);
   scale = s;
   zp = 0 - (int32_t)__builtin_rintf(mn / s);

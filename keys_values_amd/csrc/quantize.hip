@@ -127,6 +127,197 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t
   }
 }
 
+// ---- 4-bit rows -------------------------------------------------------------------------------
+
+// Codes of the lane's 8 values as bytes (0..15), same layout as quantize8.
+template <int LPR>
+__device__ __forceinline__ u32x2_t quantize4(u32x4_t raw, float& scale, int32_t& zp) {
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = bf16_lo(raw[e]);
+    x[2 * e + 1] = bf16_hi(raw[e]);
+  }
+  float mn = x[0], mx = x[0];
+#pragma unroll
+  for (int e = 1; e < 8; ++e) {
+    mn = fminf(mn, x[e]);
+    mx = fmaxf(mx, x[e]);
+  }
+  mn = row_min<LPR>(mn);
+  mx = row_max<LPR>(mx);
+  quant_params(mn, mx, scale, zp, 15.0f);
+  const float inv = 1.0f / scale;
+  const float zf = (float)zp;
+  u32x2_t out;
+  out[0] = quant_code(x[0], inv, zf, 15.0f) | (quant_code(x[1], inv, zf, 15.0f) << 8) | (quant_code(x[2], inv, zf, 15.0f) << 16) |
+           (quant_code(x[3], inv, zf, 15.0f) << 24);
+  out[1] = quant_code(x[4], inv, zf, 15.0f) | (quant_code(x[5], inv, zf, 15.0f) << 8) | (quant_code(x[6], inv, zf, 15.0f) << 16) |
+           (quant_code(x[7], inv, zf, 15.0f) << 24);
+  return out;
+}
+
+// Element d shares its byte with element d + D/2 (high nibble = first half of the row): the lanes of
+// the first half fetch their partner's codes from the lane LPR/2 away and store 8 packed bytes.
+template <int D>
+__global__ __launch_bounds__(NTHREADS) void quantize_rows4_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride, int64_t rows,
+                                                                  uint8_t* __restrict__ codes, float* __restrict__ scale,
+                                                                  int32_t* __restrict__ zp) {
+  constexpr int LPR = D / 8;
+  constexpr int RPB = NTHREADS / LPR;
+  const int col = threadIdx.x % LPR;
+  const int64_t row0 = (int64_t)blockIdx.x * (RPB * ROWS_PER_THREAD) + threadIdx.x / LPR;
+  u32x4_t raw[ROWS_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    raw[i] = r < rows ? __builtin_nontemporal_load((const u32x4_t*)(x + r * x_row_stride + col * 8)) : u32x4_t{0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    const int64_t r = row0 + (int64_t)i * RPB;
+    float s;
+    int32_t z;
+    const u32x2_t c = quantize4<LPR>(raw[i], s, z);  // executed by all lanes: the reductions and the exchange need them
+    const uint32_t p0 = __shfl_xor(c[0], LPR / 2, 64), p1 = __shfl_xor(c[1], LPR / 2, 64);
+    if (r < rows && col < LPR / 2) {
+      *(u32x2_t*)(codes + r * (D / 2) + col * 8) = u32x2_t{(c[0] << 4) | p0, (c[1] << 4) | p1};
+      if (col == 0) {
+        scale[r] = s;
+        zp[r] = z;
+      }
+    }
+  }
+}
+
+// One lane per 8 packed bytes: the high nibbles are elements col*8.., the low nibbles D/2 + col*8...
+template <int D>
+__global__ __launch_bounds__(NTHREADS) void dequantize_rows4_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scale,
+                                                                    const int32_t* __restrict__ zp, int64_t rows,
+                                                                    uint16_t* __restrict__ out, int64_t out_row_stride) {
+  constexpr int LPR = D / 16;
+  const int64_t gid = (int64_t)blockIdx.x * NTHREADS + threadIdx.x;
+  const int col = (int)(gid % LPR);
+  const int64_t r = gid / LPR;
+  if (r >= rows) return;
+  const u32x2_t c = *(const u32x2_t*)(codes + r * (D / 2) + col * 8);
+  const float s = scale[r];
+  const int32_t z = zp[r];
+  u32x4_t hi, lo;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t w = c[e >> 1] >> ((e & 1) * 16);
+    hi[e] = dequant_pair((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
+    lo[e] = dequant_pair(w & 0xf, (w >> 8) & 0xf, z, s);
+  }
+  *(u32x4_t*)(out + r * out_row_stride + col * 8) = hi;
+  *(u32x4_t*)(out + r * out_row_stride + D / 2 + col * 8) = lo;
+}
+
+// ---- general blocks (several segments per block, 8 or 4 bits): one wavefront per block ------------
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fminf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ u32x2_t codes_of_chunk(u32x4_t raw, float inv, float zf, float qmax) {
+  u32x2_t out;
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    out[h] = quant_code(bf16_lo(raw[2 * h]), inv, zf, qmax) | (quant_code(bf16_hi(raw[2 * h]), inv, zf, qmax) << 8) |
+             (quant_code(bf16_lo(raw[2 * h + 1]), inv, zf, qmax) << 16) | (quant_code(bf16_hi(raw[2 * h + 1]), inv, zf, qmax) << 24);
+  return out;
+}
+
+template <int BITS>
+__global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_block_quant_args a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t blk = (int64_t)blockIdx.x * (NTHREADS / 64) + (threadIdx.x >> 6);
+  if (blk >= (int64_t)a.n_outer * a.n_inner) return;  // a whole wavefront at a time
+  const int64_t outer = blk / a.n_inner, inner = blk % a.n_inner;
+  const uint16_t* base = (const uint16_t*)a.x + outer * a.x_stride_outer + inner * a.x_stride_inner;
+  const int cps = a.D / 8;  // chunks of 8 values per segment
+  const int nchunks = a.nseg * cps;
+  auto chunk = [&](int c) { return *(const u32x4_t*)(base + (int64_t)(c / cps) * a.x_stride_seg + (c % cps) * 8); };
+  float mn = INFINITY, mx = -INFINITY;
+  for (int c = lane; c < nchunks; c += 64) {
+    const u32x4_t raw = chunk(c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mn = fminf(mn, fminf(bf16_lo(raw[e]), bf16_hi(raw[e])));
+      mx = fmaxf(mx, fmaxf(bf16_lo(raw[e]), bf16_hi(raw[e])));
+    }
+  }
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  constexpr float qmax = BITS == 8 ? 255.0f : 15.0f;
+  float s;
+  int32_t z;
+  quant_params(mn, mx, s, z, qmax);
+  const float inv = 1.0f / s, zf = (float)z;
+  uint8_t* out = a.codes + outer * a.codes_stride_outer + inner * ((int64_t)nchunks * BITS);  // nchunks * 8 values * BITS / 8 bytes
+  if constexpr (BITS == 8) {
+    for (int c = lane; c < nchunks; c += 64) *(u32x2_t*)(out + c * 8) = codes_of_chunk(chunk(c), inv, zf, qmax);
+  } else {
+    const int half = nchunks / 2;
+    for (int c = lane; c < half; c += 64) {
+      const u32x2_t hi = codes_of_chunk(chunk(c), inv, zf, qmax), lo = codes_of_chunk(chunk(c + half), inv, zf, qmax);
+      *(u32x2_t*)(out + c * 8) = u32x2_t{(hi[0] << 4) | lo[0], (hi[1] << 4) | lo[1]};
+    }
+  }
+  if (lane == 0) {
+    a.scale[outer * a.state_stride_outer + inner] = s;
+    a.zp[outer * a.state_stride_outer + inner] = z;
+  }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(NTHREADS) void dequantize_blocks_kernel(const kvx_block_quant_args a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t blk = (int64_t)blockIdx.x * (NTHREADS / 64) + (threadIdx.x >> 6);
+  if (blk >= (int64_t)a.n_outer * a.n_inner) return;
+  const int64_t outer = blk / a.n_inner, inner = blk % a.n_inner;
+  uint16_t* base = (uint16_t*)a.x + outer * a.x_stride_outer + inner * a.x_stride_inner;
+  const int cps = a.D / 8;
+  const int nchunks = a.nseg * cps;
+  auto chunk_ptr = [&](int c) { return (u32x4_t*)(base + (int64_t)(c / cps) * a.x_stride_seg + (c % cps) * 8); };
+  const float s = a.scale[outer * a.state_stride_outer + inner];
+  const int32_t z = a.zp[outer * a.state_stride_outer + inner];
+  const uint8_t* in = a.codes + outer * a.codes_stride_outer + inner * ((int64_t)nchunks * BITS);
+  if constexpr (BITS == 8) {
+    for (int c = lane; c < nchunks; c += 64) {
+      const u32x2_t cc = *(const u32x2_t*)(in + c * 8);
+      u32x4_t o;
+      o[0] = dequant_pair(cc[0] & 0xff, (cc[0] >> 8) & 0xff, z, s);
+      o[1] = dequant_pair((cc[0] >> 16) & 0xff, cc[0] >> 24, z, s);
+      o[2] = dequant_pair(cc[1] & 0xff, (cc[1] >> 8) & 0xff, z, s);
+      o[3] = dequant_pair((cc[1] >> 16) & 0xff, cc[1] >> 24, z, s);
+      *chunk_ptr(c) = o;
+    }
+  } else {
+    const int half = nchunks / 2;
+    for (int c = lane; c < half; c += 64) {
+      const u32x2_t cc = *(const u32x2_t*)(in + c * 8);
+      u32x4_t hi, lo;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t w = cc[e >> 1] >> ((e & 1) * 16);
+        hi[e] = dequant_pair((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
+        lo[e] = dequant_pair(w & 0xf, (w >> 8) & 0xf, z, s);
+      }
+      *chunk_ptr(c) = hi;
+      *chunk_ptr(c + half) = lo;
+    }
+  }
+}
+
 // Sum over the LPR adjacent lanes holding one row; every lane gets the result.
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {
@@ -282,6 +473,52 @@ int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32
     hipLaunchKernelGGL((dequantize_rows_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
   else
     hipLaunchKernelGGL((dequantize_rows_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale, int32_t* zp,
+                          hipStream_t st) {
+  if (rows == 0) return KVX_OK;
+  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
+  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
+  if (D == 128)
+    hipLaunchKernelGGL((quantize_rows4_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  else
+    hipLaunchKernelGGL((quantize_rows4_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
+                            int64_t out_row_stride, hipStream_t st) {
+  if (rows == 0) return KVX_OK;
+  const int64_t lanes = rows * (D / 16);
+  const unsigned grid = (unsigned)((lanes + NTHREADS - 1) / NTHREADS);
+  if (D == 128)
+    hipLaunchKernelGGL((dequantize_rows4_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  else
+    hipLaunchKernelGGL((dequantize_rows4_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_quantize_blocks(const kvx_block_quant_args& a, hipStream_t st) {
+  const int64_t blocks = (int64_t)a.n_outer * a.n_inner;
+  if (blocks == 0) return KVX_OK;
+  const unsigned grid = (unsigned)((blocks + NTHREADS / 64 - 1) / (NTHREADS / 64));
+  if (a.bits == 8) hipLaunchKernelGGL((quantize_blocks_kernel<8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else hipLaunchKernelGGL((quantize_blocks_kernel<4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_dequantize_blocks(const kvx_block_quant_args& a, hipStream_t st) {
+  const int64_t blocks = (int64_t)a.n_outer * a.n_inner;
+  if (blocks == 0) return KVX_OK;
+  const unsigned grid = (unsigned)((blocks + NTHREADS / 64 - 1) / (NTHREADS / 64));
+  if (a.bits == 8) hipLaunchKernelGGL((dequantize_blocks_kernel<8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else hipLaunchKernelGGL((dequantize_blocks_kernel<4>), dim3(grid), dim3(NTHREADS), 0, st, a);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }

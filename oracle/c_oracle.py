@@ -46,6 +46,28 @@ def dequantize_rows(codes: np.ndarray, scale: np.ndarray, zp: np.ndarray):
     return out
 
 
+def quantize_blocks4(x: np.ndarray):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    blocks, E = x.shape
+    packed = np.empty((blocks, E // 2), np.uint8)
+    scale = np.empty(blocks, np.float32)
+    zp = np.empty(blocks, np.int32)
+    _lib().kvxo_quantize_blocks4(_p(x, ctypes.c_float), ctypes.c_int64(blocks), ctypes.c_int32(E),
+                                 _p(packed, ctypes.c_uint8), _p(scale, ctypes.c_float), _p(zp, ctypes.c_int32))
+    return packed, scale, zp
+
+
+def dequantize_blocks4(packed: np.ndarray, scale: np.ndarray, zp: np.ndarray):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    scale = np.ascontiguousarray(scale, dtype=np.float32)
+    zp = np.ascontiguousarray(zp, dtype=np.int32)
+    blocks, half = packed.shape
+    out = np.empty((blocks, 2 * half), np.float32)
+    _lib().kvxo_dequantize_blocks4(_p(packed, ctypes.c_uint8), _p(scale, ctypes.c_float), _p(zp, ctypes.c_int32),
+                                   ctypes.c_int64(blocks), ctypes.c_int32(2 * half), _p(out, ctypes.c_float))
+    return out
+
+
 def sdpa_weights(q, k, v, tp, input_pos, scale):
     q = np.ascontiguousarray(q, dtype=np.float32)
     k = np.ascontiguousarray(k, dtype=np.float32)

@@ -47,6 +47,49 @@ void kvxo_dequantize_rows(const uint8_t* codes, const float* scale, const int32_
     for (int d = 0; d < D; ++d) out[r * (int64_t)D + d] = (float)((int32_t)codes[r * (int64_t)D + d] - zp[r]) * scale[r];
 }
 
+/* The same quantiser with num_bits = 4 (keys_values/kvcache/quantize/pytorch.py:191-196: codes in
+ * [0, 15]) and its packing, two codes per byte with the first half of the block in the high nibbles
+ * (:384-393). Blocks of E float32 values (E = head_size, or n_query_groups * head_size when the
+ * blocks run over the heads, :235-245); packed holds E/2 bytes per block. */
+void kvxo_quantize_blocks4(const float* x, int64_t blocks, int32_t E, uint8_t* packed, float* scale, int32_t* zp) {
+  uint8_t* tmp = (uint8_t*)malloc((size_t)E);
+  for (int64_t r = 0; r < blocks; ++r) {
+    const float* row = x + r * (int64_t)E;
+    float mn = row[0], mx = row[0];
+    for (int d = 1; d < E; ++d) {
+      if (row[d] < mn) mn = row[d];
+      if (row[d] > mx) mx = row[d];
+    }
+    float s = (mx - mn) / 15.0f;
+    if (s < 1.1920929e-07f) s = 1.1920929e-07f;
+    int32_t z = 0 - (int32_t)rintf(mn / s);
+    float inv = 1.0f / s;
+    float zf = (float)z;
+    for (int d = 0; d < E; ++d) {
+      float c = rintf(row[d] * inv) + zf;
+      if (c < 0.0f) c = 0.0f;
+      if (c > 15.0f) c = 15.0f;
+      tmp[d] = (uint8_t)c;
+    }
+    for (int d = 0; d < E / 2; ++d) packed[r * (int64_t)(E / 2) + d] = (uint8_t)((tmp[d] << 4) | tmp[d + E / 2]);
+    scale[r] = s;
+    zp[r] = z;
+  }
+  free(tmp);
+}
+
+/* keys_values/kvcache/quantize/pytorch.py:457-465 (unpack: high nibbles first, then low nibbles) and
+ * :143-154. */
+void kvxo_dequantize_blocks4(const uint8_t* packed, const float* scale, const int32_t* zp, int64_t blocks, int32_t E,
+                             float* out) {
+  for (int64_t r = 0; r < blocks; ++r)
+    for (int d = 0; d < E / 2; ++d) {
+      uint8_t byte = packed[r * (int64_t)(E / 2) + d];
+      out[r * (int64_t)E + d] = (float)((int32_t)(byte >> 4) - zp[r]) * scale[r];
+      out[r * (int64_t)E + E / 2 + d] = (float)((int32_t)(byte & 15) - zp[r]) * scale[r];
+    }
+}
+
 /* keys_values/attention/base.py:660-742 + keys_values/attention/attention_utils.py:383-443 as
  * explicit loops. q (B,Hq,q_len,D), k/v (B,Hkv,T,D), tp (B,Hkv,T) or NULL, all contiguous.
  * o (B,Hq,q_len,D), w (B,Hkv,T) (sum over queries, mean over the group), lse2 (B,q_len,Hq).

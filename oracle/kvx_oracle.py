@@ -16,9 +16,11 @@ How each function is pinned (tests/test_oracle.py):
   per-head result (test/attention/test_attention.py:78-166), blocked == unblocked
   (test/attention/test_attention.py:706-797), reorder == position mask
   (test/attention/test_sdpa_wrapper.py:55-153), and the independent scalar C restatement.
-* ``quantize_rows`` / ``dequantize_rows``: the known-answer round trip of
-  test/kvcache/test_quantization.py:647-766, hand-computed vectors, and bit-equality with the
-  scalar C restatement (IEEE float32 primitives only).
+* ``quantize_rows`` / ``dequantize_rows`` (8 and 4 bits), ``compress4`` / ``uncompress4``,
+  ``quantize_store`` / ``dequantize_store``: the known-answer round trip of
+  test/kvcache/test_quantization.py:647-766 (integers with both extremes in every block, rows and
+  blocks over heads), hand-computed vectors and packed bytes, and bit-equality with the scalar C
+  restatement (IEEE float32 primitives only).
 * ``h2o_update_select`` / ``cache_write`` / ``H2OCacheOracle``: brute-force python loops on small caches
   and the bookkeeping checks of test/kvcache/test_h2o.py:109-137,227-343.
 * Tie order of ``torch.argsort`` / ``torch.topk(sorted=False)`` is implementation-defined in the
@@ -205,16 +207,17 @@ def reorder_key_value(key, value, token_positions):
 # --------------------------------------------------------------------------------------------
 
 
-def quantize_rows(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+def quantize_rows(x: torch.Tensor, num_bits: int = 8) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """keys_values/kvcache/quantize/pytorch.py:312-355 (_quantize), :100-116 (_calculate_qparams),
-    :120-139 (quantize_per_channel) for the 8-bit case, one block per row.
-    x (..., D) any float dtype. Returns codes uint8 (..., D), scale fp32 (...), zp int32 (...)."""
+    :120-139 (quantize_per_channel), one block per row; quant_max = 2**num_bits - 1 (:191-196).
+    x (..., D) any float dtype. Returns codes uint8 (..., D) (not packed), scale fp32 (...), zp int32 (...)."""
     shape = x.shape
+    qmax = 2**num_bits - 1
     v = x.to(torch.float32).reshape(-1, shape[-1])  # :333
     mn, mx = torch.aminmax(v, dim=1)  # :90
-    scale = torch.clamp((mx - mn) / float(255 - 0), min=F32_EPS)  # :111-114
+    scale = torch.clamp((mx - mn) / float(qmax - 0), min=F32_EPS)  # :111-114
     zp = 0 - torch.round(mn / scale).to(torch.int32)  # :115
-    res = torch.clamp(torch.round(v * (1.0 / scale.view(-1, 1))) + zp.view(-1, 1), 0, 255)  # :134-138
+    res = torch.clamp(torch.round(v * (1.0 / scale.view(-1, 1))) + zp.view(-1, 1), 0, qmax)  # :134-138
     return res.to(torch.uint8).reshape(shape), scale.reshape(shape[:-1]), zp.reshape(shape[:-1])
 
 
@@ -226,10 +229,44 @@ def dequantize_rows(codes: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor, 
     return res.to(torch.float32).to(dtype)
 
 
-def quantization_error(x: torch.Tensor) -> torch.Tensor:
+def compress4(codes: torch.Tensor) -> torch.Tensor:
+    """keys_values/kvcache/quantize/pytorch.py:384-393: byte j = code[j] << 4 | code[j + n/2]."""
+    half = codes.shape[-1] // 2
+    return torch.bitwise_or(torch.bitwise_left_shift(codes[..., :half], 4), codes[..., half:])
+
+
+def uncompress4(packed: torch.Tensor) -> torch.Tensor:
+    """keys_values/kvcache/quantize/pytorch.py:457-465."""
+    return torch.cat((torch.bitwise_right_shift(packed, 4), torch.bitwise_and(packed, 15)), dim=-1)
+
+
+def quantize_store(values: torch.Tensor, num_bits: int = 8, blocks_over_heads: bool = False):
+    """What TorchBasicQuantizer.quantize leaves in its buffers for values (B, Hkv, n, D)
+    (keys_values/kvcache/quantize/pytorch.py:235-245,312-355): quant_buffer (first, n, final) uint8 with
+    first = B*Hkv, final = D[/2], or first = B, final = Hkv*D[/2] when the blocks run over the heads
+    (values transposed to (B, n, Hkv, D) first, :335-337); quant_scales / quant_zero_points (first, n)."""
+    B, Hkv, n, D = values.shape
+    v = values.transpose(1, 2).reshape(B, n, Hkv * D) if blocks_over_heads else values.reshape(B * Hkv, n, D)
+    codes, scale, zp = quantize_rows(v, num_bits)
+    if num_bits == 4:
+        codes = compress4(codes)
+    return codes, scale, zp
+
+
+def dequantize_store(buffer, scale, zp, shape, num_bits: int = 8, blocks_over_heads: bool = False, dtype=torch.bfloat16):
+    """Inverse of quantize_store, to (B, Hkv, n, D) (keys_values/kvcache/quantize/pytorch.py:411-478)."""
+    B, Hkv, n, D = shape
+    codes = uncompress4(buffer) if num_bits == 4 else buffer
+    out = dequantize_rows(codes, scale, zp, dtype)
+    if blocks_over_heads:
+        return out.reshape(B, n, Hkv, D).transpose(1, 2)
+    return out.reshape(B, Hkv, n, D)
+
+
+def quantization_error(x: torch.Tensor, num_bits: int = 8) -> torch.Tensor:
     """keys_values/kvcache/quantize/pytorch.py:530-548: per-row L2 norm of x - dequant(quant(x)); the
     dequantised rows and the difference are in the source dtype, the norm accumulates in float32."""
-    c, s, z = quantize_rows(x)
+    c, s, z = quantize_rows(x, num_bits)
     return torch.linalg.vector_norm(x - dequantize_rows(c, s, z, x.dtype), dim=-1, dtype=torch.float32)
 
 

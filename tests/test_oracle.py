@@ -203,6 +203,69 @@ def test_quantization_error_bound_and_zero():
     assert (err <= 0.5001 * s * math.sqrt(128)).all() and (err > 0).all()
 
 
+def test_quantiser_4bit_hand_vector_and_packing():
+    # scale = 3/15 = 0.2; zp = -rint(-1/0.2) = 5; codes rint(x/0.2) + 5
+    x = torch.tensor([[-1.0, -0.6, 0.0, 2.0]])
+    c, s, z = O.quantize_rows(x, num_bits=4)
+    assert c.tolist() == [[0, 2, 5, 15]] and z.tolist() == [5]
+    assert s.item() == np.float32(3.0) / np.float32(15.0)
+    # keys_values/kvcache/quantize/pytorch.py:384-393: first half of the row in the high nibbles
+    assert O.compress4(c).tolist() == [[0 << 4 | 5, 2 << 4 | 15]]
+    assert torch.equal(O.uncompress4(O.compress4(c)), c)
+    codes = torch.arange(16, dtype=torch.uint8).view(1, 16)
+    assert O.compress4(codes).tolist() == [[0x08, 0x19, 0x2A, 0x3B, 0x4C, 0x5D, 0x6E, 0x7F]]
+
+
+@pytest.mark.parametrize("num_bits", [4, 8])
+@pytest.mark.parametrize("blocks_over_heads", [False, True])
+@pytest.mark.parametrize("kind", ["as_is", "shift", "scale"])
+def test_quantiser_store_known_answer(num_bits, blocks_over_heads, kind):
+    # test/kvcache/test_quantization.py:647-766 for both widths and both block shapes: integers that
+    # hold both extremes in every head row (hence in every block) round-trip exactly
+    gen = torch.Generator().manual_seed(31415927)
+    shape = (3, 4, 32, 64)
+    high = 2**num_bits
+    data = torch.randint(0, high, shape, generator=gen)
+    i0 = torch.randint(0, 64, shape[:-1], generator=gen)
+    i1 = (i0 + 1 + torch.randint(0, 63, shape[:-1], generator=gen)) % 64
+    data.scatter_(-1, i0.unsqueeze(-1), 0)
+    data.scatter_(-1, i1.unsqueeze(-1), high - 1)
+    x = data.to(torch.float32)
+    per_block = (3, 1, 32, 1) if blocks_over_heads else (3, 4, 32, 1)
+    if kind == "shift":
+        x = x + torch.randint(-1024, 1024, per_block, generator=gen)
+    if kind == "scale":
+        x = x * torch.randn(per_block, generator=gen).exp()
+    buf, s, z = O.quantize_store(x, num_bits, blocks_over_heads)
+    first, final = (3, 4 * 64) if blocks_over_heads else (12, 64)
+    assert buf.shape == (first, 32, final * num_bits // 8) and buf.dtype == torch.uint8
+    assert s.shape == (first, 32) and z.shape == (first, 32) and z.dtype == torch.int32
+    back = O.dequantize_store(buf, s, z, shape, num_bits, blocks_over_heads, torch.float32)
+    if kind == "scale":
+        torch.testing.assert_close(back, x)
+    else:
+        assert torch.equal(back, x)
+        codes = O.uncompress4(buf) if num_bits == 4 else buf
+        want = data.transpose(1, 2).reshape(3, 32, 256) if blocks_over_heads else data.reshape(12, 32, 64)
+        assert torch.equal(codes.to(torch.int64), want)
+
+
+def test_quantiser_4bit_python_and_c_bit_equal():
+    gen = torch.Generator().manual_seed(5)
+    x = (torch.randn(2048, 128, generator=gen) * 2).to(torch.bfloat16)
+    x[0] = 0.0
+    x[1] = -3.5
+    for E in (128, 1024):  # rows, and blocks over 8 heads
+        xb = x.float().reshape(-1, E)
+        c, s, z = O.quantize_rows(xb, num_bits=4)
+        p = O.compress4(c)
+        p2, s2, z2 = C.quantize_blocks4(xb.numpy())
+        assert np.array_equal(p.numpy(), p2) and np.array_equal(s.numpy(), s2) and np.array_equal(z.numpy(), z2)
+        d = O.dequantize_rows(O.uncompress4(p), s, z, torch.float32)
+        assert np.array_equal(d.numpy(), C.dequantize_blocks4(p2, s2, z2))
+        assert ((xb - d).abs() <= 0.5001 * s.unsqueeze(-1) + 1e-7).all()
+
+
 # ---- H2O bookkeeping -------------------------------------------------------------------------------
 
 
