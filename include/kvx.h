@@ -49,10 +49,13 @@ enum kvx_status {
 /* Storage type of the K/V cache handed to the attention kernels. */
 enum kvx_kv_dtype {
   KVX_KV_BF16 = 0, /* bfloat16 rows */
-  KVX_KV_U8 = 1    /* uint8 codes + per-row fp32 scale and int32 zero point (the reference's
+  KVX_KV_U8 = 1,   /* uint8 codes + per-row fp32 scale and int32 zero point (the reference's
                       "torch-quantized8" store, keys_values/kvcache/quantize/pytorch.py:281-295);
                       rows are dequantised inside the kernel exactly as
                       keys_values/kvcache/quantize/pytorch.py:143-154,467-478 would, i.e. to bf16 */
+  KVX_KV_U4 = 2    /* the 4-bit store of the same quantiser ("torch-quantized4"): rows of D/2 bytes, byte j =
+                      code[j] << 4 | code[j + D/2] (keys_values/kvcache/quantize/pytorch.py:384-393,457-465),
+                      same per-row state; strides of k / v count bytes */
 };
 
 /* One attention call. Unused pointers are NULL. All strides in elements. */

@@ -25,7 +25,7 @@ ALLOWED_HEAD_SIZES = (64, 128)  # keys_values/attention/flashinfer_wrapper.py:27
 
 
 class QuantState(NamedTuple):
-    """Per-row state of a uint8 cache: fp32 scales and int32 zero points, each (B, Hkv, T) with a
+    """Per-row state of a quantised cache (uint8 codes of D bytes per row, or the 4-bit store of D/2 bytes per row): fp32 scales and int32 zero points, each (B, Hkv, T) with a
     contiguous last axis; K and V arrays share their strides
     (keys_values/kvcache/quantize/pytorch.py:281-295)."""
 
@@ -81,7 +81,8 @@ def _fill_common(a: _lib.SdpaArgs, query, key, value, scale, input_pos, token_po
         a.v = value.data_ptr()
         a.v_stride_b, a.v_stride_h, a.v_stride_t = value.stride(0), value.stride(1), value.stride(2)
     if quant is not None:
-        a.kv_dtype = _lib.KVX_KV_U8
+        # rows of D bytes: 8-bit codes; rows of D/2 bytes: the 4-bit store, two codes per byte
+        a.kv_dtype = _lib.KVX_KV_U4 if key.shape[3] * 2 == D else _lib.KVX_KV_U8
         for t in quant:
             if t.shape != (B, Hkv, T) or t.stride(-1) != 1 or t.stride() != quant.k_scale.stride():
                 raise ValueError("quantisation state must be (B, Hkv, T) arrays sharing strides, last axis contiguous")
@@ -95,6 +96,11 @@ def _fill_common(a: _lib.SdpaArgs, query, key, value, scale, input_pos, token_po
     if token_positions is not None:
         a.token_positions = token_positions.data_ptr()
         a.tp_stride_b, a.tp_stride_h = token_positions.stride(0), token_positions.stride(1)
+
+
+def _row_len(D: int, key: torch.Tensor, quant) -> int:
+    """Last-axis length a cache row must have: D, or D/2 bytes for the 4-bit store."""
+    return D // 2 if (quant is not None and key.shape[3] * 2 == D) else D
 
 
 def _check_dtypes(query, key, value, quant):
@@ -144,7 +150,7 @@ def prefill_core(
     _check_dtypes(query, key, value, quant)
     B, Hq, q_len, D = query.shape
     Hkv, T = key.shape[1], key.shape[2]
-    if key.shape != value.shape or key.shape[0] != B or key.shape[3] != D:
+    if key.shape != value.shape or key.shape[0] != B or key.shape[3] != _row_len(D, key, quant):
         raise ValueError(f"key.shape = {tuple(key.shape)}, value.shape = {tuple(value.shape)} do not fit query {tuple(query.shape)}")
     if not (0 < q_len <= T):
         raise ValueError(f"Must have 0 < q_len = {q_len} <= kv_len = {T}")
@@ -227,7 +233,7 @@ def decode_core(
     Hkv, T = key.shape[1], key.shape[2]
     if q_len != 1:
         raise ValueError(f"decode needs q_len == 1, got {q_len}")
-    if key.shape != value.shape or key.shape[0] != B or key.shape[3] != D:
+    if key.shape != value.shape or key.shape[0] != B or key.shape[3] != _row_len(D, key, quant):
         raise ValueError(f"key.shape = {tuple(key.shape)}, value.shape = {tuple(value.shape)} do not fit query {tuple(query.shape)}")
     if Hkv <= 0 or Hq % Hkv != 0:
         raise ValueError(f"n_head = {Hq} must be a positive multiple of n_query_groups = {Hkv}")

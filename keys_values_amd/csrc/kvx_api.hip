@@ -50,8 +50,9 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
               a->kv_len);
   KVX_REQUIRE(a->Hq % a->Hkv == 0, KVX_ERR_INVALID, "%s: Hq=%d must be a multiple of Hkv=%d", who, a->Hq, a->Hkv);
   KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, a->D);
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8, KVX_ERR_UNSUPPORTED, "%s: unknown kv_dtype %d", who,
-              a->kv_dtype);
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4, KVX_ERR_UNSUPPORTED,
+              "%s: unknown kv_dtype %d", who, a->kv_dtype);
+  const int row_elems = a->kv_dtype == KVX_KV_U4 ? a->D / 2 : a->D;  // elements of the cache's own type per row
   KVX_REQUIRE(a->input_pos >= 0, KVX_ERR_INVALID, "%s: input_pos=%d must be >= 0", who, a->input_pos);
   KVX_REQUIRE(a->sm_scale > 0.0f, KVX_ERR_INVALID, "%s: sm_scale must be positive", who);
   KVX_REQUIRE((int64_t)a->input_pos + a->q_len < INT32_MAX, KVX_ERR_INVALID, "%s: positions overflow int32", who);
@@ -60,18 +61,18 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
               "%s: q must be 16-byte aligned with strides that are multiples of 8 elements", who);
   KVX_REQUIRE(aligned16(a->k) && mult8(a->k_stride_b) && mult8(a->k_stride_h) && mult8(a->k_stride_t), KVX_ERR_INVALID,
               "%s: k must be 16-byte aligned with strides that are multiples of 8 elements", who);
-  KVX_REQUIRE(a->k_stride_t >= a->D && a->q_stride_t >= 0, KVX_ERR_INVALID, "%s: bad k/q slot stride", who);
+  KVX_REQUIRE(a->k_stride_t >= row_elems && a->q_stride_t >= 0, KVX_ERR_INVALID, "%s: bad k/q slot stride", who);
   if (need_v_o) {
     KVX_REQUIRE(a->v && a->o, KVX_ERR_INVALID, "%s: v and o must be given", who);
     KVX_REQUIRE(aligned16(a->v) && mult8(a->v_stride_b) && mult8(a->v_stride_h) && mult8(a->v_stride_t), KVX_ERR_INVALID,
                 "%s: v must be 16-byte aligned with strides that are multiples of 8 elements", who);
     KVX_REQUIRE(aligned16(a->o) && mult8(a->o_stride_b) && mult8(a->o_stride_h) && mult8(a->o_stride_t), KVX_ERR_INVALID,
                 "%s: o must be 16-byte aligned with strides that are multiples of 8 elements", who);
-    KVX_REQUIRE(a->v_stride_t >= a->D, KVX_ERR_INVALID, "%s: bad v slot stride", who);
+    KVX_REQUIRE(a->v_stride_t >= row_elems, KVX_ERR_INVALID, "%s: bad v slot stride", who);
   }
-  if (a->kv_dtype == KVX_KV_U8) {
-    KVX_REQUIRE(a->k_scale && a->k_zp, KVX_ERR_INVALID, "%s: uint8 cache needs k_scale and k_zp", who);
-    if (need_v_o) KVX_REQUIRE(a->v_scale && a->v_zp, KVX_ERR_INVALID, "%s: uint8 cache needs v_scale and v_zp", who);
+  if (a->kv_dtype != KVX_KV_BF16) {
+    KVX_REQUIRE(a->k_scale && a->k_zp, KVX_ERR_INVALID, "%s: quantised cache needs k_scale and k_zp", who);
+    if (need_v_o) KVX_REQUIRE(a->v_scale && a->v_zp, KVX_ERR_INVALID, "%s: quantised cache needs v_scale and v_zp", who);
   }
   KVX_REQUIRE(a->num_splits >= 0, KVX_ERR_INVALID, "%s: num_splits must be >= 0", who);
   return KVX_OK;
@@ -241,7 +242,8 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");
   KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "kvx_cache_write: head size %d not in {64, 128}", a->D);
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8, KVX_ERR_UNSUPPORTED, "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4, KVX_ERR_UNSUPPORTED,
+              "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
   KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
   KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache && a->token_pos, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
   KVX_REQUIRE(aligned16(a->key) && aligned16(a->value) && mult8(a->key_stride_b) && mult8(a->key_stride_h) &&
@@ -250,8 +252,8 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(aligned16(a->k_cache) && aligned16(a->v_cache) && mult8(a->kc_stride_b) && mult8(a->kc_stride_h) &&
                   mult8(a->kc_stride_t) && mult8(a->vc_stride_b) && mult8(a->vc_stride_h) && mult8(a->vc_stride_t),
               KVX_ERR_INVALID, "kvx_cache_write: caches must be 16-byte aligned with strides that are multiples of 8");
-  if (a->kv_dtype == KVX_KV_U8)
-    KVX_REQUIRE(a->k_scale && a->k_zp && a->v_scale && a->v_zp, KVX_ERR_INVALID, "kvx_cache_write: uint8 cache needs scale / zero-point arrays");
+  if (a->kv_dtype != KVX_KV_BF16)
+    KVX_REQUIRE(a->k_scale && a->k_zp && a->v_scale && a->v_zp, KVX_ERR_INVALID, "kvx_cache_write: quantised cache needs scale / zero-point arrays");
   KVX_REQUIRE((int64_t)a->input_pos + a->num < INT32_MAX && a->input_pos >= 0, KVX_ERR_INVALID, "kvx_cache_write: bad input_pos");
   KVX_REQUIRE(a->grace_num >= 0 && a->grace_num <= a->num, KVX_ERR_INVALID, "kvx_cache_write: grace_num=%d must be in [0, num=%d]", a->grace_num, a->num);
   if (a->grace_num > 0) {
@@ -260,7 +262,7 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
                 "kvx_cache_write: need grace_num=%d <= grace_period=%d < cache_len=%d and input_pos=%d >= grace_period", a->grace_num,
                 a->grace_period, a->cache_len, a->input_pos);
   }
-  KVX_REQUIRE(!a->q_errors || a->kv_dtype == KVX_KV_U8, KVX_ERR_INVALID, "kvx_cache_write: q_errors needs the uint8 cache");
+  KVX_REQUIRE(!a->q_errors || a->kv_dtype != KVX_KV_BF16, KVX_ERR_INVALID, "kvx_cache_write: q_errors needs a quantised cache");
   return launch_cache_write(*a, (hipStream_t)stream);
 }
 

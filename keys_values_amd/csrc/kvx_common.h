@@ -107,4 +107,15 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t c0, uint32_t c1, int32
   return pack_bf16(a, b);
 }
 
+// 4-bit store (two codes per byte, first half of the row in the high nibbles): chunk c (values
+// 8c .. 8c+7) of a row of D values lies in one nibble of the 8 bytes at u4_byte_off, and becomes 8
+// byte-sized codes with u4_codes.
+template <int D>
+__device__ __forceinline__ uint32_t u4_byte_off(int c) { return (uint32_t)(c % (D / 16)) * 8u; }
+template <int D>
+__device__ __forceinline__ int u4_shift(int c) { return c < D / 16 ? 4 : 0; }
+__device__ __forceinline__ u32x2_t u4_codes(u32x2_t bytes, int shift) {
+  return u32x2_t{(bytes[0] >> shift) & 0x0f0f0f0fu, (bytes[1] >> shift) & 0x0f0f0f0fu};
+}
+
 }  // namespace kvx

@@ -364,8 +364,10 @@ __device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, flo
 // token j into index[b,h,j]. With one (j < grace_num) the lane first carries its 8 elements of ring
 // slot grace_slots[j] over to index[b,h,j], then writes new token num - grace_num + j into the ring
 // slot: the read and the write of that slot are issued by the same lane, in this order.
-template <int D, bool U8>
+template <int D, int KV>
 __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
+  constexpr bool U8 = KV != KVX_KV_BF16;  // a quantised store: codes + row state
+  constexpr bool U4 = KV == KVX_KV_U4;    // two codes per byte: only the lanes of the first half of a row store
   constexpr int LPR = D / 8;
   const int64_t gid = (int64_t)blockIdx.x * NTHREADS + threadIdx.x;
   const int col = (int)(gid % LPR);
@@ -391,16 +393,20 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   const int64_t sc_row = b * a.sc_stride_b + hh * a.sc_stride_h;
   const int64_t qs_row = b * a.qs_stride_b + hh * a.qs_stride_h;
   constexpr int ES = U8 ? 1 : 2;  // bytes per cache element
-  uint8_t* kc_row = (uint8_t*)a.k_cache + (b * a.kc_stride_b + hh * a.kc_stride_h) * ES + col * 8 * ES;
-  uint8_t* vc_row = (uint8_t*)a.v_cache + (b * a.vc_stride_b + hh * a.vc_stride_h) * ES + col * 8 * ES;
+  const bool stores = !U4 || col < LPR / 2;
+  const int ccol = U4 ? col % (LPR / 2) : col;
+  uint8_t* kc_row = (uint8_t*)a.k_cache + (b * a.kc_stride_b + hh * a.kc_stride_h) * ES + ccol * 8 * ES;
+  uint8_t* vc_row = (uint8_t*)a.v_cache + (b * a.vc_stride_b + hh * a.vc_stride_h) * ES + ccol * 8 * ES;
 
   if (ok && moves) {
     if constexpr (!U8) {
       *(u32x4_t*)(kc_row + (int64_t)slot * a.kc_stride_t * ES) = *(const u32x4_t*)(kc_row + (int64_t)ring * a.kc_stride_t * ES);
       *(u32x4_t*)(vc_row + (int64_t)slot * a.vc_stride_t * ES) = *(const u32x4_t*)(vc_row + (int64_t)ring * a.vc_stride_t * ES);
     } else {
-      *(u32x2_t*)(kc_row + (int64_t)slot * a.kc_stride_t) = *(const u32x2_t*)(kc_row + (int64_t)ring * a.kc_stride_t);
-      *(u32x2_t*)(vc_row + (int64_t)slot * a.vc_stride_t) = *(const u32x2_t*)(vc_row + (int64_t)ring * a.vc_stride_t);
+      if (stores) {
+        *(u32x2_t*)(kc_row + (int64_t)slot * a.kc_stride_t) = *(const u32x2_t*)(kc_row + (int64_t)ring * a.kc_stride_t);
+        *(u32x2_t*)(vc_row + (int64_t)slot * a.vc_stride_t) = *(const u32x2_t*)(vc_row + (int64_t)ring * a.vc_stride_t);
+      }
       if (col == 0) {
         a.k_scale[qs_row + slot] = a.k_scale[qs_row + ring];
         a.k_zp[qs_row + slot] = a.k_zp[qs_row + ring];
@@ -425,12 +431,18 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   } else {
     float s1, s2;
     int32_t z1, z2;
-    const u32x2_t kc = quantize8<LPR>(kr, s1, z1);
-    const u32x2_t vc = quantize8<LPR>(vr, s2, z2);
+    u32x2_t kc = U4 ? quantize4<LPR>(kr, s1, z1) : quantize8<LPR>(kr, s1, z1);
+    u32x2_t vc = U4 ? quantize4<LPR>(vr, s2, z2) : quantize8<LPR>(vr, s2, z2);
     if (a.q_errors) qerr = row_quant_error<LPR>(kr, kc, s1, z1) + row_quant_error<LPR>(vr, vc, s2, z2);  // uniform branch
+    if constexpr (U4) {  // byte j = code[j] << 4 | code[j + D/2]: the partner lane holds the low nibbles
+      kc = u32x2_t{(kc[0] << 4) | (uint32_t)__shfl_xor(kc[0], LPR / 2, 64), (kc[1] << 4) | (uint32_t)__shfl_xor(kc[1], LPR / 2, 64)};
+      vc = u32x2_t{(vc[0] << 4) | (uint32_t)__shfl_xor(vc[0], LPR / 2, 64), (vc[1] << 4) | (uint32_t)__shfl_xor(vc[1], LPR / 2, 64)};
+    }
     if (ok) {
-      *(u32x2_t*)(kc_row + (int64_t)wslot * a.kc_stride_t) = kc;
-      *(u32x2_t*)(vc_row + (int64_t)wslot * a.vc_stride_t) = vc;
+      if (stores) {
+        *(u32x2_t*)(kc_row + (int64_t)wslot * a.kc_stride_t) = kc;
+        *(u32x2_t*)(vc_row + (int64_t)wslot * a.vc_stride_t) = vc;
+      }
       if (col == 0) {
         a.k_scale[qs_row + wslot] = s1;
         a.k_zp[qs_row + wslot] = z1;
@@ -527,13 +539,14 @@ int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st) {
   const int64_t total = (int64_t)a.B * a.Hkv * a.num * (a.D / 8);
   if (total == 0) return KVX_OK;
   const unsigned grid = (unsigned)((total + NTHREADS - 1) / NTHREADS);
-  const bool u8 = a.kv_dtype == KVX_KV_U8;
   if (a.D == 128) {
-    if (u8) hipLaunchKernelGGL((cache_write_kernel<128, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else hipLaunchKernelGGL((cache_write_kernel<128, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
   } else {
-    if (u8) hipLaunchKernelGGL((cache_write_kernel<64, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else hipLaunchKernelGGL((cache_write_kernel<64, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
   }
   KVX_HIP(hipGetLastError());
   return KVX_OK;

@@ -140,7 +140,7 @@ struct QLoader {
   }
 };
 
-template <int D, bool U8>
+template <int D, int KV>
 __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParams p) {
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
     const int key = key0 + nt * 32 + n;
     const bool ok = key < p.kv_len;
     tpk[nt] = ok ? (p.tp ? p.tp[b * p.tp_sb + kvh * p.tp_sh + key] : key) : INT_MAX;
-    if constexpr (!U8) {
+    if constexpr (KV == KVX_KV_BF16) {
       const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st;
 #pragma unroll
       for (int j = 0; j < D / 16; ++j) {
@@ -174,7 +174,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
       const int32_t zp = ok ? p.k_zp[so] : 0;
 #pragma unroll
       for (int j = 0; j < D / 16; ++j) {
-        u32x2_t cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
+        u32x2_t cc;
+        if constexpr (KV == KVX_KV_U4) {  // chunk 2j + h of the row: one nibble of 8 bytes
+          cc = ok ? *(const u32x2_t*)(kp + u4_byte_off<D>(2 * j + h)) : u32x2_t{0, 0};
+          cc = u4_codes(cc, u4_shift<D>(2 * j + h));
+        } else {
+          cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
+        }
         u32x4_t t;
         t[0] = dequant_pair(cc[0] & 0xff, (cc[0] >> 8) & 0xff, zp, sc);
         t[1] = dequant_pair((cc[0] >> 16) & 0xff, cc[0] >> 24, zp, sc);
@@ -304,10 +310,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
   }
 }
 
-template <int D, bool U8>
+template <int D, int KV>
 int launch_t(const ScoreParams& p, hipStream_t st) {
   dim3 grid(p.B * p.Hkv, (p.kv_len + BK - 1) / BK);
-  hipLaunchKernelGGL((score_sum_kernel<D, U8>), grid, dim3(NTHREADS), 0, st, p);
+  hipLaunchKernelGGL((score_sum_kernel<D, KV>), grid, dim3(NTHREADS), 0, st, p);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
@@ -331,9 +337,14 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   p.k_sb = a.k_stride_b; p.k_sh = a.k_stride_h; p.k_st = a.k_stride_t;
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
-  const bool u8 = a.kv_dtype == KVX_KV_U8;
-  if (a.D == 128) return u8 ? launch_t<128, true>(p, st) : launch_t<128, false>(p, st);
-  if (a.D == 64) return u8 ? launch_t<64, true>(p, st) : launch_t<64, false>(p, st);
+  if (a.D == 128) {
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
+  }
+  if (a.D == 64) {
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
+  }
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128}", a.D);
 }
 

@@ -79,7 +79,7 @@ __device__ __forceinline__ float row_group_sum(float x) {
 constexpr float kNegBig = -1.0e30f;  // running maximum before the first key (finite: no inf - inf)
 constexpr float kRescaleSlack = 8.0f;  // the running maximum moves only when a logit exceeds it by this
 
-template <int D, int G, bool U8>
+template <int D, int G, int KV>
 __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p) {
   constexpr int LPR = D / 8;     // lanes per row: a lane owns 8 consecutive d
   constexpr int RPI = 64 / LPR;  // rows per load instruction of a wavefront
@@ -106,10 +106,13 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     for (int e = 0; e < 4; ++e) qv[g][e] = t[e];
   }
   // Rows are addressed as a uniform base plus a 32-bit byte offset (the host checks the range).
+  constexpr bool U8 = KV != KVX_KV_BF16;  // codes + row state (8-bit or 4-bit store)
+  constexpr bool U4 = KV == KVX_KV_U4;
   constexpr int ES = U8 ? 1 : 2;
   const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
   const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * ES;
-  const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES, lane_off = 8 * dc * ES;
+  const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES, lane_off = U4 ? u4_byte_off<D>(dc) : 8 * dc * ES;
+  const int nib = u4_shift<D>(dc);  // 4-bit store: which nibble holds this lane's 8 values
   const int64_t qs_off = b * p.qs_sb + kvh * p.qs_sh;
   float* lgrow = p.logits ? p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G : nullptr;
   int lg_base = k_begin;  // first key of the logits gathered in LDS
@@ -137,7 +140,8 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
       if constexpr (!U8) {
         r.k[u] = __builtin_nontemporal_load((const u32x4_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
       } else {
-        const u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
+        u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
+        if constexpr (U4) c = u4_codes(c, nib);
         r.k[u] = u32x4_t{c[0], c[1], 0, 0};
         r.ks[u] = p.k_scale[qs_off + key];
         r.kz[u] = p.k_zp[qs_off + key];
@@ -149,7 +153,8 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
       if constexpr (!U8) {
         r.v[u] = __builtin_nontemporal_load((const u32x4_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
       } else {
-        const u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
+        u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
+        if constexpr (U4) c = u4_codes(c, nib);
         r.v[u] = u32x4_t{c[0], c[1], 0, 0};
         r.vs[u] = p.v_scale[qs_off + key];
         r.vz[u] = p.v_zp[qs_off + key];
@@ -475,10 +480,11 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
 }
 
 template <int D, int G>
-int launch_dg(const DecodeParams& p, bool u8, const kvx_h2o_args* hh, hipStream_t st) {
+int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
-  if (u8) hipLaunchKernelGGL((decode_split_kernel<D, G, true>), grid, dim3(NTHREADS), 0, st, p);
-  else hipLaunchKernelGGL((decode_split_kernel<D, G, false>), grid, dim3(NTHREADS), 0, st, p);
+  if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p);
+  else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p);
+  else hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p);
   KVX_HIP(hipGetLastError());
   hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
   KVX_HIP(hipGetLastError());
@@ -498,12 +504,12 @@ int launch_dg(const DecodeParams& p, bool u8, const kvx_h2o_args* hh, hipStream_
 }
 
 template <int D>
-int launch_d(const DecodeParams& p, int G, bool u8, const kvx_h2o_args* hh, hipStream_t st) {
+int launch_d(const DecodeParams& p, int G, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   switch (G) {
-    case 1: return launch_dg<D, 1>(p, u8, hh, st);
-    case 2: return launch_dg<D, 2>(p, u8, hh, st);
-    case 4: return launch_dg<D, 4>(p, u8, hh, st);
-    case 8: return launch_dg<D, 8>(p, u8, hh, st);
+    case 1: return launch_dg<D, 1>(p, kv, hh, st);
+    case 2: return launch_dg<D, 2>(p, kv, hh, st);
+    case 4: return launch_dg<D, 4>(p, kv, hh, st);
+    case 8: return launch_dg<D, 8>(p, kv, hh, st);
   }
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in {1, 2, 4, 8}", G);
 }
@@ -516,7 +522,7 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   const Plan pl = make_plan(a, hh != nullptr);
   KVX_REQUIRE(a.workspace && a.workspace_bytes >= pl.total, KVX_ERR_WORKSPACE,
               "kvx_sdpa_decode: workspace of %zu bytes needed, %zu given", pl.total, a.workspace_bytes);
-  const int64_t es = a.kv_dtype == KVX_KV_U8 ? 1 : 2;
+  const int64_t es = a.kv_dtype != KVX_KV_BF16 ? 1 : 2;
   KVX_REQUIRE((int64_t)a.kv_len * a.k_stride_t * es < (1ll << 32) && (int64_t)a.kv_len * a.v_stride_t * es < (1ll << 32), KVX_ERR_UNSUPPORTED,
               "kvx_sdpa_decode: one (batch, head) row set of K or V must span less than 4 GiB (kv_len %d, slot strides %lld / %lld)",
               a.kv_len, (long long)a.k_stride_t, (long long)a.v_stride_t);
@@ -542,9 +548,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.v_sb = a.v_stride_b; p.v_sh = a.v_stride_h; p.v_st = a.v_stride_t;
   p.o_sb = a.o_stride_b; p.o_sh = a.o_stride_h;
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
-  const bool u8 = a.kv_dtype == KVX_KV_U8;
-  if (a.D == 128) return launch_d<128>(p, pl.G, u8, hh, st);
-  if (a.D == 64) return launch_d<64>(p, pl.G, u8, hh, st);
+  if (a.D == 128) return launch_d<128>(p, pl.G, a.kv_dtype, hh, st);
+  if (a.D == 64) return launch_d<64>(p, pl.G, a.kv_dtype, hh, st);
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128}", a.D);
 }
 

@@ -31,7 +31,7 @@ constexpr float kSlackLog2 = 8.0f;  // see the running-maximum update in the ker
 // Wavefronts per workgroup, 32 rows each. The uint8 cache takes 8: a tile is dequantised once per
 // workgroup, so twice the rows halve that vector work per row (-13 % kernel time); for bf16 tiles the
 // two sizes run alike and the smaller one leaves more workgroups for short chunks.
-constexpr int nwaves(bool u8) { return u8 ? 8 : 4; }
+constexpr int nwaves(int kv) { return kv != 0 ? 8 : 4; }  // kv: enum kvx_kv_dtype
 constexpr int BN = 64;   // keys per tile
 
 struct PrefillParams {
@@ -120,8 +120,10 @@ __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp
 // workgroup takes row groups w, w + 4, ... of the 64-row tile (NI groups each for K and for V).
 // bf16 cache: DMA into LDS. uint8 cache: codes and row state go through registers (prefetched one
 // tile ahead like the DMA), are dequantised to bf16 and written to the same LDS layout.
-template <int D, bool U8>
+template <int D, int KV>
 struct Loader {
+  static constexpr bool U8 = KV != KVX_KV_BF16;  // codes through registers (8-bit or 4-bit store)
+  static constexpr bool U4 = KV == KVX_KV_U4;
   static constexpr int CPR = D / 8;
   static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
   static constexpr int NWAVES = nwaves(U8);
@@ -139,6 +141,7 @@ struct Loader {
   int64_t k_tile_bytes, v_tile_bytes, k_st, v_st;
   int64_t k_step, v_step;       // bytes between this wavefront's consecutive row groups (NWAVES RPW rows)
   int wave, lane, kv_len, rl, cgk, cgv;
+  int shk, shv;                 // 4-bit store: nibble of this lane's K / V chunk (4 = high)
   uint32_t lds_k, lds_v;        // LDS addresses of the K and V buffers (wavefront-uniform)
   // uint8 path staging registers
   u32x2_t kc[NI], vc[NI];
@@ -146,6 +149,8 @@ struct Loader {
   int32_t kzr[NI], vzr[NI];
 
   __device__ __forceinline__ int row_of(int i) const { return (NWAVES * i + wave) * RPW + rl; }
+  // byte offset of chunk c (8 values) inside a row
+  __device__ __forceinline__ static uint32_t chunk_off(int c) { return U4 ? u4_byte_off<D>(c) : (uint32_t)(c * 8 * ESZ); }
 
   __device__ __forceinline__ void init(const PrefillParams& p, Smem<D>& sm, int b, int kvh, int tid) {
     lds_k = __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.k[0][0][0]));
@@ -171,8 +176,10 @@ struct Loader {
     const int r = row_of(0);
     cgk = (lane % CPR) ^ swz_k<CPR>(r);  // the chunk that belongs at LDS position lane % CPR of row r
     cgv = (lane % CPR) ^ swz_v<CPR>(r);
-    koff = (uint32_t)(r * p.k_st * ESZ + cgk * 8 * ESZ);
-    voff = (uint32_t)(r * p.v_st * ESZ + cgv * 8 * ESZ);
+    koff = (uint32_t)(r * p.k_st * ESZ + chunk_off(cgk));
+    voff = (uint32_t)(r * p.v_st * ESZ + chunk_off(cgv));
+    shk = u4_shift<D>(cgk);
+    shv = u4_shift<D>(cgv);
     k_step = (int64_t)NWAVES * RPW * p.k_st * ESZ;
     v_step = (int64_t)NWAVES * RPW * p.v_st * ESZ;
   }
@@ -204,7 +211,7 @@ struct Loader {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int key = min(key0 + row_of(i), kv_len - 1);
-        const uint32_t off = (uint32_t)(((int64_t)(key - key0) * st + (IS_K ? cgk : cgv) * 8) * ESZ);
+        const uint32_t off = (uint32_t)((int64_t)(key - key0) * st * ESZ) + chunk_off(IS_K ? cgk : cgv);
         if constexpr (!U8) {
           const uint32_t dst = (IS_K ? lds_k : lds_v) + (uint32_t)((buf * BN + (NWAVES * i + wave) * RPW) * CPR * 16);
           dma16(tb, off, dst);
@@ -231,8 +238,10 @@ struct Loader {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int r = row_of(i);
-        if (IS_K) sm.k[buf][r][lane % CPR] = dequant8(kc[i][0], kc[i][1], kzr[i], ksr[i]);
-        else sm.v[buf][r][lane % CPR] = dequant8(vc[i][0], vc[i][1], vzr[i], vsr[i]);
+        u32x2_t c = IS_K ? kc[i] : vc[i];
+        if constexpr (U4) c = u4_codes(c, IS_K ? shk : shv);
+        if (IS_K) sm.k[buf][r][lane % CPR] = dequant8(c[0], c[1], kzr[i], ksr[i]);
+        else sm.v[buf][r][lane % CPR] = dequant8(c[0], c[1], vzr[i], vsr[i]);
       }
     }
     if (IS_K && tid < BN) {
@@ -243,9 +252,9 @@ struct Loader {
   }
 };
 
-template <int D, bool U8>
-__global__ __launch_bounds__(64 * nwaves(U8), U8 ? 1 : 2) void sdpa_prefill_kernel(const PrefillParams p) {
-  constexpr int BM = 32 * nwaves(U8);  // rows per workgroup
+template <int D, int KV>
+__global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill_kernel(const PrefillParams p) {
+  constexpr int BM = 32 * nwaves(KV);  // rows per workgroup
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;  // k-steps of the first product
   constexpr int DT = D / 32;  // d tiles of the second product
@@ -391,7 +400,7 @@ __global__ __launch_bounds__(64 * nwaves(U8), U8 ? 1 : 2) void sdpa_prefill_kern
   // to O while the vector ALU turns S(t) into P(t). K(t) sits in k[t & 1]; V(t-1) in v[(t-1) & 1];
   // K(t+1) and V(t) are in flight to the other buffers and are published by the barrier that ends
   // the iteration.
-  Loader<D, U8> ld;
+  Loader<D, KV> ld;
   ld.init(p, sm, b, kvh, tid);
   uint32_t pb_prev[2][8];
   // every split owns at least one tile (the host sizes the splits that way)
@@ -556,7 +565,7 @@ int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
   // Aim for one resident round of workgroups (2 per compute unit, 1 with the uint8 cache): more
   // splits only add partials to write, merge and re-read. At least 8 key tiles per split.
   const int64_t base = (int64_t)a.B * a.Hkv * m_blocks;
-  const int target = (a.kv_dtype == KVX_KV_U8 ? 1 : 2) * num_cus();
+  const int target = (a.kv_dtype != KVX_KV_BF16 ? 1 : 2) * num_cus();
   int s = (int)((target + base - 1) / base);
   s = max(1, min(s, num_tiles / 8));
   return max(1, min(s, 64));
@@ -582,7 +591,7 @@ void fill_params(PrefillParams& p, const kvx_sdpa_args& a) {
   p.R = a.q_len * p.G;
   p.input_pos = a.input_pos;
   p.num_tiles = (a.kv_len + BN - 1) / BN;
-  const int bm = 32 * nwaves(a.kv_dtype == KVX_KV_U8);
+  const int bm = 32 * nwaves(a.kv_dtype);
   p.m_blocks = (p.R + bm - 1) / bm;
   p.num_splits = pick_splits(a, p.m_blocks, p.num_tiles);
   p.tiles_per_split = (p.num_tiles + p.num_splits - 1) / p.num_splits;
@@ -604,10 +613,10 @@ size_t partial_bytes(const PrefillParams& p, int D) {
   return rows * (size_t)D * 4 + rows * 2 * 4;
 }
 
-template <int D, bool U8>
+template <int D, int KV>
 int launch_t(PrefillParams& p, hipStream_t st) {
   dim3 grid(p.B * p.Hkv, p.m_blocks, p.num_splits);
-  hipLaunchKernelGGL((sdpa_prefill_kernel<D, U8>), grid, dim3(64 * nwaves(U8)), 0, st, p);
+  hipLaunchKernelGGL((sdpa_prefill_kernel<D, KV>), grid, dim3(64 * nwaves(KV)), 0, st, p);
   KVX_HIP(hipGetLastError());
   if (p.num_splits > 1) {
     constexpr int ROWS = 256 / (D / 4);
@@ -637,9 +646,14 @@ int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {
     p.part_o = (float*)a.workspace;
     p.part_ml = p.part_o + rows * (size_t)a.D;
   }
-  const bool u8 = a.kv_dtype == KVX_KV_U8;
-  if (a.D == 128) return u8 ? launch_t<128, true>(p, st) : launch_t<128, false>(p, st);
-  if (a.D == 64) return u8 ? launch_t<64, true>(p, st) : launch_t<64, false>(p, st);
+  if (a.D == 128) {
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
+  }
+  if (a.D == 64) {
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
+  }
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_prefill: head size %d not in {64, 128}", a.D);
 }
 

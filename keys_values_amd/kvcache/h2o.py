@@ -10,8 +10,9 @@ One ``forward`` is, in the reference's order (keys_values/kvcache/base.py:554-59
 tokens into the slots chosen last time (resetting their score), attend over the cache with the
 position mask, add the score-sums to the cumulative scores, choose the next slots to evict.
 
-The K/V store is either bf16 (``h2o-default``) or uint8 codes with per-row scale / zero point
-(``h2o-torch-quantized8``, keys_values/kvcache/factory.py:50-66). In the second case the codes stay
+The K/V store is either bf16 (``h2o-default``) or codes with per-row scale / zero point: 8 bits
+(``h2o-torch-quantized8``) or 4 bits, two codes per byte (``h2o-torch-quantized4``;
+keys_values/kvcache/factory.py:50-66). In the second case the codes stay
 resident and the attention kernels dequantise them on load; the reference instead dequantises the
 whole cache into a bf16 working buffer per layer and re-quantises it afterwards
 (keys_values/kvcache/quant_buffers.py:473-503,732-804).
@@ -23,7 +24,7 @@ the Q-Hitter combination with the quantisation error (``QuantizedH2OKVCache`` /
 ``QuantizedVLengthH2OKVCache``, keys_values/kvcache/qh2o.py). ``create_kv_cache`` takes the names of
 keys_values/kvcache/factory.py:50-66.
 
-Not covered (raises): replay log, fp16/fp32 caches, 4-bit and bitsandbytes stores.
+Not covered (raises): replay log, fp16/fp32 caches, bitsandbytes stores, quantisation blocks over heads.
 """
 import ctypes
 from dataclasses import dataclass
@@ -59,6 +60,7 @@ class H2OKVCache:
         normalize_scores: bool = False,
         grace_period: int = 0,
         quantized: bool = False,
+        num_bits: int = 8,
         keep_initial_fraction: float = DEFAULT_KEEP_INITIAL_FRACTION,
         device: Optional[torch.device] = None,
         v_length: bool = False,
@@ -67,6 +69,8 @@ class H2OKVCache:
     ):
         if not (0 <= grace_period < params.cache_length):  # keys_values/kvcache/attn_weights.py:440-444
             raise ValueError(f"grace_period = {grace_period}, must be in [0, {params.cache_length})")
+        if num_bits not in (4, 8):  # keys_values/kvcache/quantize/pytorch.py:191-192
+            raise ValueError(f"num_bits = {num_bits}, must be 4 or 8")
         if q_hitter and not quantized:  # keys_values/kvcache/qh2o.py:95-96
             raise TypeError("the quantisation-error policy needs the quantised store")
         if not (0 <= combination_constant <= 1):  # keys_values/kvcache/qh2o.py:97-100
@@ -91,6 +95,7 @@ class H2OKVCache:
         self.combination_constant = combination_constant
         self.normalize_scores = normalize_scores
         self.quantized = quantized
+        self.num_bits = num_bits if quantized else None
         # keys_values/kvcache/attn_weights.py:458-462: silently disabled when too large
         if max_chunk_size is not None and max_chunk_size > self.cache_length // 2:
             max_chunk_size = None
@@ -103,8 +108,9 @@ class H2OKVCache:
             raise RuntimeError(f"H2OKVCache buffers live on a ROCm device, not on {self.device}: there is no CPU path")
         b, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
         kv_dtype = torch.uint8 if quantized else torch.bfloat16
-        self.k = torch.zeros((b, h, length, d), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
-        self.v = torch.zeros((b, h, length, d), dtype=kv_dtype, device=self.device)
+        row = d // 2 if (quantized and num_bits == 4) else d  # the 4-bit store packs two codes per byte
+        self.k = torch.zeros((b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
+        self.v = torch.zeros((b, h, length, row), dtype=kv_dtype, device=self.device)
         if quantized:
             self.k_scale = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)
             self.k_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
@@ -267,7 +273,7 @@ class H2OKVCache:
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, self.head_size, self.cache_length
         a.input_pos = input_pos
-        a.kv_dtype = _lib.KVX_KV_U8 if self.quantized else _lib.KVX_KV_BF16
+        a.kv_dtype = (_lib.KVX_KV_U4 if self.num_bits == 4 else _lib.KVX_KV_U8) if self.quantized else _lib.KVX_KV_BF16
         a.index = index.data_ptr()
         a.index_stride_b, a.index_stride_h = index.stride(0), index.stride(1)
         a.key = key.data_ptr()
@@ -418,17 +424,17 @@ class QuantizedVLengthH2OKVCache(H2OKVCache):
 
 
 _CACHE_TYPES = {"h2o": H2OKVCache, "h2o-vlen": VLengthH2OKVCache, "qh2o": QuantizedH2OKVCache, "qh2o-vlen": QuantizedVLengthH2OKVCache}
-_STORES = {"default": False, "torch-quantized8": True}
+_STORES = {"default": (False, 8), "torch-quantized8": (True, 8), "torch-quantized4": (True, 4)}
 
 
 def create_kv_cache(name: str, params: KVCacheParams, **kwargs) -> H2OKVCache:
     """``<policy>-<store>`` as in keys_values/kvcache/factory.py:50-66 (``h2o-default``,
     ``h2o-vlen-torch-quantized8``, ``qh2o-torch-quantized8`` ...). Policies other than the H2O family
     and stores other than bf16 / 8-bit raise."""
-    for store, quantized in _STORES.items():
+    for store, (quantized, num_bits) in _STORES.items():
         if name.endswith("-" + store):
             policy = name[: -len(store) - 1]
             if policy not in _CACHE_TYPES:
                 raise NotImplementedError(f"cache policy '{policy}' is not implemented; have {sorted(_CACHE_TYPES)}")
-            return _CACHE_TYPES[policy](params, quantized=quantized, **kwargs)
+            return _CACHE_TYPES[policy](params, quantized=quantized, num_bits=num_bits, **kwargs)
     raise NotImplementedError(f"cache name '{name}': store must be one of {sorted(_STORES)}")

@@ -84,7 +84,7 @@ class PolicyCacheOracle:
     (keys_values/kvcache/base.py:554-595): write (with the ring move) -> attend -> score -> select."""
 
     def __init__(self, B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=None, grace_period=0, normalize_scores=False,
-                 v_length=False, q_hitter=False, combination_constant=0.5, quantized=False):
+                 v_length=False, q_hitter=False, combination_constant=0.5, quantized=False, num_bits=8):
         assert 0 <= grace_period < L
         assert not q_hitter or quantized  # keys_values/kvcache/qh2o.py:95-96
         self.B, self.Hq, self.Hkv, self.L, self.D = B, Hq, Hkv, L, D
@@ -102,6 +102,7 @@ class PolicyCacheOracle:
         self.normalize_scores = normalize_scores
         self.v_length, self.q_hitter, self.c = v_length, q_hitter, combination_constant
         self.quantized = quantized
+        self.num_bits = num_bits
         self.input_pos = 0
         self.current_length = 0
         self.prefill_length = 0
@@ -120,7 +121,7 @@ class PolicyCacheOracle:
         x = x.to(self.dtype)
         if not self.quantized:
             return x
-        c, s, z = quantize_rows(x)
+        c, s, z = quantize_rows(x, self.num_bits)
         return dequantize_rows(c, s, z, self.dtype)
 
     def _initial_scores(self, key, value):
@@ -129,7 +130,8 @@ class PolicyCacheOracle:
         if self.v_length:
             init["v_norm"] = torch.linalg.vector_norm(value, dim=-1, dtype=torch.float32)
         if self.q_hitter:
-            init["q_errors"] = quantization_error(key).to(torch.float32) + quantization_error(value).to(torch.float32)
+            init["q_errors"] = (quantization_error(key, self.num_bits).to(torch.float32)
+                                + quantization_error(value, self.num_bits).to(torch.float32))
         return init
 
     # -- prefill (keys_values/kvcache/attn_weights.py:817-869) ---------------------------------------

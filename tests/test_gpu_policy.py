@@ -33,8 +33,9 @@ def _store(cache):
     """What the cache holds, as bf16 rows."""
     if not cache.quantized:
         return cache.k.cpu(), cache.v.cpu()
-    return (O.dequantize_rows(cache.k.cpu(), cache.k_scale.cpu(), cache.k_zp.cpu()),
-            O.dequantize_rows(cache.v.cpu(), cache.v_scale.cpu(), cache.v_zp.cpu()))
+    unpack = O.uncompress4 if cache.num_bits == 4 else (lambda c: c)
+    return (O.dequantize_rows(unpack(cache.k.cpu()), cache.k_scale.cpu(), cache.k_zp.cpu()),
+            O.dequantize_rows(unpack(cache.v.cpu()), cache.v_scale.cpu(), cache.v_zp.cpu()))
 
 
 def _run_steps(gpu, cache, ref, q, k, v, n_prefill, steps):
@@ -105,6 +106,8 @@ def test_grace_period_steps(gpu, quantized):
     ("h2o-vlen-torch-quantized8", dict(grace_period=9, normalize_scores=True)),
     ("qh2o-torch-quantized8", dict(combination_constant=0.3)),
     ("qh2o-vlen-torch-quantized8", dict(grace_period=16, normalize_scores=True)),
+    ("h2o-torch-quantized4", dict()),
+    ("qh2o-vlen-torch-quantized4", dict(grace_period=16)),
 ])
 def test_policy_variants_chunked_steps(gpu, name, kwargs):
     B, Hq, Hkv, L, D, chunk = 2, 8, 2, 384, 128, 32
@@ -113,7 +116,8 @@ def test_policy_variants_chunked_steps(gpu, name, kwargs):
     cache = create_kv_cache(name, KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, device=gpu, **kwargs)
     ref = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, quantized=cache.quantized, v_length=cache.v_length,
                               q_hitter=cache.q_hitter, combination_constant=cache.combination_constant,
-                              grace_period=cache.grace_period, normalize_scores=cache.normalize_scores)
+                              grace_period=cache.grace_period, normalize_scores=cache.normalize_scores,
+                              num_bits=cache.num_bits or 8)
     _run_steps(gpu, cache, ref, q, k, v, L, steps)
 
 
@@ -122,6 +126,7 @@ def test_policy_variants_chunked_steps(gpu, name, kwargs):
     (QuantizedH2OKVCache, dict(grace_period=5)),
     (QuantizedVLengthH2OKVCache, dict(normalize_scores=True)),
     (H2OKVCache, dict(grace_period=7)),
+    (H2OKVCache, dict(quantized=True, num_bits=4, grace_period=3)),
 ])
 def test_policy_variants_single_token_steps(gpu, cls, kwargs):
     # max_chunk_size = 1: the argmin form of the selection (and, for plain H2O, the fused decode step)
@@ -131,7 +136,8 @@ def test_policy_variants_single_token_steps(gpu, cls, kwargs):
     cache = cls(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, device=gpu, **kwargs)
     ref = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=1, quantized=cache.quantized, v_length=cache.v_length,
                               q_hitter=cache.q_hitter, combination_constant=cache.combination_constant,
-                              grace_period=cache.grace_period, normalize_scores=cache.normalize_scores)
+                              grace_period=cache.grace_period, normalize_scores=cache.normalize_scores,
+                              num_bits=cache.num_bits or 8)
     _run_steps(gpu, cache, ref, q, k, v, L, steps)
 
 

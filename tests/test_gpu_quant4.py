@@ -139,3 +139,50 @@ def test_blocks_over_heads_store_feeds_attention(gpu):
     torch.cuda.synchronize()
     assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
     torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,q_len,T,D", [(1, 8, 2, 96, 2048 + 40, 128), (2, 4, 4, 33, 515, 64), (1, 8, 1, 1, 3000, 128)])
+def test_attention_over_4bit_cache(kvx, gpu, B, Hq, Hkv, q_len, T, D):
+    """Attention output, score-sums (prefill kernel + score-sum kernel) and single-token decode over the
+    4-bit store, the nibbles unpacked and dequantised inside the kernels, against the oracle run on
+    the dequantised bf16 rows. Scattered token positions."""
+    import math
+
+    from helpers import rel_err, scattered_positions
+    from keys_values_amd.attention import ops
+
+    gen = torch.Generator().manual_seed(T)
+    k = outlier_rows(2, B * Hkv * T, D).view(B, Hkv, T, D)
+    v = torch.randn(B, Hkv, T, D, generator=gen).to(torch.bfloat16)
+    q = torch.randn(B, Hq, q_len, D, generator=gen).to(torch.bfloat16)
+    input_pos = T + 100
+    tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len)
+    st = _lib.stream_ptr(gpu)
+
+    def pack(x):
+        xg = x.reshape(-1, D).to(gpu)
+        rows = xg.shape[0]
+        c = torch.empty((rows, D // 2), dtype=torch.uint8, device=gpu)
+        s = torch.empty(rows, dtype=torch.float32, device=gpu)
+        z = torch.empty(rows, dtype=torch.int32, device=gpu)
+        _lib.check(kvx.kvx_quantize_rows4(xg.data_ptr(), D, rows, D, c.data_ptr(), s.data_ptr(), z.data_ptr(), st))
+        return c.view(B, Hkv, T, D // 2), s.view(B, Hkv, T), z.view(B, Hkv, T)
+
+    kc, ks, kz = pack(k)
+    vc, vs, vz = pack(v)
+    quant = ops.QuantState(ks, kz, vs, vz)
+    kd = O.dequantize_rows(*O.quantize_rows(k, 4))
+    vd = O.dequantize_rows(*O.quantize_rows(v, 4))
+    scale = 1 / math.sqrt(D)
+    if q_len > 1:
+        o_ref, w_ref = O.sdpa_in_blocks(q, kd, vd, scale, input_pos, tp.long())
+        out, w, _ = ops.prefill_core(q.to(gpu), kc, vc, scale, input_pos, tp.to(gpu), return_weights=True, quant=quant,
+                                     output_transposed=False)
+        torch.cuda.synchronize()
+        assert rel_err(out.float().cpu(), o_ref.float()) < 2e-2
+        torch.testing.assert_close(w.cpu(), w_ref, rtol=1e-3, atol=1e-6)
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], kd, vd, scale, 10 * T, None)
+    out1, w1, _ = ops.decode_core(q[:, :, :1].to(gpu), kc, vc, scale, return_weights=True, quant=quant)
+    torch.cuda.synchronize()
+    assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
+    torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
