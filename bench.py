@@ -60,9 +60,9 @@ def parse():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
     ap.add_argument("--tokens", type=int, default=131072, help="longctx: prompt length")
-    ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8"],
+    ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8", "uint4"],
                     help="cache storage for the prefill / decode workloads; uint8 = BASELINE.json configs[2]: codes + per-row "
-                         "scale and zero point, dequantised inside the attention kernels")
+                         "scale and zero point, dequantised inside the attention kernels; uint4 = the 4-bit store of the same quantiser")
     return ap.parse_args()
 
 
@@ -84,7 +84,8 @@ def bench_prefill(args, torch, dev):
     from oracle import kvx_oracle as O
 
     lib = _lib.load()
-    u8 = args.kv == "uint8"
+    u8 = args.kv != "bf16"   # a quantised store: codes + row state
+    u4 = args.kv == "uint4"
     (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev, 65536 if u8 else 32768, 2 if u8 else 1)
     scale = D ** -0.5
     q, k, v = q_c.to(dev), k_c.to(dev), v_c.to(dev)
@@ -92,17 +93,19 @@ def bench_prefill(args, torch, dev):
     if u8:
         # quantise with the library's own kernel; the CPU sample below attends over the dequantised rows
         def quantise(x):
-            c = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+            c = torch.empty(x.shape[:-1] + (D // 2 if u4 else D,), dtype=torch.uint8, device=dev)
             sc = torch.empty(x.shape[:-1], dtype=torch.float32, device=dev)
             zp = torch.empty(x.shape[:-1], dtype=torch.int32, device=dev)
-            _lib.check(lib.kvx_quantize_rows(x.data_ptr(), D, x.numel() // D, D, c.data_ptr(), sc.data_ptr(), zp.data_ptr(), _lib.stream_ptr(dev)))
+            fn = lib.kvx_quantize_rows4 if u4 else lib.kvx_quantize_rows
+            _lib.check(fn(x.data_ptr(), D, x.numel() // D, D, c.data_ptr(), sc.data_ptr(), zp.data_ptr(), _lib.stream_ptr(dev)))
             return c, sc, zp
         k, ksc, kzp = quantise(k)
         v, vsc, vzp = quantise(v)
         quant = ops.QuantState(ksc, kzp, vsc, vzp)
         torch.cuda.synchronize()
-        k_c = O.dequantize_rows(k.cpu(), ksc.cpu(), kzp.cpu())
-        v_c = O.dequantize_rows(v.cpu(), vsc.cpu(), vzp.cpu())
+        unpack = O.uncompress4 if u4 else (lambda c: c)
+        k_c = O.dequantize_rows(unpack(k.cpu()), ksc.cpu(), kzp.cpu())
+        v_c = O.dequantize_rows(unpack(v.cpu()), vsc.cpu(), vzp.cpu())
     out = torch.empty((B, q_len, Hq, D), dtype=torch.bfloat16, device=dev)
     o_view = out.permute(0, 2, 1, 3)
     lse = torch.empty((B, q_len, Hq), dtype=torch.float32, device=dev)
@@ -214,7 +217,7 @@ def bench_prefill(args, torch, dev):
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": ("BASELINE.json configs[2]: attention + score-sum over the uint8 cache (dequantised in the kernels), B1 Hq32 Hkv8 D128 T65536 q1024, seed 2"
+            "workload": (f"BASELINE.json configs[2]: attention + score-sum over the {args.kv} cache (dequantised in the kernels), B1 Hq32 Hkv8 D128 T65536 q1024, seed 2"
                          if u8 else
                          "BASELINE.json configs[1]: chunked prefill attention + score-sum, B1 Hq32 Hkv8 D128 T32768 q1024, RoPE theta 1e6, seed 1"),
             "flops_algorithmic": flops_alg,
@@ -229,7 +232,7 @@ def bench_prefill(args, torch, dev):
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "sdpa_prefill_kernel<128,%s> (+ split merge)" % ("true" if u8 else "false"),
+            "kernel": "sdpa_prefill_kernel<128,%s> (+ split merge)" % {"bf16": "KVX_KV_BF16", "uint8": "KVX_KV_U8", "uint4": "KVX_KV_U4"}[args.kv],
             "achieved": round(attn_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
@@ -303,16 +306,18 @@ def bench_decode(args, torch, dev):
 
     B, Hq, Hkv, L, D = 8, 32, 8, 131072, 128
     gen = torch.Generator(device=dev).manual_seed(3)
-    u8 = args.kv == "uint8"
-    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, quantized=u8, device=dev)
+    u8 = args.kv != "bf16"
+    u4 = args.kv == "uint4"
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=1, quantized=u8, num_bits=4 if u4 else 8, device=dev)
     # state as after a prefill that filled the cache (the prefill itself is not part of this workload)
     if u8:
         lib = _lib.load()
         for codes, sc, zp in ((cache.k, cache.k_scale, cache.k_zp), (cache.v, cache.v_scale, cache.v_zp)):
             for bi in range(B):  # one batch row at a time keeps the bf16 temporaries small
-                x = torch.randn(codes[bi].shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
-                _lib.check(lib.kvx_quantize_rows(x.data_ptr(), D, x.numel() // D, D, codes[bi].data_ptr(), sc[bi].data_ptr(),
-                                                 zp[bi].data_ptr(), _lib.stream_ptr(dev)))
+                x = torch.randn((Hkv, L, D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                fn = lib.kvx_quantize_rows4 if u4 else lib.kvx_quantize_rows
+                _lib.check(fn(x.data_ptr(), D, x.numel() // D, D, codes[bi].data_ptr(), sc[bi].data_ptr(),
+                              zp[bi].data_ptr(), _lib.stream_ptr(dev)))
             torch.cuda.synchronize()
     else:
         cache.k.copy_(torch.randn(cache.k.shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16))
@@ -340,7 +345,7 @@ def bench_decode(args, torch, dev):
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     ms_gpu = e0.elapsed_time(e1) / args.steps
     # K + V once (bf16 rows, or codes + 8 bytes of row state), scores read-modify-write
-    bytes_alg = 2 * B * Hkv * L * (D + 8 if u8 else 2 * D) + 2 * B * Hkv * L * 4
+    bytes_alg = 2 * B * Hkv * L * ((D // 2 if u4 else D) + 8 if u8 else 2 * D) + 2 * B * Hkv * L * 4
     gbs = bytes_alg / (ms_step * 1e-3) / 1e9
     # the dominant launch alone: the fused attention + score update + argmin call (split attention,
     # merge, weights kernels), events on the launch stream around each call
@@ -359,8 +364,9 @@ def bench_decode(args, torch, dev):
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         nb = B  # the attention of one whole step
         if u8:
-            kc = O.dequantize_rows(cache.k[:nb].cpu(), cache.k_scale[:nb].cpu(), cache.k_zp[:nb].cpu())
-            vc = O.dequantize_rows(cache.v[:nb].cpu(), cache.v_scale[:nb].cpu(), cache.v_zp[:nb].cpu())
+            unpack = O.uncompress4 if u4 else (lambda c: c)
+            kc = O.dequantize_rows(unpack(cache.k[:nb].cpu()), cache.k_scale[:nb].cpu(), cache.k_zp[:nb].cpu())
+            vc = O.dequantize_rows(unpack(cache.v[:nb].cpu()), cache.v_scale[:nb].cpu(), cache.v_zp[:nb].cpu())
         else:
             kc, vc = cache.k[:nb].cpu(), cache.v[:nb].cpu()
         qc = qs[0, :nb].cpu()
@@ -374,10 +380,10 @@ def bench_decode(args, torch, dev):
         "metric": "decode + H2O step GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3" + (", uint8 cache" if u8 else ""),
+        "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3" + (f", {args.kv} cache" if u8 else ""),
                    "bytes_algorithmic_per_step": bytes_alg, "ms_per_step_gpu_events": round(ms_gpu, 4),
                    "decode_tokens_per_s": round(B / (ms_step * 1e-3), 1)},
-        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + merge + weights/score update/argmin" % ("true" if u8 else "false"),
+        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + merge + weights/score update/argmin" % {"bf16": "KVX_KV_BF16", "uint8": "KVX_KV_U8", "uint4": "KVX_KV_U4"}[args.kv],
                      "achieved": round(bytes_alg / (ms_call * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(bytes_alg / (ms_call * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "ms_per_launch": round(ms_call, 4),
                      "traffic": None if u8 else TRAFFIC_BYTES["decode"]},
