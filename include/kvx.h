@@ -229,6 +229,8 @@ int kvx_dequantize_blocks(const kvx_block_quant_args* args, void* stream);
  * A moved row of a uint8 cache keeps its codes, scale and zero point (the reference dequantises and
  * re-quantises it, which is not the identity). Slots in index must lie outside the ring.
  *
+ * replay_log (see the field comments) records the slots written.
+ *
  * Further score buffers, same layout and strides as scores, NULL if the policy has none:
  *   v_norm   |value row|_2 in fp32 (VLengthInstantScoreMixin._initial_scores_in_forward,
  *            keys_values/kvcache/h2o.py:316-341);
@@ -264,6 +266,15 @@ typedef struct kvx_cache_write_args {
   const int32_t* grace_slots; /* (grace_num) ring slots, shared by all (b, h) */
   float* v_norm;              /* (B, Hkv, cache_len) by sc_stride_*, or NULL */
   float* q_errors;            /* (B, Hkv, cache_len) by sc_stride_*, or NULL */
+  /* Replay log (AttnWeightsReplayLog.append_position_index, keys_values/kvcache/attn_weights.py:125-151):
+   * the slots index[b,h,j] this call writes to are recorded as uint32, entry p = log_pos + j of
+   * (b, h) at replay_log[(p / log_blocksize) * log_stride_block + b * log_stride_b + h * log_stride_h
+   * + p % log_blocksize]: blocks of log_blocksize positions, all blocks in one allocation.
+   * log_pos = input_pos - cache_length of the first new token. NULL: nothing is recorded. */
+  uint32_t* replay_log;
+  int32_t log_blocksize;
+  int64_t log_pos;
+  int64_t log_stride_block, log_stride_b, log_stride_h;
 } kvx_cache_write_args;
 int kvx_cache_write(const kvx_cache_write_args* args, void* stream);
 

@@ -47,6 +47,8 @@ class CacheWriteArgs(ctypes.Structure):
         ("scores", c_void_p), ("sc_stride_b", c_int64), ("sc_stride_h", c_int64),
         ("grace_num", c_int32), ("grace_period", c_int32), ("grace_slots", c_void_p),
         ("v_norm", c_void_p), ("q_errors", c_void_p),
+        ("replay_log", c_void_p), ("log_blocksize", c_int32), ("log_pos", c_int64),
+        ("log_stride_block", c_int64), ("log_stride_b", c_int64), ("log_stride_h", c_int64),
     ]
 
 

@@ -262,6 +262,8 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
                 "kvx_cache_write: need grace_num=%d <= grace_period=%d < cache_len=%d and input_pos=%d >= grace_period", a->grace_num,
                 a->grace_period, a->cache_len, a->input_pos);
   }
+  KVX_REQUIRE(!a->replay_log || (a->log_blocksize > 0 && a->log_pos >= 0), KVX_ERR_INVALID,
+              "kvx_cache_write: replay log needs log_blocksize > 0 and log_pos >= 0");
   KVX_REQUIRE(!a->q_errors || a->kv_dtype != KVX_KV_BF16, KVX_ERR_INVALID, "kvx_cache_write: q_errors needs a quantised cache");
   return launch_cache_write(*a, (hipStream_t)stream);
 }

@@ -453,6 +453,11 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   }
   float vnorm = 0.0f;
   if (a.v_norm) vnorm = row_norm<LPR>(vr);  // uniform branch: every lane takes part in the reduction
+  if (live && col == 0 && a.replay_log) {  // the slot as consumed, valid or not: the log mirrors index
+    const int64_t lp = a.log_pos + j;
+    a.replay_log[(lp / a.log_blocksize) * a.log_stride_block + b * a.log_stride_b + hh * a.log_stride_h + lp % a.log_blocksize] =
+        (uint32_t)slot;
+  }
   if (ok && col == 0) {
     a.token_pos[tp_row + wslot] = a.input_pos + src;
     if (a.scores) a.scores[sc_row + wslot] = 0.0f;

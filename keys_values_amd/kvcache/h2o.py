@@ -22,9 +22,10 @@ the most recent tokens, never evicted; keys_values/kvcache/attn_weights.py:267-3
 V-norm weighted instantaneous score (``VLengthH2OKVCache``, keys_values/kvcache/h2o.py:266-420) and
 the Q-Hitter combination with the quantisation error (``QuantizedH2OKVCache`` /
 ``QuantizedVLengthH2OKVCache``, keys_values/kvcache/qh2o.py). ``create_kv_cache`` takes the names of
-keys_values/kvcache/factory.py:50-66.
+keys_values/kvcache/factory.py:50-66. With ``switch_replay_logging(True)`` the cache records the token
+chunks and the slot every later token went to (keys_values/kvcache/attn_weights.py:43-204,939-966).
 
-Not covered (raises): replay log, fp16/fp32 caches, bitsandbytes stores, quantisation blocks over heads.
+Not covered (raises): fp16/fp32 caches, bitsandbytes stores, quantisation blocks over heads in the cache object.
 """
 import ctypes
 from dataclasses import dataclass
@@ -34,6 +35,7 @@ import torch
 
 from .. import _lib
 from ..attention import ops
+from .replay import DEFAULT_REPLAY_LOG_BLOCKSIZE, AttnWeightsReplayLog, ReplayArena
 
 DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
 DEFAULT_COMBINATION_CONSTANT = 0.5  # keys_values/kvcache/qh2o.py:25
@@ -66,7 +68,16 @@ class H2OKVCache:
         v_length: bool = False,
         q_hitter: bool = False,
         combination_constant: float = DEFAULT_COMBINATION_CONSTANT,
+        replay_log_blocksize: Optional[int] = None,
     ):
+        if replay_log_blocksize is None:  # keys_values/kvcache/attn_weights.py:436-441
+            replay_log_blocksize = DEFAULT_REPLAY_LOG_BLOCKSIZE
+        elif replay_log_blocksize <= 0:
+            raise ValueError(f"replay_log_blocksize must be positive, but got {replay_log_blocksize}")
+        self.replay_log_blocksize = replay_log_blocksize
+        self._log_on = False        # switch_replay_logging
+        self._log_chunks = None     # token chunks since the last prefill (None until a prefill was logged)
+        self._log_arena = None
         if not (0 <= grace_period < params.cache_length):  # keys_values/kvcache/attn_weights.py:440-444
             raise ValueError(f"grace_period = {grace_period}, must be in [0, {params.cache_length})")
         if num_bits not in (4, 8):  # keys_values/kvcache/quantize/pytorch.py:191-192
@@ -164,6 +175,40 @@ class H2OKVCache:
         idx = self._next_index_for(num, peek=True)
         return None if idx is None else idx.to(torch.int64)
 
+    # -- replay log (keys_values/kvcache/attn_weights.py:939-966) ---------------------------------------
+
+    def switch_replay_logging(self, status: bool):
+        self._log_on = bool(status)
+        if not status:
+            self._log_chunks, self._log_arena = None, None
+
+    @property
+    def do_replay_logging(self) -> bool:
+        return self._log_on
+
+    def get_replay_log(self) -> Optional[AttnWeightsReplayLog]:
+        """Token chunks and, for every token position >= cache_length, the slot it was written to."""
+        if not self._log_on:
+            return None
+        if self._log_chunks is None:
+            raise IndexError("Cannot switch on replay logging in the middle of inference run. Call 'prefill'.")
+        positions = max(self._input_pos - self.cache_length, 0)
+        blocks = self._log_arena.blocks(positions) if positions > 0 else []
+        return AttnWeightsReplayLog(list(self._log_chunks), blocks, self.cache_length, self.max_prefill_length,
+                                    self.replay_log_blocksize, self.grace_period)
+
+    def _log_token_chunk(self, token_idx: Optional[torch.Tensor], num: int, prefill: bool):
+        if not self._log_on:
+            return
+        if prefill:  # keys_values/kvcache/attn_weights.py:865-868: a prefill starts a new log
+            self._log_chunks = []
+            self._log_arena = ReplayArena(self.batch_size, self.n_query_groups, self.replay_log_blocksize, self.device)
+        elif self._log_chunks is None:  # :623-628
+            raise IndexError("Cannot switch on replay logging in the middle of inference run. Call 'prefill'.")
+        if token_idx is None or tuple(token_idx.shape) != (self.batch_size, num):
+            raise ValueError(f"token_idx must be given with shape {(self.batch_size, num)} while the replay log is on")
+        self._log_chunks.append(token_idx.detach().clone())  # keys_values/kvcache/base.py:844-855
+
     def _quant_state(self, T: int) -> Optional[ops.QuantState]:
         if not self.quantized:
             return None
@@ -199,7 +244,9 @@ class H2OKVCache:
             raise ValueError(f"shapes {tuple(query.shape)}, {tuple(key.shape)} do not fit the cache")
         input_pos = self._input_pos
         if input_pos == 0:
-            return self._prefill_step(query, key, value)
+            out = self._prefill_step(query, key, value)
+            self._log_token_chunk(token_idx, num, prefill=True)
+            return out
         if b != self.batch_size:
             raise ValueError(f"batch size {b} differs from the prefill batch size {self.batch_size}")
         if self._use_initial_rule is None:
@@ -212,6 +259,7 @@ class H2OKVCache:
         index = self._next_index_for(num)
         if index is None:
             raise IndexError("Cache needs to be initialized with 'prefill' before being used")
+        self._log_token_chunk(token_idx, num, prefill=False)
         self._write(index, key, value, input_pos)
         if diff > 0:
             self.current_length += num
@@ -293,6 +341,13 @@ class H2OKVCache:
         a.scores = self.scores.data_ptr()
         a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
         a.v_norm, a.q_errors = _lib.ptr(self.v_norm), _lib.ptr(self.q_errors)
+        if self._log_on and self._log_arena is not None and input_pos >= self.cache_length:
+            # keys_values/kvcache/attn_weights.py:629-633: the slots are recorded by the kernel that consumes them
+            log_pos = input_pos - self.cache_length
+            self._log_arena.reserve(log_pos + num)
+            arena = self._log_arena.data
+            a.replay_log, a.log_blocksize, a.log_pos = arena.data_ptr(), self.replay_log_blocksize, log_pos
+            a.log_stride_block, a.log_stride_b, a.log_stride_h = arena.stride(0), arena.stride(1), arena.stride(2)
         ring = None
         if self.grace_period > 0 and input_pos >= self.cache_length:
             # keys_values/kvcache/attn_weights.py:267-303: the num2 oldest ring slots move out to

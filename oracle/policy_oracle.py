@@ -12,6 +12,7 @@ Reference lines (paths relative to the reference root):
   scores, normalisation     keys_values/kvcache/h2o.py:146-199
   V-norm weighting          keys_values/kvcache/h2o.py:266-341
   Q-Hitter                  keys_values/kvcache/qh2o.py:130-210
+  replay log                keys_values/kvcache/attn_weights.py:43-204
 
 How it is pinned (tests/test_policy_oracle.py):
 * grace period: an independent model that keeps python objects per slot (no index arithmetic shared
@@ -23,6 +24,8 @@ How it is pinned (tests/test_policy_oracle.py):
 * Q-Hitter: combination constant 1 selects what plain H2O selects, constant 0 selects the rows with
   the largest quantisation error, the modified values stay in [(1 - c) / 2, 1], and the
   quantisation error is checked against explicit float loops.
+* Replay log: the concatenation of its blocks is the concatenation of every step's slots, and
+  ``extract_index`` is a slice of it, checked for every start and length on a small log.
 * A quantised store here holds dequantise(quantise(row)) for every row written; a row moved out of
   the ring keeps its stored value (the reference re-quantises the dequantised row when it writes the
   working buffer back, keys_values/kvcache/quant_buffers.py:732-775, which may change it by one
@@ -79,12 +82,74 @@ def update_select(scores, w, kv_len, limit, k, normalize=False, token_pos=None, 
     return select_smallest(s, k), s
 
 
+class ReplayLogOracle:
+    """keys_values/kvcache/attn_weights.py:43-204: slot positions of the tokens from cache_length on, in
+    blocks of `blocksize` positions (a list that grows block by block); token chunks beside them."""
+
+    def __init__(self, cache_length: int, blocksize: int):
+        self.cache_length, self.blocksize = cache_length, blocksize
+        self.token_chunks = []
+        self.blocks = []
+
+    def append_token_chunk(self, chunk):  # keys_values/kvcache/base.py:844-855
+        self.token_chunks.append(chunk.clone())
+
+    def append_position_index(self, index: torch.Tensor, input_pos: int):  # :125-151
+        bs = self.blocksize
+        shape = index.shape[:2] + (bs,)
+        bstart = (input_pos - self.cache_length) % bs
+        if bstart == 0:
+            self.blocks.append(torch.zeros(shape, dtype=torch.int64))
+        block = self.blocks[-1]
+        num = index.shape[2]
+        bend = min(bstart + num, bs)
+        iend = bend - bstart
+        block[:, :, bstart:bend] = index[:, :, :iend]
+        while iend < num:
+            istart = iend
+            block = torch.zeros(shape, dtype=torch.int64)
+            self.blocks.append(block)
+            bend = min(num - istart, bs)
+            iend = istart + bend
+            block[:, :, :bend] = index[:, :, istart:iend]
+
+    def finalize(self, input_pos: int):  # :102-123: the last block cut to the positions in use
+        if input_pos <= self.cache_length:
+            return []
+        end = (input_pos - self.cache_length) % self.blocksize
+        if end == 0:
+            return list(self.blocks)
+        return self.blocks[:-1] + [self.blocks[-1][:, :, :end]]
+
+    def extract_index(self, input_pos: int, num: int) -> torch.Tensor:  # :153-204
+        assert input_pos >= self.cache_length
+        pos, relpos, offset = self.cache_length, None, None
+        for relpos, block in enumerate(self.blocks):
+            if input_pos < pos + block.shape[-1]:
+                offset = input_pos - pos
+                break
+            pos += block.shape[-1]
+        assert offset is not None, "position too large"
+        parts = []
+        block = self.blocks[relpos]
+        bend = min(offset + num, block.shape[-1])
+        parts.append(block[:, :, offset:bend])
+        done = bend - offset
+        while done < num:
+            relpos += 1
+            block = self.blocks[relpos]
+            bend = min(num - done, block.shape[-1])
+            parts.append(block[:, :, :bend])
+            done += bend
+        return torch.cat(parts, dim=-1)
+
+
 class PolicyCacheOracle:
     """One layer's cache with the step order of DefaultKVCache.forward
     (keys_values/kvcache/base.py:554-595): write (with the ring move) -> attend -> score -> select."""
 
     def __init__(self, B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=None, grace_period=0, normalize_scores=False,
-                 v_length=False, q_hitter=False, combination_constant=0.5, quantized=False, num_bits=8):
+                 v_length=False, q_hitter=False, combination_constant=0.5, quantized=False, num_bits=8, replay_log_blocksize=None):
         assert 0 <= grace_period < L
         assert not q_hitter or quantized  # keys_values/kvcache/qh2o.py:95-96
         self.B, self.Hq, self.Hkv, self.L, self.D = B, Hq, Hkv, L, D
@@ -103,6 +168,7 @@ class PolicyCacheOracle:
         self.v_length, self.q_hitter, self.c = v_length, q_hitter, combination_constant
         self.quantized = quantized
         self.num_bits = num_bits
+        self.replay_log = ReplayLogOracle(L, replay_log_blocksize) if replay_log_blocksize else None
         self.input_pos = 0
         self.current_length = 0
         self.prefill_length = 0
@@ -186,6 +252,8 @@ class PolicyCacheOracle:
         index = index.contiguous().to(torch.int64)
         gi = lambda idx: idx.unsqueeze(-1).expand(-1, -1, -1, self.D)  # noqa: E731
         cache_full = self.input_pos >= L
+        if self.replay_log is not None and cache_full:  # attn_weights.py:629-633
+            self.replay_log.append_position_index(index, self.input_pos)
         new_k, new_v = self._stored(key), self._stored(value)
         if cache_full and gp > 0:
             # attn_weights.py:267-303: token positions

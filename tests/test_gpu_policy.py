@@ -244,3 +244,64 @@ def test_factory_names_and_errors(gpu):
         H2OKVCache(params, grace_period=64, device=gpu)
     with pytest.raises(ValueError):
         QuantizedH2OKVCache(params, combination_constant=1.5, device=gpu)
+
+
+@pytest.mark.parametrize("kwargs", [dict(), dict(grace_period=6, quantized=True)])
+def test_replay_log(gpu, kwargs):
+    """test/kvcache/test_h2o.py:227-343: the log holds the token chunks and, for every position from
+    cache_length on, the slot its K/V went to; blocks of `replay_log_blocksize` positions."""
+    B, Hq, Hkv, L, D, chunk, bs = 2, 8, 2, 128, 64, 16, 10
+    steps = (5, 16, 1, 1, 16, 7, 16, 1, 3)
+    q, k, v = _inputs(11, B, Hq, Hkv, L + sum(steps), D)
+    gen = torch.Generator().manual_seed(1)
+    tokens = torch.randint(0, 128, (B, L + sum(steps)), generator=gen)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, replay_log_blocksize=bs, device=gpu, **kwargs)
+    ref = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, replay_log_blocksize=bs,
+                              grace_period=cache.grace_period, quantized=cache.quantized)
+    assert cache.get_replay_log() is None and not cache.do_replay_logging
+    cache.switch_replay_logging(True)
+    n0 = L - 5
+    with pytest.raises(ValueError):  # logging needs the token indices
+        cache.forward(q[:, :, :n0].to(gpu), k[:, :, :n0].to(gpu), v[:, :, :n0].to(gpu))
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, replay_log_blocksize=bs, device=gpu, **kwargs)
+    cache.switch_replay_logging(True)
+    ref.prefill(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    cache.forward(q[:, :, :n0].to(gpu), k[:, :, :n0].to(gpu), v[:, :, :n0].to(gpu), tokens[:, :n0].to(gpu))
+    log = cache.get_replay_log()
+    assert len(log) == n0 and log.slot_positions == [] and log.cache_length == L and log.grace_period == cache.grace_period
+    pos, used = n0, []
+    for num in steps:
+        sl = slice(pos, pos + num)
+        had_choice = ref.next_index is not None
+        _, _, index = ref.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        if had_choice:
+            cache._next_index[:B, :, :num] = index.to(torch.int32).to(gpu)
+        cache.forward(q[:, :, sl].to(gpu), k[:, :, sl].to(gpu), v[:, :, sl].to(gpu), tokens[:, sl].to(gpu))
+        if pos >= L:
+            used.append(index)
+        pos += num
+        log = cache.get_replay_log()
+        assert len(log) == pos == cache.input_pos
+        want = ref.replay_log.finalize(pos)
+        assert len(log.slot_positions) == len(want)
+        for got, w in zip(log.slot_positions, want):
+            assert got.dtype == torch.uint32 and tuple(got.shape) == tuple(w.shape)
+            assert torch.equal(got.view(torch.int32).cpu().long(), w)
+    flat = torch.cat(used, dim=-1)
+    assert torch.equal(torch.cat([b.view(torch.int32).cpu().long() for b in log.slot_positions], dim=-1), flat)
+    assert torch.equal(log.extract_index(L + 3, 25).cpu(), flat[:, :, 3:28])
+    assert log.extract_index(L, 1, dtype=torch.int32).dtype == torch.int32
+    for c, (a, b) in zip(log.token_chunks, [(0, n0)] + [(n0 + sum(steps[:i]), n0 + sum(steps[: i + 1])) for i in range(len(steps))]):
+        assert torch.equal(c.cpu(), tokens[:, a:b])
+    with pytest.raises(ValueError):
+        log.extract_index(L - 1, 1)
+    with pytest.raises(ValueError):
+        log.extract_index(pos - 1, 5)
+    # switching on in the middle of a run needs a new prefill (keys_values/kvcache/attn_weights.py:623-628)
+    cache.switch_replay_logging(False)
+    assert cache.get_replay_log() is None
+    cache.switch_replay_logging(True)
+    with pytest.raises(IndexError):
+        cache.forward(q[:, :, :1].to(gpu), k[:, :, :1].to(gpu), v[:, :, :1].to(gpu), tokens[:, :1].to(gpu))
+    with pytest.raises(ValueError):
+        H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), replay_log_blocksize=0, device=gpu)

@@ -194,3 +194,26 @@ def test_q_hitter_values_stay_in_range_and_errors_follow_the_slots():
     k = (k.float() * (1 + 4 * torch.rand(B, Hkv, k.shape[2], 1, generator=gen))).to(torch.bfloat16)
     err = O.quantization_error(k) + O.quantization_error(v)
     torch.testing.assert_close(qh.buffers["q_errors"], err.gather(-1, qh.token_pos.long()), rtol=0, atol=0)
+
+
+def test_replay_log_blocks_are_the_concatenated_slots():
+    gen = torch.Generator().manual_seed(4)
+    L, bs = 50, 7
+    log = P.ReplayLogOracle(L, bs)
+    chunks = []
+    pos = L
+    for num in (1, 3, 7, 20, 1, 6, 2, 15):
+        idx = torch.randint(0, L, (2, 3, num), generator=gen)
+        log.append_position_index(idx, pos)
+        chunks.append(idx)
+        pos += num
+    flat = torch.cat(chunks, dim=-1)
+    total = flat.shape[-1]
+    blocks = log.finalize(pos)
+    assert all(b.shape[-1] == bs for b in blocks[:-1]) and blocks[-1].shape[-1] == total - bs * (len(blocks) - 1)
+    assert torch.equal(torch.cat(blocks, dim=-1), flat)
+    for start in range(total):
+        for num in (1, 2, bs, bs + 1, total - start):
+            if start + num <= total:
+                assert torch.equal(log.extract_index(L + start, num), flat[:, :, start : start + num])
+    assert log.finalize(L) == []
