@@ -107,6 +107,17 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t c0, uint32_t c1, int32
   return pack_bf16(a, b);
 }
 
+// 8 byte-sized codes (two dwords) -> 8 bf16 (four dwords). (Forming code - zp in fp32 from
+// byte-to-float conversions is exact for |zp| < 2^24 but measured no faster than this integer form.)
+__device__ __forceinline__ u32x4_t dequant_words(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
+  u32x4_t r;
+  r[0] = dequant_pair(c0 & 0xff, (c0 >> 8) & 0xff, zp, scale);
+  r[1] = dequant_pair((c0 >> 16) & 0xff, c0 >> 24, zp, scale);
+  r[2] = dequant_pair(c1 & 0xff, (c1 >> 8) & 0xff, zp, scale);
+  r[3] = dequant_pair((c1 >> 16) & 0xff, c1 >> 24, zp, scale);
+  return r;
+}
+
 // 4-bit store (two codes per byte, first half of the row in the high nibbles): chunk c (values
 // 8c .. 8c+7) of a row of D values lies in one nibble of the 8 bytes at u4_byte_off, and becomes 8
 // byte-sized codes with u4_codes.

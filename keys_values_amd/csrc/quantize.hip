@@ -118,12 +118,7 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
     if (r >= rows) continue;
-    u32x4_t o;
-    o[0] = dequant_pair(c[i][0] & 0xff, (c[i][0] >> 8) & 0xff, z[i], s[i]);
-    o[1] = dequant_pair((c[i][0] >> 16) & 0xff, c[i][0] >> 24, z[i], s[i]);
-    o[2] = dequant_pair(c[i][1] & 0xff, (c[i][1] >> 8) & 0xff, z[i], s[i]);
-    o[3] = dequant_pair((c[i][1] >> 16) & 0xff, c[i][1] >> 24, z[i], s[i]);
-    *(u32x4_t*)(out + r * out_row_stride + col * 8) = o;
+    *(u32x4_t*)(out + r * out_row_stride + col * 8) = dequant_words(c[i][0], c[i][1], z[i], s[i]);
   }
 }
 

@@ -181,12 +181,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
         } else {
           cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
         }
-        u32x4_t t;
-        t[0] = dequant_pair(cc[0] & 0xff, (cc[0] >> 8) & 0xff, zp, sc);
-        t[1] = dequant_pair((cc[0] >> 16) & 0xff, cc[0] >> 24, zp, sc);
-        t[2] = dequant_pair(cc[1] & 0xff, (cc[1] >> 8) & 0xff, zp, sc);
-        t[3] = dequant_pair((cc[1] >> 16) & 0xff, cc[1] >> 24, zp, sc);
-        kf[nt][j] = as_bf16x8(t);
+        kf[nt][j] = as_bf16x8(dequant_words(cc[0], cc[1], zp, sc));
       }
     }
   }

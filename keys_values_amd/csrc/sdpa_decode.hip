@@ -47,14 +47,7 @@ struct DecodeParams {
   int64_t q_sb, q_sh, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, qs_sb, qs_sh;
 };
 
-__device__ __forceinline__ u32x4_t dq8(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
-  u32x4_t r;
-  r[0] = dequant_pair(c0 & 0xff, (c0 >> 8) & 0xff, zp, scale);
-  r[1] = dequant_pair((c0 >> 16) & 0xff, c0 >> 24, zp, scale);
-  r[2] = dequant_pair(c1 & 0xff, (c1 >> 8) & 0xff, zp, scale);
-  r[3] = dequant_pair((c1 >> 16) & 0xff, c1 >> 24, zp, scale);
-  return r;
-}
+__device__ __forceinline__ u32x4_t dq8(uint32_t c0, uint32_t c1, int32_t zp, float scale) { return dequant_words(c0, c1, zp, scale); }
 
 // Sum over the LPR lanes that share a row. Every lane of the group ends with the same bits: each
 // step adds two values that the partner lane adds in the other order.

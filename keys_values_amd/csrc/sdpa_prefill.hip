@@ -107,14 +107,7 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
 }
 
 // 8 codes (two dwords) -> 8 bf16 (four dwords)
-__device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
-  u32x4_t r;
-  r[0] = dequant_pair(c0 & 0xff, (c0 >> 8) & 0xff, zp, scale);
-  r[1] = dequant_pair((c0 >> 16) & 0xff, c0 >> 24, zp, scale);
-  r[2] = dequant_pair(c1 & 0xff, (c1 >> 8) & 0xff, zp, scale);
-  r[3] = dequant_pair((c1 >> 16) & 0xff, c1 >> 24, zp, scale);
-  return r;
-}
+__device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp, float scale) { return dequant_words(c0, c1, zp, scale); }
 
 // Tile loader. A wavefront instruction covers RPW = 64 / CPR whole rows; wavefront w of the
 // workgroup takes row groups w, w + 4, ... of the 64-row tile (NI groups each for K and for V).
