@@ -327,6 +327,21 @@ size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* args);
 int kvx_rmsnorm_rows(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride,
                      const float* weight, int64_t rows, int32_t dim, float eps, void* stream);
 
+/* Residual add fused with the normalisation that follows it in a block (Block.forward,
+ * keys_values/model.py:560-584: x = attention_output + x; ... norm_2(x)):
+ *   x_out = bf16(x + delta);  out = RMSNorm(x_out) as kvx_rmsnorm_rows.
+ * The sum is rounded to bf16 before it is normalised, as the two separate steps round. x_out may be x. */
+int kvx_add_rmsnorm_rows(const void* x, int64_t x_row_stride, const void* delta, int64_t delta_row_stride,
+                         void* x_out, int64_t x_out_row_stride, void* out, int64_t out_row_stride,
+                         const float* weight, int64_t rows, int32_t dim, float eps, void* stream);
+
+/* Gated activation of the MLP (LLaMAMLP.forward of litgpt, which keys_values/model.py builds on:
+ * proj(silu(fc_1(x)) * fc_2(x))) on the output of ONE GEMM over the stacked fc_1 / fc_2 weights:
+ *   out[r, j] = bf16( bf16(silu(gate_up[r, j])) * gate_up[r, dim + j] ),  silu(t) = t / (1 + exp(-t)) in fp32.
+ * gate_up: bf16 (rows, 2 * dim) by row stride; out: bf16 (rows, dim). dim a multiple of 8. */
+int kvx_swiglu_rows(const void* gate_up, int64_t gate_up_row_stride, void* out, int64_t out_row_stride,
+                    int64_t rows, int32_t dim, void* stream);
+
 /* Per-head normalisation of the new queries and keys followed by the rotary position encoding, in
  * place on the output of the QKV projection: what CausalSelfAttention.forward does between the
  * projection and the cache (keys_values/model.py:733-775: norm_q / norm_k, then

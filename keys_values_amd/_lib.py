@@ -102,6 +102,9 @@ SYMBOLS = {
     "kvx_h2o_update_select": (ctypes.c_int, [POINTER(H2OArgs), c_void_p]),
     "kvx_h2o_workspace_bytes": (c_size_t, [POINTER(H2OArgs)]),
     "kvx_rmsnorm_rows": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, ctypes.c_float, c_void_p]),
+    "kvx_add_rmsnorm_rows": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                            c_int32, ctypes.c_float, c_void_p]),
+    "kvx_swiglu_rows": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32, c_void_p]),
     "kvx_qk_norm_rope": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
                                         ctypes.c_float, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
 }

@@ -317,6 +317,34 @@ int kvx_rmsnorm_rows(const void* x, int64_t x_row_stride, void* out, int64_t out
   return launch_rmsnorm_rows(x, x_row_stride, out, out_row_stride, weight, rows, dim, eps, (hipStream_t)stream);
 }
 
+int kvx_add_rmsnorm_rows(const void* x, int64_t x_row_stride, const void* delta, int64_t delta_row_stride, void* x_out,
+                         int64_t x_out_row_stride, void* out, int64_t out_row_stride, const float* weight, int64_t rows, int32_t dim,
+                         float eps, void* stream) {
+  KVX_REQUIRE(rows >= 0 && dim > 0, KVX_ERR_INVALID, "kvx_add_rmsnorm_rows: rows=%lld, dim=%d", (long long)rows, dim);
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(x && delta && x_out && out && weight, KVX_ERR_INVALID, "kvx_add_rmsnorm_rows: NULL pointer");
+  KVX_REQUIRE(dim % 8 == 0 && dim <= 8192, KVX_ERR_UNSUPPORTED, "kvx_add_rmsnorm_rows: dim=%d must be a multiple of 8, at most 8192", dim);
+  KVX_REQUIRE(aligned16(x) && aligned16(delta) && aligned16(x_out) && aligned16(out) && aligned16(weight) && mult8(x_row_stride) &&
+                  mult8(delta_row_stride) && mult8(x_out_row_stride) && mult8(out_row_stride),
+              KVX_ERR_INVALID, "kvx_add_rmsnorm_rows: rows must be 16-byte aligned");
+  KVX_REQUIRE(out != x && out != delta, KVX_ERR_INVALID, "kvx_add_rmsnorm_rows: out must not alias the inputs");
+  return launch_add_rmsnorm_rows(x, x_row_stride, delta, delta_row_stride, x_out, x_out_row_stride, out, out_row_stride, weight, rows, dim,
+                                 eps, (hipStream_t)stream);
+}
+
+int kvx_swiglu_rows(const void* gate_up, int64_t gate_up_row_stride, void* out, int64_t out_row_stride, int64_t rows, int32_t dim,
+                    void* stream) {
+  KVX_REQUIRE(rows >= 0 && dim > 0, KVX_ERR_INVALID, "kvx_swiglu_rows: rows=%lld, dim=%d", (long long)rows, dim);
+  if (rows == 0) return KVX_OK;
+  KVX_REQUIRE(gate_up && out, KVX_ERR_INVALID, "kvx_swiglu_rows: NULL pointer");
+  KVX_REQUIRE(dim % 8 == 0, KVX_ERR_UNSUPPORTED, "kvx_swiglu_rows: dim=%d must be a multiple of 8", dim);
+  KVX_REQUIRE(aligned16(gate_up) && aligned16(out) && mult8(gate_up_row_stride) && mult8(out_row_stride) &&
+                  gate_up_row_stride >= 2 * (int64_t)dim && out_row_stride >= dim,
+              KVX_ERR_INVALID, "kvx_swiglu_rows: rows must be 16-byte aligned, gate_up rows 2 * dim long");
+  KVX_REQUIRE(out != gate_up, KVX_ERR_INVALID, "kvx_swiglu_rows: out must not alias gate_up");
+  return launch_swiglu_rows(gate_up, gate_up_row_stride, out, out_row_stride, rows, dim, (hipStream_t)stream);
+}
+
 int kvx_qk_norm_rope(void* qkv, int64_t stride_b, int64_t stride_t, int32_t B, int32_t num, int32_t Hq, int32_t Hkv, int32_t D,
                      const float* q_weight, const float* k_weight, float eps, const float* cos, const float* sin, int32_t table_rows,
                      int32_t input_pos, void* stream) {

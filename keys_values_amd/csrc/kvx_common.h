@@ -57,6 +57,9 @@ int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st);
 size_t h2o_workspace(const kvx_h2o_args& a);
 int launch_rmsnorm_rows(const void* x, int64_t x_rs, void* out, int64_t o_rs, const float* weight, int64_t rows, int dim, float eps,
                         hipStream_t st);
+int launch_add_rmsnorm_rows(const void* x, int64_t x_rs, const void* delta, int64_t d_rs, void* x_out, int64_t xo_rs, void* out,
+                            int64_t o_rs, const float* weight, int64_t rows, int dim, float eps, hipStream_t st);
+int launch_swiglu_rows(const void* gate_up, int64_t g_rs, void* out, int64_t o_rs, int64_t rows, int dim, hipStream_t st);
 int launch_qk_norm_rope(void* qkv, int64_t sb, int64_t stt, int B, int num, int Hq, int Hkv, int D, const float* qw, const float* kw,
                         float eps, const float* cos_t, const float* sin_t, int input_pos, hipStream_t st);
 

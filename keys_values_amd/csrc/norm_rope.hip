@@ -69,6 +69,82 @@ __global__ __launch_bounds__(NT) void rmsnorm_rows_kernel(const uint16_t* __rest
   }
 }
 
+// x_out = bf16(x + delta) and out = RMSNorm(x_out) in one pass: the residual add of a block fused with
+// the normalisation that follows it (keys_values/model.py:560-584: x = attention_output + x, then
+// norm_2(x); x = mlp_output + x, then the next block's norm_1). The sum is rounded to bf16 before it is
+// normalised, as the two separate steps do. In place is allowed (x_out == x).
+template <int MAXC>
+__global__ __launch_bounds__(NT) void add_rmsnorm_rows_kernel(const uint16_t* x, int64_t x_rs, const uint16_t* __restrict__ delta,
+                                                              int64_t d_rs, uint16_t* x_out, int64_t xo_rs,
+                                                              uint16_t* __restrict__ out, int64_t o_rs, const float* __restrict__ weight,
+                                                              int64_t rows, int dim, float eps, float factor) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunks = dim / 8;
+  u32x4_t v[MAXC];
+  float ss = 0.0f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = lane + 64 * c;
+    v[c] = u32x4_t{0, 0, 0, 0};
+    if (ch < nchunks) {
+      const u32x4_t a = *(const u32x4_t*)(x + row * x_rs + ch * 8);
+      const u32x4_t b = *(const u32x4_t*)(delta + row * d_rs + ch * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[c][e] = pack_bf16(bf16_lo(a[e]) + bf16_lo(b[e]), bf16_hi(a[e]) + bf16_hi(b[e]));
+      *(u32x4_t*)(x_out + row * xo_rs + ch * 8) = v[c];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float a = bf16_lo(v[c][e]), b = bf16_hi(v[c][e]);
+      ss += a * a;
+      ss += b * b;
+    }
+  }
+  ss = wave_sum(ss);
+  const float denom = sqrtf(ss) * factor + eps;
+  uint16_t* orow = out + row * o_rs;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ch = lane + 64 * c;
+    if (ch >= nchunks) break;
+    const f32x4_t w0 = *(const f32x4_t*)(weight + ch * 8);
+    const f32x4_t w1 = *(const f32x4_t*)(weight + ch * 8 + 4);
+    u32x4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float wa = e < 2 ? w0[2 * e] : w1[2 * e - 4];
+      const float wb = e < 2 ? w0[2 * e + 1] : w1[2 * e - 3];
+      o[e] = pack_bf16((bf16_lo(v[c][e]) / denom) * wa, (bf16_hi(v[c][e]) / denom) * wb);
+    }
+    *(u32x4_t*)(orow + ch * 8) = o;
+  }
+}
+
+// out[r, j] = bf16( bf16(silu(g[r, j])) * u[r, j] ), g = gate_up[r, j], u = gate_up[r, dim + j]: the
+// gated activation of LLaMAMLP (proj(silu(fc_1 x) * fc_2 x)) on the output of one GEMM over the stacked
+// fc_1 / fc_2 weights. silu is x / (1 + exp(-x)) in fp32, rounded to bf16 before the product, as the
+// two separate tensor operations round.
+__global__ __launch_bounds__(NT) void swiglu_rows_kernel(const uint16_t* __restrict__ gate_up, int64_t g_rs, uint16_t* __restrict__ out,
+                                                         int64_t o_rs, int64_t rows, int dim) {
+  const int cpr = dim / 8;
+  const int64_t gid = (int64_t)blockIdx.x * NT + threadIdx.x;
+  if (gid >= rows * cpr) return;
+  const int64_t r = gid / cpr;
+  const int c = (int)(gid % cpr);
+  const u32x4_t g = *(const u32x4_t*)(gate_up + r * g_rs + c * 8);
+  const u32x4_t u = *(const u32x4_t*)(gate_up + r * g_rs + dim + c * 8);
+  u32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float g0 = bf16_lo(g[e]), g1 = bf16_hi(g[e]);
+    const uint32_t act = pack_bf16(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+    o[e] = pack_bf16(bf16_lo(act) * bf16_lo(u[e]), bf16_hi(act) * bf16_hi(u[e]));
+  }
+  *(u32x4_t*)(out + r * o_rs + c * 8) = o;
+}
+
 // One lane per 8 elements of a head row; LPR = D / 8 lanes share a row. Rows are (b, t, head) with
 // head in [0, Hq + Hkv): the query heads, then the key heads, of token t.
 template <int D>
@@ -148,6 +224,30 @@ int launch_rmsnorm_rows(const void* x, int64_t x_rs, void* out, int64_t o_rs, co
   else
     hipLaunchKernelGGL(rmsnorm_rows_kernel<16>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs, weight, rows,
                        dim, eps, factor);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_add_rmsnorm_rows(const void* x, int64_t x_rs, const void* delta, int64_t d_rs, void* x_out, int64_t xo_rs, void* out,
+                            int64_t o_rs, const float* weight, int64_t rows, int dim, float eps, hipStream_t st) {
+  if (rows == 0) return KVX_OK;
+  const float factor = 1.0f / sqrtf((float)dim);
+  const unsigned grid = (unsigned)((rows + NT / 64 - 1) / (NT / 64));
+  if ((dim / 8 + 63) / 64 <= 4)
+    hipLaunchKernelGGL(add_rmsnorm_rows_kernel<4>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
+                       (uint16_t*)x_out, xo_rs, (uint16_t*)out, o_rs, weight, rows, dim, eps, factor);
+  else
+    hipLaunchKernelGGL(add_rmsnorm_rows_kernel<16>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
+                       (uint16_t*)x_out, xo_rs, (uint16_t*)out, o_rs, weight, rows, dim, eps, factor);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_swiglu_rows(const void* gate_up, int64_t g_rs, void* out, int64_t o_rs, int64_t rows, int dim, hipStream_t st) {
+  const int64_t total = rows * (dim / 8);
+  if (total == 0) return KVX_OK;
+  hipLaunchKernelGGL(swiglu_rows_kernel, dim3((unsigned)((total + NT - 1) / NT)), dim3(NT), 0, st, (const uint16_t*)gate_up, g_rs,
+                     (uint16_t*)out, o_rs, rows, dim);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }

@@ -69,7 +69,16 @@ class H2OKVCache:
         q_hitter: bool = False,
         combination_constant: float = DEFAULT_COMBINATION_CONSTANT,
         replay_log_blocksize: Optional[int] = None,
+        overlap_select: bool = False,
     ):
+        # overlap_select: launch the score update + eviction choice of a chunk step on a second stream, so
+        # that it runs beside whatever the caller enqueues next; the next forward waits for it. The scores,
+        # the next slots and token_pos must then not be read from the caller's stream before
+        # wait_for_selection() (the properties of this class do that).
+        self._overlap = bool(overlap_select)
+        self._side_stream = None
+        self._select_done = None
+        self._select_keep = None
         if replay_log_blocksize is None:  # keys_values/kvcache/attn_weights.py:436-441
             replay_log_blocksize = DEFAULT_REPLAY_LOG_BLOCKSIZE
         elif replay_log_blocksize <= 0:
@@ -169,9 +178,16 @@ class H2OKVCache:
             raise IndexError("Cache is not initialized, call 'prefill' first")
         return self.token_pos[: self.batch_size, :, : self.current_length]
 
+    def wait_for_selection(self):
+        """Make the caller's stream wait for an eviction choice still running on the second stream."""
+        if self._select_done is not None:
+            torch.cuda.current_stream(self.device).wait_event(self._select_done)
+            self._select_done, self._select_keep = None, None
+
     def next_positions(self, num: int) -> Optional[torch.Tensor]:
         """Slots the next ``forward`` writes to, int64 (batch, n_query_groups, num), or None
         (keys_values/kvcache/attn_weights.py:490-499)."""
+        self.wait_for_selection()
         idx = self._next_index_for(num, peek=True)
         return None if idx is None else idx.to(torch.int64)
 
@@ -243,6 +259,7 @@ class H2OKVCache:
         if key.shape != (b, self.n_query_groups, num, d) or hq != self.n_head or d != self.head_size:
             raise ValueError(f"shapes {tuple(query.shape)}, {tuple(key.shape)} do not fit the cache")
         input_pos = self._input_pos
+        self.wait_for_selection()
         if input_pos == 0:
             out = self._prefill_step(query, key, value)
             self._log_token_chunk(token_idx, num, prefill=True)
@@ -446,10 +463,27 @@ class H2OKVCache:
                 nxt = torch.empty((self.batch_size, self.n_query_groups, 1), dtype=torch.int32, device=self.device)
             a.next_index = nxt.data_ptr()
             nbytes = lib.kvx_h2o_workspace_bytes(ctypes.byref(a))
-            ws = _lib.workspace(self.device, nbytes)
-            a.workspace = _lib.ptr(ws)
-            a.workspace_bytes = 0 if ws is None else ws.numel()
-            _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
+            if not self._overlap:
+                ws = _lib.workspace(self.device, nbytes)
+                a.workspace = _lib.ptr(ws)
+                a.workspace_bytes = 0 if ws is None else ws.numel()
+                _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
+            else:
+                main = torch.cuda.current_stream(self.device)
+                if self._side_stream is None:
+                    self._side_stream = torch.cuda.Stream(self.device)  # default priority
+                ready = torch.cuda.Event()
+                ready.record(main)
+                with torch.cuda.stream(self._side_stream):
+                    self._side_stream.wait_event(ready)
+                    ws = _lib.workspace(self.device, nbytes)  # one buffer per stream
+                    a.workspace = _lib.ptr(ws)
+                    a.workspace_bytes = 0 if ws is None else ws.numel()
+                    _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), self._side_stream.cuda_stream))
+                    done = torch.cuda.Event()
+                    done.record(self._side_stream)
+                self._select_done = done
+                self._select_keep = (attn_weights, nxt)  # alive until the second stream is done with them
         self._have_next = full
 
 

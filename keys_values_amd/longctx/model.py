@@ -47,8 +47,9 @@ class _Layer:
         d = cfg.head_size
         self.qkv = w((cfg.n_head + 2 * cfg.n_query_groups) * d, cfg.n_embd)
         self.proj = w(cfg.n_embd, cfg.n_head * d)
-        self.fc_1 = w(cfg.intermediate_size, cfg.n_embd)
-        self.fc_2 = w(cfg.intermediate_size, cfg.n_embd)
+        # fc_1 and fc_2 stacked: one GEMM gives [gate | up] (the two halves are views of it)
+        self.fc_12 = torch.cat((w(cfg.intermediate_size, cfg.n_embd), w(cfg.intermediate_size, cfg.n_embd)))
+        self.fc_1, self.fc_2 = self.fc_12[: cfg.intermediate_size], self.fc_12[cfg.intermediate_size :]
         self.mlp_proj = w(cfg.n_embd, cfg.intermediate_size)
         self.norm_1 = torch.ones(cfg.n_embd, dtype=torch.float32, device=device)
         self.norm_2 = torch.ones(cfg.n_embd, dtype=torch.float32, device=device)
@@ -73,7 +74,10 @@ class LongContextPrefillModel:
         self.chunk_size = chunk_size
         self.cache_length = cache_length
         params = KVCacheParams(max_batch_size, cfg.n_query_groups, cache_length, cfg.head_size, cfg.n_head)
-        self.caches = [H2OKVCache(params, max_chunk_size=chunk_size, quantized=quantized, device=self.device) for _ in range(cfg.n_layer)]
+        # the eviction choice of a layer is first needed when the next chunk reaches that layer: it runs beside
+        # the layer's dense part on a second stream
+        self.caches = [H2OKVCache(params, max_chunk_size=chunk_size, quantized=quantized, device=self.device, overlap_select=True)
+                       for _ in range(cfg.n_layer)]
         self.cos, self.sin = ops.rope_tables(max_context, cfg.head_size, cfg.rope_base, self.device)
         self.input_pos = 0
 
@@ -87,32 +91,34 @@ class LongContextPrefillModel:
         mpl = min(c.max_prefill_length for c in self.caches)
         return create_chunk_sizes(mpl, [c.cache_length for c in self.caches], seq_length, self.chunk_size)
 
-    def _block(self, li: int, x: torch.Tensor) -> torch.Tensor:
-        """Block.forward, keys_values/model.py:524-584 (non-parallel residual, no post-norms)."""
+    def _block(self, li: int, x: torch.Tensor, xn: torch.Tensor, next_norm: torch.Tensor) -> torch.Tensor:
+        """Block.forward, keys_values/model.py:524-584 (non-parallel residual, no post-norms). x is the
+        residual stream (updated in place), xn = norm_1(x); returns the next block's norm_1 (or the final
+        norm) of the updated stream: each residual add is fused with the normalisation that follows it."""
         cfg, layer = self.cfg, self.layers[li]
         B, num, _ = x.shape
         d, hq, hkv = cfg.head_size, cfg.n_head, cfg.n_query_groups
-        xn = ops.rmsnorm(x, layer.norm_1, cfg.norm_eps)
         qkv = F.linear(xn, layer.qkv)
         ops.qk_norm_rope_(qkv, hq, hkv, d, layer.norm_q, layer.norm_k, cfg.norm_eps, self.cos, self.sin, self.input_pos)
         q = qkv[..., : hq * d].view(B, num, hq, d).transpose(1, 2)
         k = qkv[..., hq * d : (hq + hkv) * d].view(B, num, hkv, d).transpose(1, 2)
         v = qkv[..., (hq + hkv) * d :].view(B, num, hkv, d).transpose(1, 2)
         y = self.caches[li].forward(q, k, v)
-        x = x + F.linear(y, layer.proj)
-        xn = ops.rmsnorm(x, layer.norm_2, cfg.norm_eps)
-        h = F.silu(F.linear(xn, layer.fc_1)) * F.linear(xn, layer.fc_2)  # LLaMAMLP: proj(silu(fc_1 x) * fc_2 x)
-        return x + F.linear(h, layer.mlp_proj)
+        xn = ops.add_rmsnorm_(x, F.linear(y, layer.proj), layer.norm_2, cfg.norm_eps)  # x = attention_output + x; norm_2(x)
+        h = ops.swiglu(F.linear(xn, layer.fc_12))  # LLaMAMLP: proj(silu(fc_1 x) * fc_2 x)
+        return ops.add_rmsnorm_(x, F.linear(h, layer.mlp_proj), next_norm, cfg.norm_eps)  # x = mlp_output + x
 
     def forward_chunk(self, input_ids: torch.Tensor) -> torch.Tensor:
         """One chunk through all layers; returns the final-norm hidden states (B, num, n_embd)."""
         if input_ids.ndim != 2:
             raise ValueError(f"input_ids.shape = {tuple(input_ids.shape)}, must be 2D")
+        n = self.cfg.n_layer
         x = F.embedding(input_ids.to(self.device), self.wte)
-        for li in range(self.cfg.n_layer):
-            x = self._block(li, x)
+        xn = ops.rmsnorm(x, self.layers[0].norm_1, self.cfg.norm_eps) if n > 0 else ops.rmsnorm(x, self.ln_f, self.cfg.norm_eps)
+        for li in range(n):
+            xn = self._block(li, x, xn, self.layers[li + 1].norm_1 if li + 1 < n else self.ln_f)
         self.input_pos += input_ids.shape[1]
-        return ops.rmsnorm(x, self.ln_f, self.cfg.norm_eps)
+        return xn
 
     def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
         """Process whole sequences chunk by chunk; returns the hidden states of the last chunk."""

@@ -1,4 +1,5 @@
-"""Host wrappers of the normalisation / rotary kernels (C ABI: kvx_rmsnorm_rows, kvx_qk_norm_rope)."""
+"""Host wrappers of the normalisation / rotary / gated-activation kernels (C ABI: kvx_rmsnorm_rows,
+kvx_add_rmsnorm_rows, kvx_swiglu_rows, kvx_qk_norm_rope)."""
 from typing import Optional, Tuple
 
 import torch
@@ -33,6 +34,44 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
     with torch.cuda.device(x.device):
         _lib.check(lib.kvx_rmsnorm_rows(x2.data_ptr(), x2.stride(0), o2.data_ptr(), o2.stride(0), weight.data_ptr(), x2.shape[0], dim,
                                         float(eps), _lib.stream_ptr(x.device)))
+    return out
+
+
+def add_rmsnorm_(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``x += delta`` (in place, rounded to bf16) and ``RMSNorm(x)`` in one pass: the residual add of a
+    block with the normalisation that follows it (keys_values/model.py:560-584). Returns the normed rows."""
+    _lib.require_gpu(x, delta, weight)
+    if x.dtype != torch.bfloat16 or delta.dtype != torch.bfloat16 or weight.dtype != torch.float32:
+        raise ValueError("add_rmsnorm_ takes bfloat16 rows and a float32 weight")
+    dim = x.shape[-1]
+    if x.shape != delta.shape or weight.shape != (dim,) or not x.is_contiguous():
+        raise ValueError(f"x {tuple(x.shape)} (contiguous), delta {tuple(delta.shape)}, weight {tuple(weight.shape)} do not fit")
+    d2 = delta.reshape(-1, dim)
+    if d2.stride(-1) != 1:
+        d2 = d2.contiguous()
+    x2 = x.view(-1, dim)
+    out = torch.empty_like(x)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.kvx_add_rmsnorm_rows(x2.data_ptr(), dim, d2.data_ptr(), d2.stride(0), x2.data_ptr(), dim, out.data_ptr(), dim,
+                                            weight.data_ptr(), x2.shape[0], dim, float(eps), _lib.stream_ptr(x.device)))
+    return out
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` for ``gate_up = [gate | up]`` (..., 2 * dim), the output of one GEMM over the
+    stacked fc_1 / fc_2 weights; same rounding as ``F.silu(gate) * up`` on bf16 tensors."""
+    _lib.require_gpu(gate_up)
+    if gate_up.dtype != torch.bfloat16 or gate_up.shape[-1] % 16 != 0:
+        raise ValueError("swiglu takes bfloat16 rows of even width, a multiple of 16")
+    dim = gate_up.shape[-1] // 2
+    g2 = gate_up.reshape(-1, 2 * dim)
+    if g2.stride(-1) != 1:
+        g2 = g2.contiguous()
+    out = torch.empty(gate_up.shape[:-1] + (dim,), dtype=gate_up.dtype, device=gate_up.device)
+    lib = _lib.load()
+    with torch.cuda.device(gate_up.device):
+        _lib.check(lib.kvx_swiglu_rows(g2.data_ptr(), g2.stride(0), out.data_ptr(), dim, g2.shape[0], dim, _lib.stream_ptr(gate_up.device)))
     return out
 
 

@@ -387,3 +387,32 @@ def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, B, Hq, Hkv, T, D, lim
     n_ref = O.h2o_update_select(s_ref, w_ref, T, limit, 1, normalize=normalize, token_pos=tp, input_pos=input_pos, prefill_len=prefill_len)
     torch.testing.assert_close(sc_g.cpu(), s_ref, rtol=1e-3, atol=1e-6)
     _sets_equal_away_from_ties(nxt.cpu().long(), n_ref, (s_ref[..., :limit] / (input_pos - torch.maximum(tp, torch.tensor(prefill_len - 1)))[..., :limit].float()) if normalize else s_ref[..., :limit], 1)
+
+
+def test_overlapped_selection_equals_in_order_selection(gpu):
+    """overlap_select=True runs the score update + eviction choice on a second stream beside the
+    caller's next launches; every result must equal the in-order cache's bit for bit."""
+    B, Hq, Hkv, L, D, chunk = 1, 8, 2, 2048, 128, 128
+    gen = torch.Generator().manual_seed(5)
+    total = L + 6 * chunk
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    a = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, quantized=True, device=gpu)
+    b = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, quantized=True, device=gpu, overlap_select=True)
+    busy = torch.randn(2048, 2048, device=gpu)
+    for cache in (a, b):
+        cache.forward(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L])
+    pos = L
+    for step in range(6):
+        sl = slice(pos, pos + chunk)
+        oa = a.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        ob = b.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        for _ in range(3):  # the caller's own work, enqueued while the choice may still be running
+            busy = (busy @ busy).clamp_(-1, 1)
+        assert torch.equal(a.next_positions(chunk), b.next_positions(chunk))  # waits for the second stream
+        torch.cuda.synchronize()
+        assert torch.equal(oa, ob)
+        assert torch.equal(a.scores, b.scores) and torch.equal(a.token_pos, b.token_pos)
+        assert torch.equal(a.k, b.k) and torch.equal(a.v, b.v)
+        pos += chunk

@@ -109,6 +109,47 @@ def test_rmsnorm_kernel(gpu, rows, dim):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,dim", [(5, 64), (1024, 2560), (3, 8192), (17, 200)])
+def test_add_rmsnorm_kernel(gpu, rows, dim):
+    # x = x + delta (rounded to bf16), then RMSNorm(x): the two separate steps of the oracle
+    from keys_values_amd.longctx import ops
+
+    gen = torch.Generator().manual_seed(rows * dim)
+    x = (torch.randn(2, rows, dim, generator=gen) * 3).to(torch.bfloat16)
+    delta = torch.randn(2, rows, dim, generator=gen).to(torch.bfloat16)
+    w = torch.rand(dim, generator=gen) + 0.5
+    xg = x.to(gpu)
+    y = ops.add_rmsnorm_(xg, delta.to(gpu), w.to(gpu), 1e-6).cpu()
+    x_ref = x + delta
+    assert torch.equal(xg.cpu(), x_ref), "the residual stream must hold the rounded sum"
+    ref = LO.rmsnorm(x_ref, w, 1e-6)
+    torch.testing.assert_close(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+    assert (y != ref).float().mean().item() < 0.02
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,dim", [(7, 16), (1024, 9728), (33, 200)])
+def test_swiglu_kernel(gpu, rows, dim):
+    # silu(gate) * up with the activation rounded to bf16 before the product, as F.silu(g) * u rounds
+    import torch.nn.functional as F
+
+    from keys_values_amd.longctx import ops
+
+    gen = torch.Generator().manual_seed(dim)
+    gu = (torch.randn(rows, 2 * dim, generator=gen) * 2).to(torch.bfloat16)
+    gu[0, :4] = torch.tensor([0.0, -30.0, 30.0, -100.0]).to(torch.bfloat16)  # silu(0) = 0, tails: exp under / overflow
+    out = ops.swiglu(gu.to(gpu)).cpu()
+    ref = F.silu(gu[:, :dim]) * gu[:, dim:]
+    torch.testing.assert_close(out.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+    assert (out != ref).float().mean().item() < 0.01  # exp implementations differ in the last fp32 bits
+    # closed form in float64 of the un-rounded function
+    g64, u64 = gu[:, :dim].double(), gu[:, dim:].double()
+    exact = g64 / (1 + torch.exp(-g64)) * u64
+    torch.testing.assert_close(out.double(), exact, rtol=2 ** -6, atol=1e-6)
+    assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("B,num,Hq,Hkv,D,norm,input_pos", [(1, 64, 8, 2, 64, True, 0), (2, 100, 32, 8, 128, True, 4000), (1, 33, 4, 4, 128, False, 77)])
 def test_qk_norm_rope_kernel(gpu, B, num, Hq, Hkv, D, norm, input_pos):
     from keys_values_amd.longctx import ops
