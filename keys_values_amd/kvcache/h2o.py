@@ -240,6 +240,9 @@ class H2OKVCache:
             return torch.arange(start, start + num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, h, -1).contiguous()
         if self._use_initial_rule:  # attn_weights.py:536-550
             n0 = min(int(self._keep_initial_fraction * self.cache_length), self.cache_length - num)
+            # with a grace period the evicted slots must stay below the ring (the reference's formula
+            # does not look at it; it only matters for chunks nearly as long as the evictable part)
+            n0 = min(n0, self.cache_length - self.grace_period - num)
             if not peek:
                 self._use_initial_rule = False
             return torch.arange(n0, n0 + num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, h, -1).contiguous()
