@@ -570,8 +570,8 @@ def bench_calib(args, torch, dev):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path shards without communication over KV heads; "
-              "see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (the path would shard over KV heads without communication; "
+              "no multi-GPU code exists). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     import torch
 

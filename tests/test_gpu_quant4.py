@@ -27,7 +27,7 @@ def outlier_rows(seed, rows, D):
     return x
 
 
-@pytest.mark.parametrize("rows,D", [(1, 128), (7, 64), (1000, 128), (4099, 64), (65536, 128)])
+@pytest.mark.parametrize("rows,D", [(1, 128), (7, 64), (1000, 128), (4099, 64), (65536, 128), (8 * 65536, 128)])
 def test_quantize_rows4_bit_exact(kvx, gpu, rows, D):
     x = outlier_rows(rows, rows, D)
     c_ref, s_ref, z_ref = O.quantize_rows(x, num_bits=4)
