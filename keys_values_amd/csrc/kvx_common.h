@@ -86,6 +86,18 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // Exchange with the lane 32 away (the other half of the wavefront).
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// max / sum of a value with the lane 32 away, in every lane, through v_permlane32_swap (a vector ALU
+// exchange of the two wavefront halves; no LDS round trip as with a shuffle).
+typedef uint32_t u32pair_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float max_halves(float v) {
+  const u32pair_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_halves(float v) {
+  const u32pair_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // The affine 8-bit row quantiser, one element. `inv` = 1.0f / scale, `zf` = (float) zero point.
 // rint before the add, so the multiply can never fuse with it.
 // `qmax` = 255 (8-bit) or 15 (4-bit codes).

@@ -299,7 +299,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
 
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
-    const float tot = wacc[nt] + xor32(wacc[nt]);
+    const float tot = sum_halves(wacc[nt]);
     const int key = key0 + nt * 32 + n;
     if (h == 0 && key < p.kv_len) p.w[((int64_t)b * p.Hkv + kvh) * p.kv_len + key] = tot * p.inv_g;
   }

@@ -415,7 +415,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, s[0][i]), s[1][i]);
-    mx = fmaxf(mx, xor32(mx));
+    mx = max_halves(mx);
     float alpha = 1.0f;
     // m is a reference, not the exact maximum: it moves only when a score exceeds it by 2^kSlackLog2
     // in the exponent, which keeps every p below 2^kSlackLog2 and makes rescaling rare
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
   pv(pb_prev, (tile_end - 1 - tile_begin) & 1);
 
   // ---- epilogue -----------------------------------------------------------------------------
-  const float lt = l + xor32(l);
+  const float lt = sum_halves(l);
   if (p.num_splits == 1) {
     const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
     if (row_ok) {
