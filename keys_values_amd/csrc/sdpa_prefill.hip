@@ -368,26 +368,31 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     }
   };
 
-  // second product for one tile: O^T += V^T P^T with V from v[buf]
-  auto pv = [&](const uint32_t (&pb)[2][8], int buf) {
+  // second product for one tile: O^T += V^T P^T with V from v[buf]; matrix instructions FIRST ..
+  // FIRST + COUNT - 1 of the 4 DT in (key block, d tile) order
+  auto pv_part = [&](const uint32_t (&pb)[2][8], int buf, auto first_tag, auto count_tag) {
+    constexpr int FIRST_I = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
     // one LDS pointer per d tile; every read below is that pointer plus a compile-time offset
     lds_ptr_t vl[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) vl[dt] = (lds_ptr_t)((const char*)&sm.v[buf][0][0] + va[dt]);
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
-        const int rb = (32 * mt + 16 * j) * CPR * 16;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const u32x2_t lo = lds_read_tr16(vl[dt] + rb);
-          const u32x2_t hi = lds_read_tr16(vl[dt] + rb + 8 * CPR * 16);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
-        }
-      }
+    for (int i = FIRST_I; i < FIRST_I + COUNT; ++i) {
+      const int mt = i / (2 * DT), j = (i / DT) % 2, dt = i % DT;
+      const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
+      const int rb = (32 * mt + 16 * j) * CPR * 16;
+      const u32x2_t lo = lds_read_tr16(vl[dt] + rb);
+      const u32x2_t hi = lds_read_tr16(vl[dt] + rb + 8 * CPR * 16);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
+    }
   };
+  auto pv = [&](const uint32_t (&pb)[2][8], int buf) {
+    pv_part(pb, buf, std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * DT>{});
+  };
+  // The first NPRE matrix instructions of the second product go out right behind the first product:
+  // they keep the matrix core busy while the vector ALU reduces the maximum of S(t), which has to wait
+  // for the first product anyway.
+  constexpr int NPRE = DT;
 
   // Pipeline: iteration t multiplies S(t) = K(t) Q^T, then lets the matrix cores add V(t-1) P(t-1)
   // to O while the vector ALU turns S(t) into P(t). K(t) sits in k[t & 1]; V(t-1) in v[(t-1) & 1];
@@ -410,6 +415,10 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     if (has1) ld.template issue_one<true>(sm, t + 1, cur ^ 1, tid);
     f32x16_t s[2];
     qk(s, cur);
+    if constexpr (!FIRST) {
+      pv_part(pb_prev, cur ^ 1, std::integral_constant<int, 0>{}, std::integral_constant<int, NPRE>{});
+      __builtin_amdgcn_sched_barrier(0);
+    }
     mask(s, cur);
     // ---- running maximum; rescale only when some row of the wavefront has a new maximum ------
     float mx = fmaxf(s[0][0], s[1][0]);
@@ -428,7 +437,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
       m = m_new;
     }
     // ---- O += V(t-1) P(t-1) on the matrix cores, P(t) = exp2(c S(t) - c m) on the vector ALU ----
-    if constexpr (!FIRST) pv(pb_prev, cur ^ 1);
+    if constexpr (!FIRST) pv_part(pb_prev, cur ^ 1, std::integral_constant<int, NPRE>{}, std::integral_constant<int, 4 * DT - NPRE>{});
     const float mc = (m == -INFINITY) ? 0.0f : m * p.c;
     float rs0 = 0.0f, rs1 = 0.0f;
     uint32_t pb[2][8];
@@ -449,11 +458,11 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
       // so the vector ALU works in the shadow of the matrix core instead of after it
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // operands of the first two go out ahead
 #pragma unroll
-      for (int i = 0; i < 4 * DT; ++i) {
+      for (int i = 0; i < 4 * DT - NPRE; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 LDS reads
-        __builtin_amdgcn_sched_group_barrier(0x002, 20 / DT, 0);  // VALU (fma, add, cvt)
-        __builtin_amdgcn_sched_group_barrier(0x400, 8 / DT, 0);   // transcendental (exp2)
+        __builtin_amdgcn_sched_group_barrier(0x002, (80 + 4 * DT - NPRE - 1) / (4 * DT - NPRE), 0);  // VALU: 80 per tile (fma, add, cvt)
+        __builtin_amdgcn_sched_group_barrier(0x400, (32 + 4 * DT - NPRE - 1) / (4 * DT - NPRE), 0);  // transcendental: 32 exp2 per tile
       }
       // keep the softmax arithmetic in this block: without a use here the optimiser sinks it
       // past the barrier below, out of the matrix core's shadow
