@@ -95,6 +95,15 @@ __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t 
                : "s"(lds_addr), "v"(voff), "s"(base)
                : "memory", "m0");
 }
+// the same with the LDS address formed as lds_base + IMM in M0 by the one scalar instruction the
+// transfer needs anyway
+template <uint32_t IMM>
+__device__ __forceinline__ void dma16_at(const char* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base), "v"(voff), "s"(base), "n"(IMM)
+               : "memory", "m0", "scc");
+}
 // same for 4 bytes per lane (global_load_lds_dword): lane l lands at lds_addr + 4 l
 __device__ __forceinline__ void dma4(const char* base, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
@@ -136,6 +145,8 @@ struct Loader {
   int wave, lane, kv_len, rl, cgk, cgv;
   int shk, shv;                 // 4-bit store: nibble of this lane's K / V chunk (4 = high)
   uint32_t lds_k, lds_v;        // LDS addresses of the K and V buffers (wavefront-uniform)
+  uint32_t lds_kw, lds_vw;      // the same plus this wavefront's row-group offset
+  uint32_t koffs[NI], voffs[NI];  // byte offset of this lane's chunk of row group i inside a tile
   // uint8 path staging registers
   u32x2_t kc[NI], vc[NI];
   float ksr[NI], vsr[NI];
@@ -175,11 +186,37 @@ struct Loader {
     shv = u4_shift<D>(cgv);
     k_step = (int64_t)NWAVES * RPW * p.k_st * ESZ;
     v_step = (int64_t)NWAVES * RPW * p.v_st * ESZ;
+    lds_kw = lds_k + (uint32_t)(wave * RPW * CPR * 16);
+    lds_vw = lds_v + (uint32_t)(wave * RPW * CPR * 16);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      koffs[i] = koff + (uint32_t)(i * k_step);
+      voffs[i] = voff + (uint32_t)(i * v_step);
+    }
+  }
+
+  // a full tile of the bf16 cache into buffer BUF: one scalar add (into M0) per DMA instruction
+  template <bool IS_K, int BUF, int I = 0>
+  __device__ __forceinline__ void issue_full(const char* tb) {
+    dma16_at<(uint32_t)((BUF * BN + NWAVES * I * RPW) * CPR * 16)>(tb, IS_K ? koffs[I] : voffs[I], IS_K ? lds_kw : lds_vw);
+    if constexpr (I + 1 < NI) issue_full<IS_K, BUF, I + 1>(tb);
+  }
+  template <bool IS_K, int BUF>
+  __device__ __forceinline__ void issue_full(int tile) {
+    issue_full<IS_K, BUF, 0>((IS_K ? kbase : vbase) + tile * (IS_K ? k_tile_bytes : v_tile_bytes));
   }
 
   template <bool IS_K>
   __device__ __forceinline__ void issue_one(Smem<D>& sm, int tile, int buf, int tid) {
     const int key0 = tile * BN;
+    if constexpr (!U8) {
+      if (key0 + BN <= kv_len) {  // the common case: immediate LDS offsets, shared scalar base
+        if (buf == 0) issue_full<IS_K, 0>(tile);
+        else issue_full<IS_K, 1>(tile);
+        issue_tp<IS_K>(sm, tile, buf);
+        return;
+      }
+    }
     const char* base = IS_K ? kbase : vbase;
     const int64_t st = IS_K ? k_st : v_st;
     const int64_t step = IS_K ? k_step : v_step;
@@ -215,9 +252,15 @@ struct Loader {
         }
       }
     }
-    // token positions of the K tile: one 4-byte DMA per lane of wavefront 0 (slots past the end
-    // re-read the last valid one and are overwritten with INT_MAX when the tile lands)
+    issue_tp<IS_K>(sm, tile, buf);
+  }
+
+  // token positions of the K tile: one 4-byte DMA per lane of wavefront 0 (slots past the end
+  // re-read the last valid one and are overwritten with INT_MAX when the tile lands)
+  template <bool IS_K>
+  __device__ __forceinline__ void issue_tp(Smem<D>& sm, int tile, int buf) {
     if (IS_K && tp && wave == 0) {
+      const int key0 = tile * BN;
       const uint32_t dst = lds_addr_of(&sm.tp[buf][0]);
       dma4((const char*)(tp + key0), (uint32_t)min(lane, kv_len - 1 - key0) * 4, __builtin_amdgcn_readfirstlane(dst));
     }
@@ -400,16 +443,20 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
   // the iteration.
   Loader<D, KV> ld;
   ld.init(p, sm, b, kvh, tid);
-  uint32_t pb_prev[2][8];
+  uint32_t pbs[2][2][8];  // packed P of the tile in buffer 0 / 1: written by one step, multiplied by the next
   // every split owns at least one tile (the host sizes the splits that way)
   ld.template issue_one<true>(sm, tile_begin, 0, tid);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first K tile and the Q fragments have arrived
   ld.template land<true>(sm, tile_begin, 0, tid);
   __syncthreads();
   // one pipeline step; the first one has no previous tile to multiply
-  auto step = [&](auto first_tag, int t) {
+  // one pipeline step on the tile in buffer CUR (compile time: LDS offsets become immediates and P
+  // alternates between two register sets instead of being copied)
+  auto step = [&](auto first_tag, auto cur_tag, int t) {
     constexpr bool FIRST = decltype(first_tag)::value;
-    const int cur = (t - tile_begin) & 1;
+    constexpr int cur = decltype(cur_tag)::value;
+    uint32_t (&pb_prev)[2][8] = pbs[cur ^ 1];
+    uint32_t (&pb)[2][8] = pbs[cur];
     const bool has1 = t + 1 < tile_end;
     ld.template issue_one<false>(sm, t, cur, tid);
     if (has1) ld.template issue_one<true>(sm, t + 1, cur ^ 1, tid);
@@ -440,7 +487,6 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     if constexpr (!FIRST) pv_part(pb_prev, cur ^ 1, std::integral_constant<int, NPRE>{}, std::integral_constant<int, 4 * DT - NPRE>{});
     const float mc = (m == -INFINITY) ? 0.0f : m * p.c;
     float rs0 = 0.0f, rs1 = 0.0f;
-    uint32_t pb[2][8];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -478,19 +524,26 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
           for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
       }
     }
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) pb_prev[mt][i] = pb[mt][i];
     // ---- publish the tiles that were in flight -------------------------------------------------
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's DMA / loads have landed
     ld.template land<false>(sm, t, cur, tid);
     if (has1) ld.template land<true>(sm, t + 1, cur ^ 1, tid);
     __syncthreads();
   };
-  step(std::true_type{}, tile_begin);
-  for (int t = tile_begin + 1; t < tile_end; ++t) step(std::false_type{}, t);
-  pv(pb_prev, (tile_end - 1 - tile_begin) & 1);
+  constexpr std::integral_constant<int, 0> B0{};
+  constexpr std::integral_constant<int, 1> B1{};
+  step(std::true_type{}, B0, tile_begin);
+  int t = tile_begin + 1;
+  for (; t + 1 < tile_end; t += 2) {
+    step(std::false_type{}, B1, t);
+    step(std::false_type{}, B0, t + 1);
+  }
+  if (t < tile_end) {
+    step(std::false_type{}, B1, t);
+    pv(pbs[1], 1);
+  } else {
+    pv(pbs[0], 0);
+  }
 
   // ---- epilogue -----------------------------------------------------------------------------
   const float lt = sum_halves(l);
