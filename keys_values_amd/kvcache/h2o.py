@@ -486,7 +486,10 @@ class H2OKVCache:
                     done = torch.cuda.Event()
                     done.record(self._side_stream)
                 self._select_done = done
-                self._select_keep = (attn_weights, nxt)  # alive until the second stream is done with them
+                # the second stream reads these: tell the allocator, and keep them until the wait
+                attn_weights.record_stream(self._side_stream)
+                nxt.record_stream(self._side_stream)
+                self._select_keep = (attn_weights, nxt)
         self._have_next = full
 
 
