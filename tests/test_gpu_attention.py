@@ -198,3 +198,56 @@ def test_full_size_prefill_properties(gpu):
     assert rel_err(out_s.float().cpu(), out.float().cpu()) < 1e-2
     w_back = torch.zeros_like(w_c).scatter_(-1, perm, w_s.cpu())
     torch.testing.assert_close(w_back, w_c, rtol=W_RTOL, atol=1e-6)
+
+
+def _random_cases(n, seed):
+    """Seeded shapes that mix what the fixed cases vary one at a time: group size, head size, ragged
+    query and key counts, forced splits, position layout, store."""
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        G = rnd.choice([1, 2, 4, 8])
+        Hkv = rnd.choice([1, 2, 3])
+        D = rnd.choice([64, 128])
+        T = rnd.choice([1, 2, 63, 64, 65, 127, 200, 333, 512, 777, 1025, 2049])
+        q_len = rnd.randint(1, min(T, 150))
+        cases.append((len(cases), rnd.choice([1, 2]), G * Hkv, Hkv, q_len, T, D, rnd.choice([0, 0, 1, 2, 3, 5]), rnd.choice(["contig", "scattered"]),
+                      rnd.choice(["bf16", "bf16", "u8", "u4"])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(28, 20240607), ids=lambda c: "-".join(str(x) for x in c))
+def test_prefill_and_decode_random_shapes(gpu, case):
+    n, B, Hq, Hkv, q_len, T, D, splits, layout, store = case
+    q, k, v, gen = make_qkv(5000 + n, B, Hq, Hkv, q_len, T, D)
+    scale = 1.0 / math.sqrt(D)
+    if layout == "contig":
+        input_pos, tp = T - q_len, None
+    else:
+        input_pos = T + 37
+        tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len)
+    quant = None
+    kg, vg = k.to(gpu), v.to(gpu)
+    if store != "bf16":
+        bits = 8 if store == "u8" else 4
+        (kc, ks, kz), (vc, vs, vz) = O.quantize_rows(k, bits), O.quantize_rows(v, bits)
+        k, v = O.dequantize_rows(kc, ks, kz), O.dequantize_rows(vc, vs, vz)
+        if bits == 4:
+            kc, vc = O.compress4(kc), O.compress4(vc)
+        kg, vg = kc.to(gpu), vc.to(gpu)
+        quant = ops.QuantState(ks.to(gpu), kz.to(gpu), vs.to(gpu), vz.to(gpu))
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, None if tp is None else tp.long())
+    out, w, lse = ops.prefill_core(q.to(gpu), kg, vg, scale, input_pos, None if tp is None else tp.to(gpu), return_weights=True,
+                                   return_lse=True, output_transposed=False, quant=quant, num_splits=splits)
+    torch.cuda.synchronize()
+    assert rel_err(out.float().cpu(), o_ref.float()) < 2e-2
+    torch.testing.assert_close(w.cpu(), w_ref, rtol=1e-3, atol=1e-6)
+    torch.testing.assert_close(lse.cpu(), O.lse2(q, k, scale, input_pos, None if tp is None else tp.long()), rtol=0, atol=2e-3)
+    # single-token decode over the same store (unmasked: the new token is the newest)
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], k, v, scale, 10 * T + 100, None)
+    out1, w1, _ = ops.decode_core(q[:, :, :1].to(gpu), kg, vg, scale, return_weights=True, quant=quant)
+    torch.cuda.synchronize()
+    assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
+    torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
