@@ -44,8 +44,10 @@ def _run_steps(gpu, cache, ref, q, k, v, n_prefill, steps):
     cache.forward(q[:, :, :n_prefill].to(gpu), k[:, :, :n_prefill].to(gpu), v[:, :, :n_prefill].to(gpu))
     pos = n_prefill
     for num in steps:
-        sl = slice(pos, pos + num)
         assert cache.max_forward_length() == ref.max_forward_length()
+        if callable(num):  # a step size drawn from what the cache accepts now
+            num = num(ref.max_forward_length())
+        sl = slice(pos, pos + num)
         had_choice = ref.next_index is not None
         o_ref, w_ref, index = ref.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
         if had_choice:
@@ -119,6 +121,43 @@ def test_policy_variants_chunked_steps(gpu, name, kwargs):
                               grace_period=cache.grace_period, normalize_scores=cache.normalize_scores,
                               num_bits=cache.num_bits or 8)
     _run_steps(gpu, cache, ref, q, k, v, L, steps)
+
+
+def _random_policies(n, seed):
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for i in range(n):
+        Hkv = rnd.choice([1, 2, 3])
+        L = rnd.choice([130, 256, 333, 600])
+        chunk = rnd.choice([1, 8, 33, 64])
+        quantized = rnd.random() < 0.5
+        cases.append(dict(i=i, B=rnd.choice([1, 2]), Hq=Hkv * rnd.choice([1, 2, 4]), Hkv=Hkv, L=L, D=rnd.choice([64, 128]), chunk=chunk,
+                          gp=rnd.choice([0, 0, 3, chunk, 40]), quantized=quantized, bits=rnd.choice([4, 8]) if quantized else 8,
+                          v_length=rnd.random() < 0.4, q_hitter=quantized and rnd.random() < 0.5, normalize=rnd.random() < 0.4,
+                          c=rnd.choice([0.25, 0.5, 0.8]), short=rnd.randint(0, 50)))
+    return cases
+
+
+@pytest.mark.parametrize("cfg", _random_policies(16, 424242), ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items()))
+def test_random_policy_configurations(gpu, cfg):
+    """Seeded mixes of the options the fixed cases vary one at a time, with step sizes drawn from what
+    the cache accepts at each step (test/kvcache/test_h2o.py:49-106, test/kvcache/test_attn_weights.py)."""
+    import random
+
+    rnd = random.Random(cfg["i"])
+    B, Hq, Hkv, L, D, chunk = cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["L"], cfg["D"], cfg["chunk"]
+    nsteps = 14
+    steps = [lambda m: rnd.randint(1, min(m, chunk))] * nsteps
+    q, k, v = _inputs(900 + cfg["i"], B, Hq, Hkv, L + nsteps * chunk, D, spread=True)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, normalize_scores=cfg["normalize"], grace_period=cfg["gp"],
+                       quantized=cfg["quantized"], num_bits=cfg["bits"], v_length=cfg["v_length"], q_hitter=cfg["q_hitter"],
+                       combination_constant=cfg["c"], device=gpu)
+    ref = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, quantized=cfg["quantized"], v_length=cfg["v_length"],
+                              q_hitter=cfg["q_hitter"], combination_constant=cfg["c"], grace_period=cfg["gp"],
+                              normalize_scores=cfg["normalize"], num_bits=cfg["bits"])
+    _run_steps(gpu, cache, ref, q, k, v, L - cfg["short"], steps)
 
 
 @pytest.mark.parametrize("cls,kwargs", [
