@@ -121,13 +121,22 @@ def load():
     if not os.path.exists(LIB_PATH):
         _load_error = f"{LIB_PATH} not found: build it with `python -m keys_values_amd.build`"
         raise ImportError(_load_error)
-    lib = ctypes.CDLL(LIB_PATH)
-    for name, (res, args) in SYMBOLS.items():
-        fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
-        fn.restype = res
-        fn.argtypes = args
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+    except (OSError, AttributeError) as ex:
+        _load_error = f"{LIB_PATH}: {ex}"
+        raise
+    _load_error = None
     _lib = lib
     return lib
+
+
+def load_error():
+    return _load_error
 
 
 class KvxError(RuntimeError):

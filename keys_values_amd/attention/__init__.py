@@ -2,6 +2,7 @@ from .ops import (  # noqa: F401
     QuantState,
     get_device_count,
     get_device_info,
+    get_load_error,
     is_available,
     sdpa_decode,
     sdpa_prefill,

@@ -46,6 +46,12 @@ def is_available() -> bool:
         return False
 
 
+def get_load_error() -> Optional[str]:
+    """Message of the last failed attempt to load the library, None if it loaded or was not tried
+    (keys_values/attention/flashinfer_ops.py:134-147)."""
+    return _lib.load_error()
+
+
 def get_device_count() -> int:
     return _lib.load().kvx_device_count()
 

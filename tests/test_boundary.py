@@ -83,6 +83,24 @@ def test_no_cpu_fallback():
         ops.decode_core(q[:, :, :1], k, k, 0.125)
 
 
+def test_load_error_is_reported(monkeypatch, tmp_path):
+    # keys_values/attention/flashinfer_ops.py:86-147: a failed load leaves a message, a good one None
+    from keys_values_amd import attention
+
+    _lib.load()
+    assert attention.get_load_error() is None
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "_load_error", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libkvx.so"))
+    with pytest.raises(ImportError):
+        _lib.load()
+    assert "not found" in attention.get_load_error()
+    assert not attention.is_available()
+    monkeypatch.undo()
+    _lib.load()
+    assert attention.get_load_error() is None
+
+
 def test_hip_sdpa_keeps_reference_errors():
     # keys_values/attention/flashinfer_wrapper.py:406-432, keys_values/attention/sdpa_wrapper.py:24-47
     s = HipSDPA.__new__(HipSDPA)
