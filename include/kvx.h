@@ -226,8 +226,10 @@ int kvx_dequantize_blocks(const kvx_block_quant_args* args, void* stream);
  *              input_pos - grace_period + j, scores, v_norm, q_errors) moves to index[b,h,j];
  *              then the new token num1 + j goes into `ring` (position input_pos + num1 + j);
  *   j >= num2: the new token j - num2 goes into index[b,h,j] (position input_pos + j - num2).
- * A moved row of a uint8 cache keeps its codes, scale and zero point (the reference dequantises and
- * re-quantises it, which is not the identity). Slots in index must lie outside the ring.
+ * A moved row of a quantised cache is dequantised and quantised again on its way to index[b,h,j], as
+ * the reference's write does (the ring rows come out of its dequantised buffer,
+ * keys_values/kvcache/quant_buffers.py:732-775); its q_errors entry moves unchanged. Slots in index
+ * must lie outside the ring.
  *
  * replay_log (see the field comments) records the slots written.
  *

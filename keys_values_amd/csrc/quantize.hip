@@ -356,9 +356,10 @@ __device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, flo
 }
 
 // One lane per 8 elements of one job (b, h, j), for K and V. Without a ring move job j writes new
-// token j into index[b,h,j]. With one (j < grace_num) the lane first carries its 8 elements of ring
-// slot grace_slots[j] over to index[b,h,j], then writes new token num - grace_num + j into the ring
-// slot: the read and the write of that slot are issued by the same lane, in this order.
+// token j into index[b,h,j]. With one (j < grace_num) the lanes of the job first carry ring slot
+// grace_slots[j] over to index[b,h,j], then write new token num - grace_num + j into the ring slot:
+// the read and the write of that slot are issued by the same wavefront, in this order, and the
+// read's data is consumed before the write is issued.
 template <int D, int KV>
 __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
   constexpr bool U8 = KV != KVX_KV_BF16;  // a quantised store: codes + row state
@@ -393,23 +394,58 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   uint8_t* kc_row = (uint8_t*)a.k_cache + (b * a.kc_stride_b + hh * a.kc_stride_h) * ES + ccol * 8 * ES;
   uint8_t* vc_row = (uint8_t*)a.v_cache + (b * a.vc_stride_b + hh * a.vc_stride_h) * ES + ccol * 8 * ES;
 
-  if (ok && moves) {
-    if constexpr (!U8) {
-      *(u32x4_t*)(kc_row + (int64_t)slot * a.kc_stride_t * ES) = *(const u32x4_t*)(kc_row + (int64_t)ring * a.kc_stride_t * ES);
-      *(u32x4_t*)(vc_row + (int64_t)slot * a.vc_stride_t * ES) = *(const u32x4_t*)(vc_row + (int64_t)ring * a.vc_stride_t * ES);
-    } else {
+  // a quantised store: quantise the row held as (krow, vrow) by the LPR lanes of this job and store
+  // it in slot `target`; every lane of the wavefront calls it (the row reductions need all lanes of a row)
+  auto put = [&](const u32x4_t& krow, const u32x4_t& vrow, int target, bool doit, bool want_err) -> float {
+    float s1, s2, err = 0.0f;
+    int32_t z1, z2;
+    u32x2_t kc = U4 ? quantize4<LPR>(krow, s1, z1) : quantize8<LPR>(krow, s1, z1);
+    u32x2_t vc = U4 ? quantize4<LPR>(vrow, s2, z2) : quantize8<LPR>(vrow, s2, z2);
+    if (want_err) err = row_quant_error<LPR>(krow, kc, s1, z1) + row_quant_error<LPR>(vrow, vc, s2, z2);  // uniform branch
+    if constexpr (U4) {  // byte j = code[j] << 4 | code[j + D/2]: the partner lane holds the low nibbles
+      kc = u32x2_t{(kc[0] << 4) | (uint32_t)__shfl_xor(kc[0], LPR / 2, 64), (kc[1] << 4) | (uint32_t)__shfl_xor(kc[1], LPR / 2, 64)};
+      vc = u32x2_t{(vc[0] << 4) | (uint32_t)__shfl_xor(vc[0], LPR / 2, 64), (vc[1] << 4) | (uint32_t)__shfl_xor(vc[1], LPR / 2, 64)};
+    }
+    if (doit) {
       if (stores) {
-        *(u32x2_t*)(kc_row + (int64_t)slot * a.kc_stride_t) = *(const u32x2_t*)(kc_row + (int64_t)ring * a.kc_stride_t);
-        *(u32x2_t*)(vc_row + (int64_t)slot * a.vc_stride_t) = *(const u32x2_t*)(vc_row + (int64_t)ring * a.vc_stride_t);
+        *(u32x2_t*)(kc_row + (int64_t)target * a.kc_stride_t) = kc;
+        *(u32x2_t*)(vc_row + (int64_t)target * a.vc_stride_t) = vc;
       }
       if (col == 0) {
-        a.k_scale[qs_row + slot] = a.k_scale[qs_row + ring];
-        a.k_zp[qs_row + slot] = a.k_zp[qs_row + ring];
-        a.v_scale[qs_row + slot] = a.v_scale[qs_row + ring];
-        a.v_zp[qs_row + slot] = a.v_zp[qs_row + ring];
+        a.k_scale[qs_row + target] = s1;
+        a.k_zp[qs_row + target] = z1;
+        a.v_scale[qs_row + target] = s2;
+        a.v_zp[qs_row + target] = z2;
       }
     }
-    if (col == 0) {
+    return err;
+  };
+
+  if (a.grace_num > 0) {  // uniform over the launch
+    const bool mv = ok && moves;
+    if constexpr (!U8) {
+      if (mv) {
+        *(u32x4_t*)(kc_row + (int64_t)slot * a.kc_stride_t * ES) = *(const u32x4_t*)(kc_row + (int64_t)ring * a.kc_stride_t * ES);
+        *(u32x4_t*)(vc_row + (int64_t)slot * a.vc_stride_t * ES) = *(const u32x4_t*)(vc_row + (int64_t)ring * a.vc_stride_t * ES);
+      }
+    } else {
+      // The moved row is written like any other: its dequantised values are quantised again
+      // (keys_values/kvcache/attn_weights.py:578-590 reads the ring rows from the dequantised buffer
+      // and hands them to the same write as the new rows), which is not the identity on the codes.
+      u32x4_t krow = {0, 0, 0, 0}, vrow = {0, 0, 0, 0};
+      if (mv) {
+        u32x2_t kq = *(const u32x2_t*)(kc_row + (int64_t)ring * a.kc_stride_t);
+        u32x2_t vq = *(const u32x2_t*)(vc_row + (int64_t)ring * a.vc_stride_t);
+        if constexpr (U4) {
+          kq = u4_codes(kq, col < LPR / 2 ? 4 : 0);
+          vq = u4_codes(vq, col < LPR / 2 ? 4 : 0);
+        }
+        krow = dequant_words(kq[0], kq[1], a.k_zp[qs_row + ring], a.k_scale[qs_row + ring]);
+        vrow = dequant_words(vq[0], vq[1], a.v_zp[qs_row + ring], a.v_scale[qs_row + ring]);
+      }
+      put(krow, vrow, slot, mv, false);
+    }
+    if (mv && col == 0) {
       a.token_pos[tp_row + slot] = a.input_pos - a.grace_period + j;
       if (a.scores) a.scores[sc_row + slot] = a.scores[sc_row + ring];
       if (a.v_norm) a.v_norm[sc_row + slot] = a.v_norm[sc_row + ring];
@@ -424,27 +460,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
       *(u32x4_t*)(vc_row + (int64_t)wslot * a.vc_stride_t * ES) = vr;
     }
   } else {
-    float s1, s2;
-    int32_t z1, z2;
-    u32x2_t kc = U4 ? quantize4<LPR>(kr, s1, z1) : quantize8<LPR>(kr, s1, z1);
-    u32x2_t vc = U4 ? quantize4<LPR>(vr, s2, z2) : quantize8<LPR>(vr, s2, z2);
-    if (a.q_errors) qerr = row_quant_error<LPR>(kr, kc, s1, z1) + row_quant_error<LPR>(vr, vc, s2, z2);  // uniform branch
-    if constexpr (U4) {  // byte j = code[j] << 4 | code[j + D/2]: the partner lane holds the low nibbles
-      kc = u32x2_t{(kc[0] << 4) | (uint32_t)__shfl_xor(kc[0], LPR / 2, 64), (kc[1] << 4) | (uint32_t)__shfl_xor(kc[1], LPR / 2, 64)};
-      vc = u32x2_t{(vc[0] << 4) | (uint32_t)__shfl_xor(vc[0], LPR / 2, 64), (vc[1] << 4) | (uint32_t)__shfl_xor(vc[1], LPR / 2, 64)};
-    }
-    if (ok) {
-      if (stores) {
-        *(u32x2_t*)(kc_row + (int64_t)wslot * a.kc_stride_t) = kc;
-        *(u32x2_t*)(vc_row + (int64_t)wslot * a.vc_stride_t) = vc;
-      }
-      if (col == 0) {
-        a.k_scale[qs_row + wslot] = s1;
-        a.k_zp[qs_row + wslot] = z1;
-        a.v_scale[qs_row + wslot] = s2;
-        a.v_zp[qs_row + wslot] = z2;
-      }
-    }
+    qerr = put(kr, vr, wslot, ok, a.q_errors != nullptr);
   }
   float vnorm = 0.0f;
   if (a.v_norm) vnorm = row_norm<LPR>(vr);  // uniform branch: every lane takes part in the reduction

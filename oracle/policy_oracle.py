@@ -26,10 +26,10 @@ How it is pinned (tests/test_policy_oracle.py):
   quantisation error is checked against explicit float loops.
 * Replay log: the concatenation of its blocks is the concatenation of every step's slots, and
   ``extract_index`` is a slice of it, checked for every start and length on a small log.
-* A quantised store here holds dequantise(quantise(row)) for every row written; a row moved out of
-  the ring keeps its stored value (the reference re-quantises the dequantised row when it writes the
-  working buffer back, keys_values/kvcache/quant_buffers.py:732-775, which may change it by one
-  quantisation step: parity unpinned for that difference, see the tests' tolerances).
+* A quantised store here holds dequantise(quantise(row)) for every row written, and a row moved out
+  of the ring is written once more (the reference reads it from the dequantised buffer and writes it
+  back through the quantiser, keys_values/kvcache/quant_buffers.py:732-775): checked against the row
+  quantiser applied by hand, twice for moved rows, once for all others.
 """
 
 import math
@@ -266,8 +266,10 @@ class PolicyCacheOracle:
             new_tps = torch.arange(self.input_pos - gp, self.input_pos - gp + num, dtype=torch.int32)
             self.token_pos.scatter_(-1, index, new_tps.view(1, 1, -1).expand(B, Hkv, -1))
             # :578-590: [ring rows | new rows] go to [index | ring slots]
-            key_cp = torch.cat((self.k.gather(-2, gi(positions)), new_k), dim=-2)
-            value_cp = torch.cat((self.v.gather(-2, gi(positions)), new_v), dim=-2)
+            # the ring rows come out of the dequantised buffer and go through the same write as the new
+            # rows, which quantises them again (keys_values/kvcache/quant_buffers.py:732-775)
+            key_cp = torch.cat((self._stored(self.k.gather(-2, gi(positions))), new_k), dim=-2)
+            value_cp = torch.cat((self._stored(self.v.gather(-2, gi(positions))), new_v), dim=-2)
             fused = torch.cat((index, positions), dim=-1)
             self.k.scatter_(-2, gi(fused), key_cp)
             self.v.scatter_(-2, gi(fused), value_cp)

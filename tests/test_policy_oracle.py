@@ -83,6 +83,32 @@ def test_grace_period_against_a_per_slot_model(gp, steps):
         pos += num
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantised_ring_row_is_written_like_a_new_row(bits):
+    """A row that leaves the ring is read as bf16 values and written by the same write as the new rows
+    (keys_values/kvcache/attn_weights.py:578-590, keys_values/kvcache/quant_buffers.py:732-775): its
+    second stay in the store holds quantise(dequantise(.)) of the first, once; rows that are not
+    written keep their content."""
+    B, Hq, Hkv, L, D, gp = 1, 2, 1, 32, 16, 4
+    q, k, v = _inputs(11, B, Hq, Hkv, L + 12, D)
+    ora = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=4, grace_period=gp, quantized=True, num_bits=bits)
+    ora.prefill(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    first = {t: O.dequantize_rows(*O.quantize_rows(k[0, 0, t : t + 1], bits))[0] for t in range(L + 12)}
+    second = {t: O.dequantize_rows(*O.quantize_rows(first[t].unsqueeze(0), bits))[0] for t in first}
+    moved = set()
+    changed = 0
+    pos = L
+    for num in (3, 4, 1, 4):
+        ora.forward(q[:, :, pos : pos + num], k[:, :, pos : pos + num], v[:, :, pos : pos + num])
+        pos += num
+        moved |= {t for t in range(L - gp, pos - gp)}  # tokens that have left the ring by now
+        for slot, t in enumerate(ora.token_pos[0, 0].tolist()):
+            want = second[t] if t in moved else first[t]
+            assert torch.equal(ora.k[0, 0, slot], want), (t, slot)
+            changed += int(t in moved and not torch.equal(first[t], second[t]))
+    assert changed > 0, "the case must contain a row for which writing twice is not the identity"
+
+
 def test_v_length_with_equal_norms_is_plain_h2o():
     # sum_k W = q_len, so a constant |v| cancels: instantaneous score == W
     B, Hq, Hkv, L, D, chunk = 1, 4, 2, 64, 16, 8
