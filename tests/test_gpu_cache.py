@@ -33,7 +33,7 @@ def gpu_quantize(lib, x_gpu):
     return codes, sc, zp
 
 
-@pytest.mark.parametrize("rows,D", [(1, 128), (7, 64), (1000, 128), (4099, 64), (65536, 128)])
+@pytest.mark.parametrize("rows,D", [(1, 128), (7, 64), (1000, 128), (4099, 64), (65536, 128), (8 * 65536, 128)])
 def test_quantize_rows_bit_exact(kvx, gpu, rows, D):
     x = outlier_rows(2, rows, D)
     if rows >= 7:  # edge rows: constant, all negative, tiny range, extremes of bf16 dynamics
@@ -387,6 +387,51 @@ def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, B, Hq, Hkv, T, D, lim
     n_ref = O.h2o_update_select(s_ref, w_ref, T, limit, 1, normalize=normalize, token_pos=tp, input_pos=input_pos, prefill_len=prefill_len)
     torch.testing.assert_close(sc_g.cpu(), s_ref, rtol=1e-3, atol=1e-6)
     _sets_equal_away_from_ties(nxt.cpu().long(), n_ref, (s_ref[..., :limit] / (input_pos - torch.maximum(tp, torch.tensor(prefill_len - 1)))[..., :limit].float()) if normalize else s_ref[..., :limit], 1)
+
+
+def test_full_size_decode_h2o_properties(kvx, gpu):
+    """Configuration 4 at its real shape (B8, 32/8 heads, D128, 131072 slots, 4.3 GB of bf16 K/V, byte
+    offsets beyond 2^31): the fused decode + H2O step against the separate calls, the weights of a
+    token sum to one, the scores grow by exactly the weights, the evicted slot holds the minimum, and
+    the last (batch, KV head) pair — the largest offsets — against the oracle."""
+    B, Hq, Hkv, T, D = 8, 32, 8, 131072, 128
+    G = Hq // Hkv
+    torch.manual_seed(3)
+    k = torch.randn(B, Hkv, T, D, device=gpu, dtype=torch.bfloat16)
+    v = torch.randn(B, Hkv, T, D, device=gpu, dtype=torch.bfloat16)
+    q = torch.randn(B, Hq, 1, D, device=gpu, dtype=torch.bfloat16)
+    scores0 = torch.rand(B, Hkv, T, device=gpu) * 0.01
+    scale = 1.0 / math.sqrt(D)
+    out_a, w_a, _ = ops.decode_core(q, k, v, scale, return_weights=True)
+    out_b = torch.empty((B, Hq, D), dtype=torch.bfloat16, device=gpu)
+    ov = out_b.unsqueeze(2)
+    sc_g = scores0.clone()
+    nxt = torch.full((B, Hkv, 1), -1, dtype=torch.int32, device=gpu)
+    a = _lib.SdpaArgs()
+    ops._fill_common(a, q, k, v, scale, T - 1, None, None, 0)
+    a.o, a.o_stride_b, a.o_stride_h, a.o_stride_t = ov.data_ptr(), ov.stride(0), ov.stride(1), ov.stride(2)
+    h = _lib.H2OArgs()
+    h.B, h.Hkv, h.kv_len, h.limit, h.k = B, Hkv, T, T, 1
+    h.scores, h.sc_stride_b, h.sc_stride_h = sc_g.data_ptr(), sc_g.stride(0), sc_g.stride(1)
+    h.next_index = nxt.data_ptr()
+    nb_h = (kvx.kvx_h2o_workspace_bytes(ctypes.byref(h)) + 255) // 256 * 256
+    nb_a = kvx.kvx_sdpa_decode_h2o_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(nb_h + nb_a + 256, dtype=torch.uint8, device=gpu)
+    h.workspace, h.workspace_bytes = ws.data_ptr(), nb_h
+    a.workspace, a.workspace_bytes = ws.data_ptr() + nb_h, nb_a
+    _lib.check(kvx.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    assert torch.equal(out_b, out_a)
+    assert (w_a >= 0).all()
+    torch.testing.assert_close(w_a.sum(-1), torch.ones(B, Hkv, device=gpu), rtol=2e-5, atol=0)
+    assert torch.equal(sc_g, scores0 + w_a)
+    chosen = sc_g.gather(-1, nxt.long())
+    assert torch.equal(chosen.squeeze(-1), sc_g.min(-1).values)
+    b, kh = B - 1, Hkv - 1
+    o_ref, w_ref = O.sdpa_in_blocks(q[b : b + 1, G * kh : G * kh + G].cpu(), k[b : b + 1, kh : kh + 1].cpu(), v[b : b + 1, kh : kh + 1].cpu(),
+                                    scale, T - 1, None)
+    assert rel_err(out_b[b, G * kh : G * kh + G].float().cpu(), o_ref[0, :, 0].float()) < 2e-2
+    torch.testing.assert_close(w_a[b : b + 1, kh : kh + 1].cpu(), w_ref, rtol=1e-3, atol=1e-9)
 
 
 def test_overlapped_selection_equals_in_order_selection(gpu):
