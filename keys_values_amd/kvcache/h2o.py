@@ -12,9 +12,12 @@ position mask, add the score-sums to the cumulative scores, choose the next slot
 
 The K/V store is either bf16 (``h2o-default``) or codes with per-row scale / zero point: 8 bits
 (``h2o-torch-quantized8``) or 4 bits, two codes per byte (``h2o-torch-quantized4``;
-keys_values/kvcache/factory.py:50-66). In the second case the codes stay
-resident and the attention kernels dequantise them on load; the reference instead dequantises the
-whole cache into a bf16 working buffer per layer and re-quantises it afterwards
+keys_values/kvcache/factory.py:50-66). In the second case the codes stay resident and are never
+written back: single tokens and short chunks are attended to by kernels that dequantise on load; for a
+long chunk (``dequantize_chunk_rows`` query rows or more) the store is dequantised once into a bf16
+buffer shared by all caches of a device and stream, because every workgroup of the attention kernels
+would otherwise dequantise the whole store again. The reference dequantises the whole cache into a
+bf16 working buffer per layer and re-quantises it afterwards
 (keys_values/kvcache/quant_buffers.py:473-503,732-804).
 
 Policy variants on the same kernels: a grace period (the last ``grace_period`` slots are a ring of
@@ -40,6 +43,24 @@ from .replay import DEFAULT_REPLAY_LOG_BLOCKSIZE, AttnWeightsReplayLog, ReplayAr
 DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
 DEFAULT_COMBINATION_CONSTANT = 0.5  # keys_values/kvcache/qh2o.py:25
 MAX_SELECT = 4096  # largest k of kvx_h2o_update_select
+# Query rows (tokens x heads per KV head) of a chunk from which dequantising the store once per chunk
+# is faster than dequantising it inside the attention kernels (every 256 rows walk the whole store):
+# the copy costs two passes over the store, the kernels gain in proportion to the rows.
+DEFAULT_DEQUANTIZE_CHUNK_ROWS = 2048
+
+_dequant_buffers = {}
+
+
+def _dequant_scratch(device, numel: int):
+    """Two bf16 buffers of ``numel`` elements, grow-only, shared by the caches of one device and stream
+    (launches on a stream are ordered: a layer's attention has read them before the next layer's
+    dequantisation overwrites them)."""
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    buf = _dequant_buffers.get(key)
+    if buf is None or buf.numel() < 2 * numel:
+        buf = torch.empty(2 * numel, dtype=torch.bfloat16, device=device)
+        _dequant_buffers[key] = buf
+    return buf[:numel], buf[numel : 2 * numel]
 
 
 @dataclass(frozen=True)
@@ -70,7 +91,11 @@ class H2OKVCache:
         combination_constant: float = DEFAULT_COMBINATION_CONSTANT,
         replay_log_blocksize: Optional[int] = None,
         overlap_select: bool = False,
+        dequantize_chunk_rows: Optional[int] = DEFAULT_DEQUANTIZE_CHUNK_ROWS,
     ):
+        # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
+        # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
+        self.dequantize_chunk_rows = dequantize_chunk_rows
         # overlap_select: launch the score update + eviction choice of a chunk step on a second stream, so
         # that it runs beside whatever the caller enqueues next; the next forward waits for it. The scores,
         # the next slots and token_pos must then not be read from the caller's stream before
@@ -297,12 +322,30 @@ class H2OKVCache:
             out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
             out = out.unsqueeze(1)
         else:
+            rows = num * (hq // self.n_query_groups)
+            if quant is not None and self.dequantize_chunk_rows is not None and rows >= self.dequantize_chunk_rows:
+                kc, vc = self._dequantized(b, T)
+                quant = None
             out, w, _ = ops.prefill_core(query, kc, vc, self.scale_factor, input_pos, tp, return_weights=True,
                                          output_transposed=True, quant=quant)
         self._update(w, num)
         return out.reshape(b, num, hq * d)
 
     __call__ = forward
+
+    def _dequantized(self, b: int, T: int):
+        """bf16 views (b, n_query_groups, T, head_size) of the quantised store, dequantised into the shared
+        scratch by one launch per tensor (all slots of the first ``b`` batch entries: they are contiguous)."""
+        h, length, d = self.n_query_groups, self.cache_length, self.head_size
+        rows = b * h * length
+        kd, vd = _dequant_scratch(self.device, rows * d)
+        lib = _lib.load()
+        fn = lib.kvx_dequantize_rows4 if self.num_bits == 4 else lib.kvx_dequantize_rows
+        with torch.cuda.device(self.device):
+            stream = _lib.stream_ptr(self.device)
+            _lib.check(fn(self.k.data_ptr(), self.k_scale.data_ptr(), self.k_zp.data_ptr(), rows, d, kd.data_ptr(), d, stream))
+            _lib.check(fn(self.v.data_ptr(), self.v_scale.data_ptr(), self.v_zp.data_ptr(), rows, d, vd.data_ptr(), d, stream))
+        return kd.view(b, h, length, d)[:, :, :T], vd.view(b, h, length, d)[:, :, :T]
 
     def _prefill_step(self, query, key, value):
         """keys_values/kvcache/attn_weights.py:817-869 and keys_values/kvcache/base.py:567-581: fill the

@@ -434,6 +434,38 @@ def test_full_size_decode_h2o_properties(kvx, gpu):
     torch.testing.assert_close(w_a[b : b + 1, kh : kh + 1].cpu(), w_ref, rtol=1e-3, atol=1e-9)
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+def test_chunk_over_dequantised_copy_equals_fused_dequantisation(gpu, bits):
+    """Long chunks attend over a bf16 copy of the quantised store made once per chunk, short ones
+    dequantise inside the kernels: same values either way, so outputs, scores and evicted slots agree
+    (to summation order) and the store itself is bit-identical."""
+    B, Hq, Hkv, L, D, chunk = 2, 8, 2, 1024, 128, 96
+    steps = (96, 50, 96, 7, 96)
+    gen = torch.Generator().manual_seed(77)
+    total = L - 96 + sum(steps)
+    q = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    k = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    v = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    params = KVCacheParams(B, Hkv, L, D, Hq)
+    copy = H2OKVCache(params, max_chunk_size=chunk, quantized=True, num_bits=bits, device=gpu, dequantize_chunk_rows=1)
+    fused = H2OKVCache(params, max_chunk_size=chunk, quantized=True, num_bits=bits, device=gpu, dequantize_chunk_rows=None)
+    n0 = L - 96  # the first step fills the cache exactly
+    for c in (copy, fused):
+        c.forward(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    pos = n0
+    for num in steps:
+        sl = slice(pos, pos + num)
+        o1 = copy.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        o2 = fused.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        torch.cuda.synchronize()
+        assert rel_err(o1.float().cpu(), o2.float().cpu()) < 1e-2
+        torch.testing.assert_close(copy.scores, fused.scores, rtol=1e-3, atol=1e-6)
+        assert torch.equal(copy.k, fused.k) and torch.equal(copy.v, fused.v) and torch.equal(copy.token_pos, fused.token_pos)
+        if copy._have_next:
+            fused._next_index.copy_(copy._next_index)  # keep the two in step where scores tie in the last bits
+        pos += num
+
+
 def test_overlapped_selection_equals_in_order_selection(gpu):
     """overlap_select=True runs the score update + eviction choice on a second stream beside the
     caller's next launches; every result must equal the in-order cache's bit for bit."""
