@@ -14,7 +14,8 @@ Inputs are resident in HBM before the timed region.
 `--workload longctx` : BASELINE.json configs[4]: random-init Qwen3-4B-shaped stack (36 layers), 131072 random
                        tokens in chunks of 1024 after a 16384-token first chunk, uint8 H2O caches of 16384
                        slots per layer; end-to-end prefill tokens/s. One step = one whole sequence.
-                       `--layers N --tokens T` shrink it (stated in the output).
+                       `--layers N --tokens T` shrink it (stated in the output); `--tune-gemms` lets the GEMM
+                       library choose its kernels by measurement during the warm-up pass.
 `--workload policy`  : the same 1024-token chunk through the cache object (write with the ring move, attention,
                        score-sum, score update, choice of the next 1024 slots) for each eviction-policy variant
                        (grace period, normalised scores, V-norm weighting, Q-Hitter); ms per chunk step.
@@ -31,6 +32,7 @@ import json
 import math
 import os
 import sys
+import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -60,6 +62,8 @@ def parse():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
     ap.add_argument("--tokens", type=int, default=131072, help="longctx: prompt length")
+    ap.add_argument("--tune-gemms", action="store_true",
+                    help="longctx: let PyTorch's TunableOp pick the library GEMM kernels during the warm-up pass (adds about a minute)")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8", "uint4"],
                     help="cache storage for the prefill / decode workloads; uint8 = BASELINE.json configs[2]: codes + per-row "
                          "scale and zero point, dequantised inside the attention kernels; uint4 = the 4-bit store of the same quantiser")
@@ -404,6 +408,15 @@ def bench_longctx(args, torch, dev):
     sizes = model.chunk_sizes(seq)
     steps = max(1, min(args.steps, 3))
     warm = 1 if args.warmup > 0 else 0
+    if args.tune_gemms:  # the linear layers are plain library GEMMs: which kernel serves each shape is the library's choice
+        import torch.cuda.tunable as tunable
+
+        tunable.enable(True)
+        tunable.tuning_enable(True)
+        tunable.set_max_tuning_duration(15)
+        tunable.set_max_tuning_iterations(20)
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), "kvx_bench_tunableop.csv"))  # its results file: not into the tree
+        warm = 1
     for _ in range(warm):
         model.prefill(ids)
     torch.cuda.synchronize()
@@ -453,7 +466,7 @@ def bench_longctx(args, torch, dev):
         "config": {"workload": f"BASELINE.json configs[4]: random-init Qwen3-4B-shaped stack, {cfg.n_layer} layers, {seq} random tokens, "
                                f"chunks {sizes[0]} + {len(sizes) - 1} x {chunk}, uint8 H2O caches of {L} slots, seed 4",
                    "ms_per_step_gpu_events": round(ms_gpu, 2), "flops_attention_score_sums": attn, "flops_dense_layers": dense,
-                   "tflops_total": round((attn + dense) / (ms_step * 1e-3) / 1e12, 1)},
+                   "tflops_total": round((attn + dense) / (ms_step * 1e-3) / 1e12, 1), "library_gemms": "tuned (TunableOp)" if args.tune_gemms else "default"},
         "roofline": {"bound": "mfma", "kernel": "whole prefill (attention + score-sum kernels and library GEMMs)",
                      "achieved": round((attn + dense) / (ms_gpu * 1e-3) / 1e12, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round((attn + dense) / (ms_gpu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None},
