@@ -74,6 +74,97 @@ def test_validation_answers_without_a_gpu(kvx):
     assert kvx.kvx_device_count() >= 0
 
 
+def test_random_arguments_are_answered_not_trusted(kvx):
+    """Seeded random argument blocks (sizes from a set of edge values, pointers NULL / aligned /
+    misaligned, strides zero / negative / odd) through every entry point that takes one: each call must
+    come back with a status (no division by a zero size, no walk over a NULL pointer on the host).
+    Only where no device is visible: a block that happens to pass every check would be launched."""
+    import random
+
+    if kvx.kvx_device_count() > 0:
+        pytest.skip("a device is visible: random pointers must not reach a kernel")
+    rnd = random.Random(2024)
+    ints = [-1, 0, 1, 2, 3, 7, 8, 64, 100, 128, 256, 4096, 4097, 2**31 - 1]
+    ptrs = [0, 0, 0x10000, 0x10008, 0x10001]
+    strides = [-8, 0, 1, 8, 64, 128, 1024, 2**40]
+    codes = {_lib.KVX_OK, _lib.KVX_ERR_INVALID, _lib.KVX_ERR_UNSUPPORTED, _lib.KVX_ERR_WORKSPACE, _lib.KVX_ERR_HIP}
+
+    def fill(obj):
+        for name, ctype in obj._fields_:
+            if ctype is ctypes.c_void_p:
+                v = rnd.choice(ptrs)
+            elif ctype is ctypes.c_int64 or ctype is ctypes.c_size_t:
+                v = rnd.choice(strides)
+                if ctype is ctypes.c_size_t:
+                    v = abs(v)
+            elif ctype is ctypes.c_int32:
+                v = rnd.choice(ints)
+            else:
+                v = rnd.choice([-1.0, 0.0, 0.125, 0.5, 2.0])
+            setattr(obj, name, v)
+        return obj
+
+    def valid_sdpa():
+        a = _lib.SdpaArgs()
+        a.B, a.Hkv, a.D, a.kv_dtype = rnd.choice([1, 2]), rnd.choice([1, 2]), rnd.choice([64, 128]), rnd.choice([0, 1, 2])
+        a.Hq = a.Hkv * rnd.choice([1, 2, 4])
+        a.kv_len = rnd.choice([1, 63, 64, 1000, 70000])
+        a.q_len = rnd.choice([1, min(a.kv_len, 100)])
+        a.input_pos, a.sm_scale = a.kv_len - a.q_len, 0.125
+        for name, ctype in a._fields_:
+            if ctype is ctypes.c_void_p:
+                setattr(a, name, 0x10000)
+        a.q_stride_t = a.k_stride_t = a.v_stride_t = a.o_stride_h = a.D
+        a.q_stride_h, a.k_stride_h = a.q_len * a.D, a.kv_len * a.D
+        a.v_stride_h, a.o_stride_t = a.k_stride_h, a.Hq * a.D
+        a.q_stride_b, a.k_stride_b = a.Hq * a.q_stride_h, a.Hkv * a.k_stride_h
+        a.v_stride_b, a.o_stride_b = a.k_stride_b, a.q_len * a.o_stride_t
+        a.qs_stride_h = a.tp_stride_h = a.kv_len
+        a.qs_stride_b = a.tp_stride_b = a.Hkv * a.kv_len
+        a.workspace_bytes = 1 << 40
+        return a
+
+    def mutate(obj, times):
+        for _ in range(times):
+            name, ctype = rnd.choice(obj._fields_)
+            if ctype is ctypes.c_void_p:
+                setattr(obj, name, rnd.choice(ptrs))
+            elif ctype is ctypes.c_int64 or ctype is ctypes.c_size_t:
+                setattr(obj, name, abs(rnd.choice(strides)) if ctype is ctypes.c_size_t else rnd.choice(strides))
+            elif ctype is ctypes.c_int32:
+                setattr(obj, name, rnd.choice(ints))
+            else:
+                setattr(obj, name, rnd.choice([-1.0, 0.0, 0.125, 0.5, 2.0]))
+        return obj
+
+    for it in range(600):
+        # half of the blocks are random throughout, half are valid ones with up to two fields replaced
+        a = fill(_lib.SdpaArgs()) if it % 2 else mutate(valid_sdpa(), rnd.choice([0, 1, 1, 2]))
+        h = fill(_lib.H2OArgs())
+        for fn in (kvx.kvx_sdpa_prefill, kvx.kvx_score_sum, kvx.kvx_sdpa_decode):
+            assert fn(ctypes.byref(a), None) in codes
+        assert kvx.kvx_sdpa_decode_h2o(ctypes.byref(a), ctypes.byref(h), None) in codes
+        for fn in (kvx.kvx_sdpa_prefill_workspace_bytes, kvx.kvx_sdpa_decode_workspace_bytes, kvx.kvx_sdpa_decode_h2o_workspace_bytes):
+            assert fn(ctypes.byref(a)) >= 0
+        assert kvx.kvx_h2o_update_select(ctypes.byref(h), None) in codes
+        assert kvx.kvx_h2o_workspace_bytes(ctypes.byref(h)) >= 0
+        assert kvx.kvx_cache_write(ctypes.byref(fill(_lib.CacheWriteArgs())), None) in codes
+        q = fill(_lib.BlockQuantArgs())
+        assert kvx.kvx_quantize_blocks(ctypes.byref(q), None) in codes
+        assert kvx.kvx_dequantize_blocks(ctypes.byref(q), None) in codes
+        r = lambda: rnd.choice(ptrs)  # noqa: E731
+        n, d, st = rnd.choice(ints), rnd.choice(ints), rnd.choice(strides)
+        assert kvx.kvx_quantize_rows(r(), st, n, d, r(), r(), r(), None) in codes
+        assert kvx.kvx_dequantize_rows(r(), r(), r(), n, d, r(), st, None) in codes
+        assert kvx.kvx_quantize_rows4(r(), st, n, d, r(), r(), r(), None) in codes
+        assert kvx.kvx_dequantize_rows4(r(), r(), r(), n, d, r(), st, None) in codes
+        assert kvx.kvx_rmsnorm_rows(r(), st, r(), st, r(), n, d, 1e-6, None) in codes
+        assert kvx.kvx_add_rmsnorm_rows(r(), st, r(), st, r(), st, r(), st, r(), n, d, 1e-6, None) in codes
+        assert kvx.kvx_swiglu_rows(r(), st, r(), st, n, d, None) in codes
+        assert kvx.kvx_qk_norm_rope(r(), st, st, rnd.choice(ints), n, rnd.choice(ints), rnd.choice(ints), d, r(), r(), 1e-6, r(), r(),
+                                    rnd.choice(ints), rnd.choice(ints), None) in codes
+
+
 def test_no_cpu_fallback():
     q = torch.zeros(1, 4, 2, 64, dtype=torch.bfloat16)
     k = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
