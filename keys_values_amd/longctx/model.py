@@ -123,6 +123,7 @@ class LongContextPrefillModel:
     def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
         """Process whole sequences chunk by chunk; returns the hidden states of the last chunk."""
         self.reset()
+        input_ids = input_ids.to(self.device)  # one copy: a copy per chunk from pageable memory would drain the stream every chunk
         out = None
         start = 0
         for n in self.chunk_sizes(input_ids.shape[1]):
