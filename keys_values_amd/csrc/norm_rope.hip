@@ -25,21 +25,41 @@ __device__ __forceinline__ float wave_sum(float x) {
   return x;
 }
 
-// One wavefront per row; a lane holds up to MAXC chunks of 8 elements (dim <= 64 * 8 * MAXC).
-template <int MAXC>
+// Sum over the WPR wavefronts that share a row (WPR = 1: the wavefront's own sum; WPR = NT / 64: the
+// whole workgroup, through LDS, added in wavefront order).
+template <int WPR>
+__device__ __forceinline__ float row_total(float ss) {
+  ss = wave_sum(ss);
+  if constexpr (WPR > 1) {
+    static_assert(WPR == NT / 64, "a row is one wavefront or the whole workgroup");
+    __shared__ float part[WPR];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = part[0];
+#pragma unroll
+    for (int i = 1; i < WPR; ++i) ss += part[i];
+  }
+  return ss;
+}
+
+// WPR wavefronts per row; a lane holds up to MAXC chunks of 8 elements (dim <= 64 * WPR * 8 * MAXC).
+// Few long rows (a 1024-token chunk of hidden states) take the whole workgroup per row: four times the
+// loads in flight per row, and enough workgroups to cover the chip.
+template <int MAXC, int WPR>
 __global__ __launch_bounds__(NT) void rmsnorm_rows_kernel(const uint16_t* __restrict__ x, int64_t x_rs, uint16_t* __restrict__ out,
                                                           int64_t o_rs, const float* __restrict__ weight, int64_t rows, int dim,
                                                           float eps, float factor) {
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  constexpr int TPR = 64 * WPR;  // threads per row
+  const int lane = threadIdx.x % TPR;
+  const int64_t row = (int64_t)blockIdx.x * (NT / TPR) + threadIdx.x / TPR;
+  if (row >= rows) return;  // uniform over the threads of a row (and over the workgroup when WPR > 1)
   const int nchunks = dim / 8;
   const uint16_t* xr = x + row * x_rs;
   u32x4_t v[MAXC];
   float ss = 0.0f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
-    const int ch = lane + 64 * c;
+    const int ch = lane + TPR * c;
     v[c] = u32x4_t{0, 0, 0, 0};
     if (ch < nchunks) v[c] = *(const u32x4_t*)(xr + ch * 8);
 #pragma unroll
@@ -49,12 +69,12 @@ __global__ __launch_bounds__(NT) void rmsnorm_rows_kernel(const uint16_t* __rest
       ss += b * b;
     }
   }
-  ss = wave_sum(ss);
+  ss = row_total<WPR>(ss);
   const float denom = sqrtf(ss) * factor + eps;
   uint16_t* orow = out + row * o_rs;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
-    const int ch = lane + 64 * c;
+    const int ch = lane + TPR * c;
     if (ch >= nchunks) break;
     const f32x4_t w0 = *(const f32x4_t*)(weight + ch * 8);
     const f32x4_t w1 = *(const f32x4_t*)(weight + ch * 8 + 4);
@@ -73,20 +93,21 @@ __global__ __launch_bounds__(NT) void rmsnorm_rows_kernel(const uint16_t* __rest
 // the normalisation that follows it (keys_values/model.py:560-584: x = attention_output + x, then
 // norm_2(x); x = mlp_output + x, then the next block's norm_1). The sum is rounded to bf16 before it is
 // normalised, as the two separate steps do. In place is allowed (x_out == x).
-template <int MAXC>
+template <int MAXC, int WPR>
 __global__ __launch_bounds__(NT) void add_rmsnorm_rows_kernel(const uint16_t* x, int64_t x_rs, const uint16_t* __restrict__ delta,
                                                               int64_t d_rs, uint16_t* x_out, int64_t xo_rs,
                                                               uint16_t* __restrict__ out, int64_t o_rs, const float* __restrict__ weight,
                                                               int64_t rows, int dim, float eps, float factor) {
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+  constexpr int TPR = 64 * WPR;
+  const int lane = threadIdx.x % TPR;
+  const int64_t row = (int64_t)blockIdx.x * (NT / TPR) + threadIdx.x / TPR;
   if (row >= rows) return;
   const int nchunks = dim / 8;
   u32x4_t v[MAXC];
   float ss = 0.0f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
-    const int ch = lane + 64 * c;
+    const int ch = lane + TPR * c;
     v[c] = u32x4_t{0, 0, 0, 0};
     if (ch < nchunks) {
       const u32x4_t a = *(const u32x4_t*)(x + row * x_rs + ch * 8);
@@ -102,12 +123,12 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_rows_kernel(const uint16_t* x,
       ss += b * b;
     }
   }
-  ss = wave_sum(ss);
+  ss = row_total<WPR>(ss);
   const float denom = sqrtf(ss) * factor + eps;
   uint16_t* orow = out + row * o_rs;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
-    const int ch = lane + 64 * c;
+    const int ch = lane + TPR * c;
     if (ch >= nchunks) break;
     const f32x4_t w0 = *(const f32x4_t*)(weight + ch * 8);
     const f32x4_t w1 = *(const f32x4_t*)(weight + ch * 8 + 4);
@@ -210,6 +231,9 @@ __global__ __launch_bounds__(NT) void qk_norm_rope_kernel(uint16_t* __restrict__
   if (live) *(u32x4_t*)p = o;
 }
 
+// Rows of at least 2048 values, too few of them to fill the chip with a wavefront each.
+bool workgroup_per_row(int64_t rows, int dim) { return dim >= 2048 && dim <= NT * 8 * 4 && rows <= 16384; }
+
 }  // namespace
 
 int launch_rmsnorm_rows(const void* x, int64_t x_rs, void* out, int64_t o_rs, const float* weight, int64_t rows, int dim, float eps,
@@ -218,11 +242,14 @@ int launch_rmsnorm_rows(const void* x, int64_t x_rs, void* out, int64_t o_rs, co
   const float factor = 1.0f / sqrtf((float)dim);
   const unsigned grid = (unsigned)((rows + NT / 64 - 1) / (NT / 64));
   const int chunks_per_lane = (dim / 8 + 63) / 64;
-  if (chunks_per_lane <= 4)
-    hipLaunchKernelGGL(rmsnorm_rows_kernel<4>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs, weight, rows,
+  if (workgroup_per_row(rows, dim))
+    hipLaunchKernelGGL((rmsnorm_rows_kernel<4, NT / 64>), dim3((unsigned)rows), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs,
+                       weight, rows, dim, eps, factor);
+  else if (chunks_per_lane <= 4)
+    hipLaunchKernelGGL((rmsnorm_rows_kernel<4, 1>), dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs, weight, rows,
                        dim, eps, factor);
   else
-    hipLaunchKernelGGL(rmsnorm_rows_kernel<16>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs, weight, rows,
+    hipLaunchKernelGGL((rmsnorm_rows_kernel<16, 1>), dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (uint16_t*)out, o_rs, weight, rows,
                        dim, eps, factor);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
@@ -233,11 +260,14 @@ int launch_add_rmsnorm_rows(const void* x, int64_t x_rs, const void* delta, int6
   if (rows == 0) return KVX_OK;
   const float factor = 1.0f / sqrtf((float)dim);
   const unsigned grid = (unsigned)((rows + NT / 64 - 1) / (NT / 64));
-  if ((dim / 8 + 63) / 64 <= 4)
-    hipLaunchKernelGGL(add_rmsnorm_rows_kernel<4>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
+  if (workgroup_per_row(rows, dim))
+    hipLaunchKernelGGL((add_rmsnorm_rows_kernel<4, NT / 64>), dim3((unsigned)rows), dim3(NT), 0, st, (const uint16_t*)x, x_rs,
+                       (const uint16_t*)delta, d_rs, (uint16_t*)x_out, xo_rs, (uint16_t*)out, o_rs, weight, rows, dim, eps, factor);
+  else if ((dim / 8 + 63) / 64 <= 4)
+    hipLaunchKernelGGL((add_rmsnorm_rows_kernel<4, 1>), dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
                        (uint16_t*)x_out, xo_rs, (uint16_t*)out, o_rs, weight, rows, dim, eps, factor);
   else
-    hipLaunchKernelGGL(add_rmsnorm_rows_kernel<16>, dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
+    hipLaunchKernelGGL((add_rmsnorm_rows_kernel<16, 1>), dim3(grid), dim3(NT), 0, st, (const uint16_t*)x, x_rs, (const uint16_t*)delta, d_rs,
                        (uint16_t*)x_out, xo_rs, (uint16_t*)out, o_rs, weight, rows, dim, eps, factor);
   KVX_HIP(hipGetLastError());
   return KVX_OK;

@@ -94,7 +94,7 @@ def test_rope_oracle_invariants():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("rows,dim", [(5, 64), (1024, 2560), (3, 8192), (17, 200)])
+@pytest.mark.parametrize("rows,dim", [(5, 64), (1024, 2560), (3, 8192), (17, 200), (7, 2048), (100, 4104), (20000, 2048)])
 def test_rmsnorm_kernel(gpu, rows, dim):
     from keys_values_amd.longctx import ops
 
@@ -109,7 +109,7 @@ def test_rmsnorm_kernel(gpu, rows, dim):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("rows,dim", [(5, 64), (1024, 2560), (3, 8192), (17, 200)])
+@pytest.mark.parametrize("rows,dim", [(5, 64), (1024, 2560), (3, 8192), (17, 200), (7, 2048), (100, 4104), (20000, 2048)])
 def test_add_rmsnorm_kernel(gpu, rows, dim):
     # x = x + delta (rounded to bf16), then RMSNorm(x): the two separate steps of the oracle
     from keys_values_amd.longctx import ops
