@@ -154,13 +154,14 @@ class H2OKVCache:
         b, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
         kv_dtype = torch.uint8 if quantized else torch.bfloat16
         row = d // 2 if (quantized and num_bits == 4) else d  # the 4-bit store packs two codes per byte
-        self.k = torch.zeros((b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
-        self.v = torch.zeros((b, h, length, row), dtype=kv_dtype, device=self.device)
+        # K and V (and their row states) are the two halves of one allocation each: one launch can walk both
+        self._kv = torch.zeros((2, b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
+        self.k, self.v = self._kv[0], self._kv[1]
         if quantized:
-            self.k_scale = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)
-            self.k_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
-            self.v_scale = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)
-            self.v_zp = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)
+            self._kv_scale = torch.zeros((2, b, h, length), dtype=torch.float32, device=self.device)
+            self._kv_zp = torch.zeros((2, b, h, length), dtype=torch.int32, device=self.device)
+            self.k_scale, self.v_scale = self._kv_scale[0], self._kv_scale[1]
+            self.k_zp, self.v_zp = self._kv_zp[0], self._kv_zp[1]
         self.token_pos = torch.zeros((b, h, length), dtype=torch.int32, device=self.device)  # attn_weights.py:466-470
         self.scores = torch.zeros((b, h, length), dtype=torch.float32, device=self.device)  # h2o.py:85-91
         # further score buffers, moved and initialised with the slots (h2o.py:405-413, qh2o.py:107-113)
@@ -343,8 +344,11 @@ class H2OKVCache:
         fn = lib.kvx_dequantize_rows4 if self.num_bits == 4 else lib.kvx_dequantize_rows
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
-            _lib.check(fn(self.k.data_ptr(), self.k_scale.data_ptr(), self.k_zp.data_ptr(), rows, d, kd.data_ptr(), d, stream))
-            _lib.check(fn(self.v.data_ptr(), self.v_scale.data_ptr(), self.v_zp.data_ptr(), rows, d, vd.data_ptr(), d, stream))
+            if b == self.max_batch_size:  # K and V are adjacent in the store and in the scratch: one launch
+                _lib.check(fn(self._kv.data_ptr(), self._kv_scale.data_ptr(), self._kv_zp.data_ptr(), 2 * rows, d, kd.data_ptr(), d, stream))
+            else:
+                _lib.check(fn(self.k.data_ptr(), self.k_scale.data_ptr(), self.k_zp.data_ptr(), rows, d, kd.data_ptr(), d, stream))
+                _lib.check(fn(self.v.data_ptr(), self.v_scale.data_ptr(), self.v_zp.data_ptr(), rows, d, vd.data_ptr(), d, stream))
         return kd.view(b, h, length, d)[:, :, :T], vd.view(b, h, length, d)[:, :, :T]
 
     def _prefill_step(self, query, key, value):
