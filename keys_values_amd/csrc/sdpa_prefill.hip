@@ -503,12 +503,17 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
       // followed by the two LDS reads of the next one and by its share of the softmax arithmetic,
       // so the vector ALU works in the shadow of the matrix core instead of after it
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // operands of the first two go out ahead
+      constexpr int NREST = 4 * DT - NPRE;
+      constexpr int NV = (80 + NREST - 1) / NREST;  // VALU per matrix instruction: 80 per tile (fma, add, cvt)
+      constexpr int NX = (32 + NREST - 1) / NREST;  // transcendental: 32 exp2 per tile
 #pragma unroll
-      for (int i = 0; i < 4 * DT - NPRE; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 LDS reads
-        __builtin_amdgcn_sched_group_barrier(0x002, (80 + 4 * DT - NPRE - 1) / (4 * DT - NPRE), 0);  // VALU: 80 per tile (fma, add, cvt)
-        __builtin_amdgcn_sched_group_barrier(0x400, (32 + 4 * DT - NPRE - 1) / (4 * DT - NPRE), 0);  // transcendental: 32 exp2 per tile
+      for (int i = 0; i < NREST; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // 1 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, (NV + 1) / 2, 0);  // half of its vector work,
+        __builtin_amdgcn_sched_group_barrier(0x400, (NX + 1) / 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);             // the 2 LDS reads of the next one,
+        __builtin_amdgcn_sched_group_barrier(0x002, NV / 2, 0);        // the other half
+        __builtin_amdgcn_sched_group_barrier(0x400, NX / 2, 0);
       }
       // keep the softmax arithmetic in this block: without a use here the optimiser sinks it
       // past the barrier below, out of the matrix core's shadow
