@@ -397,16 +397,21 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
   // mask (only tiles that hold a position some row of this wavefront may not see)
   auto mask = [&](f32x16_t (&s)[2], int buf) {
     const int tpl = sm.tp[buf][lane];
-    if (__any(tpl > qpos_min_w)) {
+    // bit k: key k of the tile holds a position some row of this wavefront may not see. In a cache with
+    // scattered slots nearly every tile has a few such keys: only their groups of 8 keys are masked.
+    const unsigned long long hidden = __ballot(tpl > qpos_min_w);
+    if (hidden) {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-          const int4 tq = *(const int4*)&sm.tp[buf][mt * 32 + 8 * a + 4 * h];
-          if (tq.x > qpos) s[mt][4 * a + 0] = -INFINITY;
-          if (tq.y > qpos) s[mt][4 * a + 1] = -INFINITY;
-          if (tq.z > qpos) s[mt][4 * a + 2] = -INFINITY;
-          if (tq.w > qpos) s[mt][4 * a + 3] = -INFINITY;
+          if ((hidden >> (mt * 32 + 8 * a)) & 0xffull) {
+            const int4 tq = *(const int4*)&sm.tp[buf][mt * 32 + 8 * a + 4 * h];
+            if (tq.x > qpos) s[mt][4 * a + 0] = -INFINITY;
+            if (tq.y > qpos) s[mt][4 * a + 1] = -INFINITY;
+            if (tq.z > qpos) s[mt][4 * a + 2] = -INFINITY;
+            if (tq.w > qpos) s[mt][4 * a + 3] = -INFINITY;
+          }
         }
     }
   };
