@@ -240,7 +240,7 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   uint32_t* keys = (uint32_t*)(dyn_lds + (size_t)kpad * 8);   // a.limit entries (CACHED only)
   __shared__ uint32_t hist[256];
   __shared__ uint32_t wave_cnt[SEL_THREADS / 64];
-  __shared__ uint32_t sh_prefix, sh_krem, sh_nless, sh_diff;
+  __shared__ uint32_t sh_prefix, sh_krem, sh_diff;
   __shared__ int sh_hi;
 
   const int tid = threadIdx.x;
@@ -286,7 +286,6 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   if (tid == 0) {
     sh_prefix = 0;
     sh_krem = (uint32_t)a.k;
-    sh_nless = 0;
     sh_diff = 0;
   }
   __syncthreads();
@@ -309,6 +308,7 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
     }
     __syncthreads();
   }
+  constexpr int RB = 8;
   // radix select over the remaining bits, 8 at a time from the top: after a pass sh_prefix holds the
   // bits [lo, 32) of the k-th smallest key and sh_krem its rank among the keys sharing them.
   for (int hi = sh_hi; hi > 0;) {
@@ -318,9 +318,18 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
     const uint32_t prefix = sh_prefix;
     const uint32_t himask = hi >= 32 ? 0u : (0xffffffffu << hi);
     const uint32_t dmask = (1u << (hi - lo)) - 1u;
-    for (int i = tid; i < a.limit; i += SEL_THREADS) {
-      const uint32_t u = key_of(i);
-      if ((u & himask) == prefix) atomicAdd(&hist[(u >> lo) & dmask], 1u);
+    // keys are fetched eight at a time: a loop of one dependent LDS read per counter update would run at
+    // the latency of that read
+    for (int i0 = tid; i0 < a.limit; i0 += RB * SEL_THREADS) {
+      uint32_t u[RB];
+#pragma unroll
+      for (int j = 0; j < RB; ++j) {
+        const int i = i0 + j * SEL_THREADS;
+        u[j] = i < a.limit ? key_of(i) : ~prefix;  // a key that cannot match the prefix
+      }
+#pragma unroll
+      for (int j = 0; j < RB; ++j)
+        if (i0 + j * SEL_THREADS < a.limit && (u[j] & himask) == prefix) atomicAdd(&hist[(u[j] >> lo) & dmask], 1u);
     }
     __syncthreads();
     if (tid < 64) {
@@ -356,39 +365,56 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   const uint32_t need_eq = sh_krem;   // how many slots equal to it are taken (lowest slots first)
   const uint32_t nless = (uint32_t)a.k - need_eq;
 
-  // gather: slots below ustar in any order; slots equal to it by ascending slot. Every wavefront
-  // owns a contiguous stretch of the row, so slot order is (wavefront, step, lane) order and the
-  // ties need two barriers in all: count per wavefront, prefix, place.
+  // gather: slots below ustar, then slots equal to it by ascending slot. Every wavefront owns a
+  // contiguous stretch of the row, so slot order is (wavefront, step, lane) order: one sweep counts
+  // both kinds per wavefront, a prefix over the wavefronts gives each its places, a second sweep writes
+  // them (no atomics, nothing a step has to wait for).
   const int lane = tid & 63, wave = tid >> 6;
   constexpr int NWV = SEL_THREADS / 64;
+  __shared__ uint32_t wave_less[NWV];
   const int chunk = ((a.limit + NWV - 1) / NWV + 63) / 64 * 64;
   const int c_begin = wave * chunk, c_end = min(c_begin + chunk, a.limit);
-  uint32_t my_eq = 0;
-  for (int i0 = c_begin; i0 < c_end; i0 += 64) {
-    const int i = i0 + lane;
-    const uint32_t u = i < c_end ? key_of(i) : 0xffffffffu;
-    const bool less = i < c_end && u < ustar;
-    const unsigned long long lm = __ballot(less);
-    if (lm) {
-      uint32_t base = 0;
-      if (lane == 0) base = atomicAdd(&sh_nless, (uint32_t)__popcll(lm));
-      base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
-      if (less) cand[base + (uint32_t)__popcll(lm & ((1ull << lane) - 1ull))] = ((unsigned long long)u << 32) | (unsigned)i;
+  uint32_t my_less = 0, my_eq = 0;
+  for (int i0 = c_begin; i0 < c_end; i0 += 64 * RB) {
+    uint32_t u[RB];
+#pragma unroll
+    for (int j = 0; j < RB; ++j) {
+      const int i = i0 + 64 * j + lane;
+      u[j] = i < c_end ? key_of(i) : 0xffffffffu;
     }
-    my_eq += (uint32_t)__popcll(__ballot(i < c_end && u == ustar));
+#pragma unroll
+    for (int j = 0; j < RB; ++j) {
+      const bool in = i0 + 64 * j + lane < c_end;
+      my_less += (uint32_t)__popcll(__ballot(in && u[j] < ustar));
+      my_eq += (uint32_t)__popcll(__ballot(in && u[j] == ustar));
+    }
   }
-  if (lane == 0) wave_cnt[wave] = my_eq;
+  if (lane == 0) {
+    wave_less[wave] = my_less;
+    wave_cnt[wave] = my_eq;
+  }
   __syncthreads();
-  uint32_t rank = 0;  // ties in the wavefronts before this one
-  for (int ww = 0; ww < wave; ++ww) rank += wave_cnt[ww];
-  if (rank < need_eq && my_eq) {
+  uint32_t pos_less = 0, rank = 0;  // places taken by the wavefronts before this one
+  for (int ww = 0; ww < wave; ++ww) {
+    pos_less += wave_less[ww];
+    rank += wave_cnt[ww];
+  }
+  const bool place_eq = rank < need_eq && my_eq;
+  if (my_less || place_eq) {
     for (int i0 = c_begin; i0 < c_end; i0 += 64) {
       const int i = i0 + lane;
-      const bool eq = i < c_end && key_of(i) == ustar;
-      const unsigned long long eqm = __ballot(eq);
-      const uint32_t r = rank + (uint32_t)__popcll(eqm & ((1ull << lane) - 1ull));
-      if (eq && r < need_eq) cand[nless + r] = ((unsigned long long)ustar << 32) | (unsigned)i;
-      rank += (uint32_t)__popcll(eqm);
+      const uint32_t u = i < c_end ? key_of(i) : 0xffffffffu;
+      const bool less = i < c_end && u < ustar;
+      const unsigned long long lm = __ballot(less);
+      if (less) cand[pos_less + (uint32_t)__popcll(lm & ((1ull << lane) - 1ull))] = ((unsigned long long)u << 32) | (unsigned)i;
+      pos_less += (uint32_t)__popcll(lm);
+      if (place_eq) {
+        const bool eq = i < c_end && u == ustar;
+        const unsigned long long eqm = __ballot(eq);
+        const uint32_t r = rank + (uint32_t)__popcll(eqm & ((1ull << lane) - 1ull));
+        if (eq && r < need_eq) cand[nless + r] = ((unsigned long long)ustar << 32) | (unsigned)i;
+        rank += (uint32_t)__popcll(eqm);
+      }
     }
   }
   __syncthreads();
