@@ -157,6 +157,35 @@ def bench_prefill(args, torch, dev):
     rows = w.sum(-1).cpu()
     assert torch.allclose(rows, torch.full_like(rows, float(q_len)), rtol=1e-4, atol=5e-2), rows
 
+    # A quantised store, long chunk: what the cache object does instead of dequantising inside the attention
+    # kernels (where every workgroup of 256 rows dequantises the whole store again) is one dequantisation
+    # of the store into a bf16 copy for the attention kernel (the score-sum kernel dequantises each key once
+    # per wavefront anyway and stays on the codes). Timed here on the same inputs.
+    dq_ms = None
+    if u8:
+        from keys_values_amd.kvcache.h2o import _dequant_scratch
+
+        kd, vd = (t.view(B, Hkv, T, D) for t in _dequant_scratch(dev, B * Hkv * T * D))  # the cache object's own buffer
+        dq = lib.kvx_dequantize_rows4 if u4 else lib.kvx_dequantize_rows
+
+        def step_copy():
+            _lib.check(dq(k.data_ptr(), ksc.data_ptr(), kzp.data_ptr(), B * Hkv * T, D, kd.data_ptr(), D, st))
+            _lib.check(dq(v.data_ptr(), vsc.data_ptr(), vzp.data_ptr(), B * Hkv * T, D, vd.data_ptr(), D, st))
+            _, _, lse_c = ops.prefill_core(q, kd, vd, scale, input_pos, None, return_lse=True)
+            return ops.score_sum_core(q, k, lse_c, scale, input_pos, None, quant=quant)  # the score-sum pass keeps the codes
+
+        for _ in range(3):
+            w_copy = step_copy()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(w_copy, w, rtol=1e-3, atol=1e-6)
+        d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        d0.record()
+        for _ in range(10):
+            step_copy()
+        d1.record()
+        torch.cuda.synchronize()
+        dq_ms = d0.elapsed_time(d1) / 10
+
     # The same chunk through the cache object (keys_values/kvcache/base.py:554-595): write the 1024 new
     # rows into the slots chosen by the step before, attend, score-sum, scores += W, choose the next
     # 1024 lowest-score slots. Steady state: after the first step the positions are scattered.
@@ -231,6 +260,7 @@ def bench_prefill(args, torch, dev):
             "ms_attention_kernel": round(ms_attn, 4),
             "ms_score_sum_kernel": round(ms_score, 4),
             "score_sum_tflops": round(2.0 * B * Hq * q_len * T * D / (ms_score * 1e-3) / 1e12, 2),
+            "ms_step_over_dequantised_copy": None if dq_ms is None else round(dq_ms, 4),
             "h2o_cache_chunk_ms": None if h2o_ms is None else round(h2o_ms, 4),
             "h2o_cache_chunk_tokens_per_s": None if h2o_ms is None else round(q_len / (h2o_ms * 1e-3), 1),
         },

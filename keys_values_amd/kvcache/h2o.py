@@ -325,10 +325,14 @@ class H2OKVCache:
         else:
             rows = num * (hq // self.n_query_groups)
             if quant is not None and self.dequantize_chunk_rows is not None and rows >= self.dequantize_chunk_rows:
-                kc, vc = self._dequantized(b, T)
-                quant = None
-            out, w, _ = ops.prefill_core(query, kc, vc, self.scale_factor, input_pos, tp, return_weights=True,
-                                         output_transposed=True, quant=quant)
+                # attention over the bf16 copy; the score-sum pass keeps the codes (it dequantises each key
+                # once per wavefront whatever the chunk length, and reads half the bytes)
+                kd, vd = self._dequantized(b, T)
+                out, _, lse = ops.prefill_core(query, kd, vd, self.scale_factor, input_pos, tp, return_lse=True, output_transposed=True)
+                w = ops.score_sum_core(query, kc, lse, self.scale_factor, input_pos, tp, quant=quant)
+            else:
+                out, w, _ = ops.prefill_core(query, kc, vc, self.scale_factor, input_pos, tp, return_weights=True,
+                                             output_transposed=True, quant=quant)
         self._update(w, num)
         return out.reshape(b, num, hq * d)
 
