@@ -255,6 +255,18 @@ struct Loader {
     issue_tp<IS_K>(sm, tile, buf);
   }
 
+  // a full tile, not the last one of the walk: no bounds to check (bf16 tiles only)
+  template <bool IS_K, int BUF>
+  __device__ __forceinline__ void issue_steady(Smem<D>& sm, int tile) {
+    static_assert(!U8, "codes go through registers");
+    issue_full<IS_K, BUF>(tile);
+    if (IS_K && tp && wave == 0)
+      dma4((const char*)(tp + tile * BN), (uint32_t)lane * 4, __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.tp[BUF][0])));
+  }
+  __device__ __forceinline__ void land_steady(Smem<D>& sm, int tile, int buf, int tid) {
+    if (!tp && tid < BN) sm.tp[buf][tid] = tile * BN + tid;
+  }
+
   // token positions of the K tile: one 4-byte DMA per lane of wavefront 0 (slots past the end
   // re-read the last valid one and are overwritten with INT_MAX when the tile lands)
   template <bool IS_K>
@@ -457,14 +469,21 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
   // one pipeline step; the first one has no previous tile to multiply
   // one pipeline step on the tile in buffer CUR (compile time: LDS offsets become immediates and P
   // alternates between two register sets instead of being copied)
-  auto step = [&](auto first_tag, auto cur_tag, int t) {
+  auto step = [&](auto first_tag, auto cur_tag, auto steady_tag, int t) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr int cur = decltype(cur_tag)::value;
+    // STEADY: tiles t and t + 1 are full and tile t + 1 belongs to this walk
+    constexpr bool STEADY = decltype(steady_tag)::value && KV == KVX_KV_BF16;
     uint32_t (&pb_prev)[2][8] = pbs[cur ^ 1];
     uint32_t (&pb)[2][8] = pbs[cur];
-    const bool has1 = t + 1 < tile_end;
-    ld.template issue_one<false>(sm, t, cur, tid);
-    if (has1) ld.template issue_one<true>(sm, t + 1, cur ^ 1, tid);
+    const bool has1 = STEADY || t + 1 < tile_end;
+    if constexpr (STEADY) {
+      ld.template issue_steady<false, cur>(sm, t);
+      ld.template issue_steady<true, cur ^ 1>(sm, t + 1);
+    } else {
+      ld.template issue_one<false>(sm, t, cur, tid);
+      if (has1) ld.template issue_one<true>(sm, t + 1, cur ^ 1, tid);
+    }
     f32x16_t s[2];
     qk(s, cur);
     if constexpr (!FIRST) {
@@ -536,20 +555,32 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     }
     // ---- publish the tiles that were in flight -------------------------------------------------
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's DMA / loads have landed
-    ld.template land<false>(sm, t, cur, tid);
-    if (has1) ld.template land<true>(sm, t + 1, cur ^ 1, tid);
+    if constexpr (STEADY) {
+      ld.land_steady(sm, t + 1, cur ^ 1, tid);
+    } else {
+      ld.template land<false>(sm, t, cur, tid);
+      if (has1) ld.template land<true>(sm, t + 1, cur ^ 1, tid);
+    }
     __syncthreads();
   };
   constexpr std::integral_constant<int, 0> B0{};
   constexpr std::integral_constant<int, 1> B1{};
-  step(std::true_type{}, B0, tile_begin);
+  constexpr std::true_type YES{};
+  constexpr std::false_type NO{};
+  step(YES, B0, NO, tile_begin);
   int t = tile_begin + 1;
+  // tiles whose successor is a full tile of this walk take the step without bounds checks
+  const int steady_end = min(tile_end - 1, p.kv_len / BN - 1);  // t < steady_end: tiles t, t + 1 full, t + 1 < tile_end
+  for (; t + 1 < steady_end; t += 2) {
+    step(NO, B1, YES, t);
+    step(NO, B0, YES, t + 1);
+  }
   for (; t + 1 < tile_end; t += 2) {
-    step(std::false_type{}, B1, t);
-    step(std::false_type{}, B0, t + 1);
+    step(NO, B1, NO, t);
+    step(NO, B0, NO, t + 1);
   }
   if (t < tile_end) {
-    step(std::false_type{}, B1, t);
+    step(NO, B1, NO, t);
     pv(pbs[1], 1);
   } else {
     pv(pbs[0], 0);
