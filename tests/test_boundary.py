@@ -215,6 +215,17 @@ def test_hip_sdpa_keeps_reference_errors():
         s.scaled_dot_product_attention(q[:, :, :1], k[:, :, :1], k[:, :, :1], None, 6, None)
 
 
+def test_bench_refuses_more_than_one_gpu_and_runs_nothing_without_one():
+    import sys
+
+    bench = os.path.join(ROOT, "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+    if not torch.cuda.is_available():  # no device: it must say so, not fall back to the CPU
+        r = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True)
+        assert r.returncode != 0 and "no CPU fallback" in r.stderr and r.stdout.strip() == ""
+
+
 def test_c_oracle_builds():
     from oracle import c_oracle
 
