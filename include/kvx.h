@@ -321,6 +321,20 @@ typedef struct kvx_h2o_args {
 int kvx_h2o_update_select(const kvx_h2o_args* args, void* stream);
 size_t kvx_h2o_workspace_bytes(const kvx_h2o_args* args);
 
+/* kvx_h2o_update_select for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+ * arguments, same kernels, same results; args->workspace and args->workspace_bytes are ignored: the
+ * scratch (the per-row minimum keys of k == 1, the per-row statistics of the q_errors combination)
+ * lives in a device array of KVX_H2O_STATIC_SCRATCH_BYTES that is part of the library image, one copy
+ * per GPU, held until the process ends. Calls whose kvx_h2o_workspace_bytes() exceeds that size return
+ * KVX_ERR_WORKSPACE. The call allocates nothing and frees nothing; the first call on a device looks
+ * the array's device address up (do that call outside a graph capture). All calls on one GPU share
+ * the array: two calls that overlap on one GPU (different streams, no ordering between them) race;
+ * calls on one stream, or ordered by events, do not. What the kernels need cleared they clear
+ * themselves with a fill kernel, so the array's previous contents never matter. */
+#define KVX_H2O_STATIC_SCRATCH_BYTES (128 * 1024)
+int kvx_h2o_update_select_static(const kvx_h2o_args* args, void* stream);
+
 /* ---- callers of the path: normalisation and rotary encoding of the new tokens ---------------- */
 
 /* RMS normalisation of `rows` rows of `dim` bf16 values: out = (x / (|x|_2 / sqrt(dim) + eps)) * weight,

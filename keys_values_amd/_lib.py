@@ -101,6 +101,7 @@ SYMBOLS = {
     "kvx_cache_write": (ctypes.c_int, [POINTER(CacheWriteArgs), c_void_p]),
     "kvx_h2o_update_select": (ctypes.c_int, [POINTER(H2OArgs), c_void_p]),
     "kvx_h2o_workspace_bytes": (c_size_t, [POINTER(H2OArgs)]),
+    "kvx_h2o_update_select_static": (ctypes.c_int, [POINTER(H2OArgs), c_void_p]),
     "kvx_rmsnorm_rows": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int32, ctypes.c_float, c_void_p]),
     "kvx_add_rmsnorm_rows": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                             c_int32, ctypes.c_float, c_void_p]),

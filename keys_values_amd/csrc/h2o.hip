@@ -13,6 +13,8 @@
 //          re-read from global memory). A 4-pass 8-bit radix select finds the k-th smallest value;
 //          elements below it, plus the lowest-slot elements equal to it, are gathered and
 //          bitonic-sorted as 64-bit (value, slot) keys.
+#include <mutex>
+
 #include "kvx_common.h"
 
 namespace kvx {
@@ -488,6 +490,50 @@ int launch_h2o_update_select(const kvx_h2o_args& a_in, hipStream_t st) {
   }
   KVX_HIP(hipGetLastError());
   return KVX_OK;
+}
+
+// ---- the same call for callers that cannot allocate -------------------------------------------
+//
+// The workspace of the selection (the per-row 64-bit minimum keys of k == 1, the per-row statistics of
+// the Q-Hitter combination) lives in a file-scope device array instead of caller memory. `scratch`
+// is only a host-side stand-in for that array: its device address is looked up once per device with
+// hipGetSymbolAddress (every device holds its own copy at its own address) and only that address is
+// handed to kernels.
+constexpr size_t kStaticScratchBytes = 128 * 1024;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+size_t h2o_static_scratch_bytes() { return kStaticScratchBytes; }
+
+static int static_scratch_ptr(void** out) {
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = 0;
+  KVX_HIP(hipGetDevice(&dev));
+  KVX_REQUIRE(dev >= 0 && dev < kMaxDevices, KVX_ERR_UNSUPPORTED, "kvx_h2o_update_select_static: device %d beyond the %d this library keeps scratch for", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    KVX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    KVX_REQUIRE(p != nullptr, KVX_ERR_HIP, "kvx_h2o_update_select_static: no device address for the static scratch on device %d", dev);
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return KVX_OK;
+}
+
+int launch_h2o_update_select_static(const kvx_h2o_args& a_in, hipStream_t st) {
+  kvx_h2o_args a = a_in;
+  const size_t need = h2o_workspace(a);
+  KVX_REQUIRE(need <= kStaticScratchBytes, KVX_ERR_WORKSPACE,
+              "kvx_h2o_update_select_static: B * Hkv = %d rows need %zu bytes of scratch, the static array holds %zu", a.B * a.Hkv, need,
+              kStaticScratchBytes);
+  void* p = nullptr;
+  const int rc = static_scratch_ptr(&p);
+  if (rc != KVX_OK) return rc;
+  a.workspace = p;
+  a.workspace_bytes = kStaticScratchBytes;
+  return launch_h2o_update_select(a, st);
 }
 
 }  // namespace kvx

@@ -289,6 +289,12 @@ int kvx_h2o_update_select(const kvx_h2o_args* a, void* stream) {
   return launch_h2o_update_select(*a, (hipStream_t)stream);
 }
 
+int kvx_h2o_update_select_static(const kvx_h2o_args* a, void* stream) {
+  int rc = check_h2o(a, "kvx_h2o_update_select_static");
+  if (rc != KVX_OK) return rc;
+  return launch_h2o_update_select_static(*a, (hipStream_t)stream);
+}
+
 int kvx_sdpa_decode_h2o(const kvx_sdpa_args* a, const kvx_h2o_args* h, void* stream) {
   int rc = check_sdpa_common(a, "kvx_sdpa_decode_h2o", true);
   if (rc != KVX_OK) return rc;

@@ -55,6 +55,8 @@ int launch_dequantize_blocks(const kvx_block_quant_args& a, hipStream_t st);
 int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st);
 int launch_h2o_update_select(const kvx_h2o_args& a, hipStream_t st);
 size_t h2o_workspace(const kvx_h2o_args& a);
+int launch_h2o_update_select_static(const kvx_h2o_args& a, hipStream_t st);
+size_t h2o_static_scratch_bytes();
 int launch_rmsnorm_rows(const void* x, int64_t x_rs, void* out, int64_t o_rs, const float* weight, int64_t rows, int dim, float eps,
                         hipStream_t st);
 int launch_add_rmsnorm_rows(const void* x, int64_t x_rs, const void* delta, int64_t d_rs, void* x_out, int64_t xo_rs, void* out,
