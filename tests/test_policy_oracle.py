@@ -243,3 +243,106 @@ def test_replay_log_blocks_are_the_concatenated_slots():
             if start + num <= total:
                 assert torch.equal(log.extract_index(L + start, num), flat[:, :, start : start + num])
     assert log.finalize(L) == []
+
+
+# ---- normalised scores (keys_values/kvcache/h2o.py:183-196) ------------------------------------------
+
+
+def _normalised_choice_by_loop(score_rows, pos_rows, limit, k, input_pos_after, prefill_len, clamp_shift=1, pos_shift=0):
+    """Per-slot restatement with numpy float32 scalars: a slot holding the token at position p with
+    cumulative score s is compared by s / float32(input_pos_after - max(p, prefill_len - 1)); the k
+    smallest (value, slot) tuples. clamp_shift / pos_shift build the off-by-one variants a mistake would
+    produce, to show that the test data tells them apart."""
+    out = []
+    for srow, prow in zip(score_rows, pos_rows):
+        cands = []
+        for slot in range(limit):
+            resident_since = max(int(prow[slot]), prefill_len - clamp_shift)
+            den = np.float32(input_pos_after - pos_shift - resident_since)
+            cands.append((np.float32(srow[slot]) / den, slot))
+        cands.sort()
+        out.append([slot for _, slot in cands[:k]])
+    return out
+
+
+def test_normalised_selection_against_a_per_slot_loop():
+    """Both restatements of the normalised selection (oracle.kvx_oracle.h2o_update_select and
+    oracle.policy_oracle.update_select) against explicit per-slot loops. A third of the slots hold tokens
+    of the prefill (position < prefill_len - 1: the clamp decides their residency), the others later
+    tokens; the case is built so that clamping at prefill_len instead of prefill_len - 1, or dividing
+    by the position count before this step's advance, selects a different set."""
+    B, Hkv, L, limit, k = 2, 3, 96, 90, 17
+    prefill_len, q_len = 40, 4
+    input_pos_after = 200
+    gen = torch.Generator().manual_seed(21)
+    tp = torch.empty(B, Hkv, L, dtype=torch.int32)
+    for b in range(B):
+        for h in range(Hkv):
+            old = torch.randperm(prefill_len - 1, generator=gen)[: L // 3]              # < prefill_len - 1
+            new = prefill_len - 1 + torch.randperm(input_pos_after - q_len - prefill_len, generator=gen)[: L - L // 3]  # >= prefill_len - 1
+            tp[b, h] = torch.cat((old, new))[torch.randperm(L, generator=gen)].to(torch.int32)
+    assert (tp < prefill_len - 1).any() and (tp >= prefill_len - 1).any() and int(tp.max()) < input_pos_after
+    # scores proportional to the residency, so that all ratios are close and an off-by-one in the
+    # denominator reorders them; a little noise keeps exact ties away
+    res = (input_pos_after - tp.clamp_min(prefill_len - 1)).float()
+    scores0 = res * (1.0 + 0.02 * torch.rand(B, Hkv, L, generator=gen))
+    w = 0.01 * torch.rand(B, Hkv, L, generator=gen)
+    summed = (scores0 + w)  # fp32 add, as the update does
+    flat_s = summed.view(B * Hkv, L).numpy()
+    flat_p = tp.view(B * Hkv, L).numpy()
+    want = _normalised_choice_by_loop(flat_s, flat_p, limit, k, input_pos_after, prefill_len)
+    s1 = scores0.clone()
+    got1 = O.h2o_update_select(s1, w, L, limit, k, normalize=True, token_pos=tp, input_pos=input_pos_after, prefill_len=prefill_len)
+    s2 = scores0.clone()
+    got2, compared = P.update_select(s2, w, L, limit, k, normalize=True, token_pos=tp, input_pos=input_pos_after, prefill_len=prefill_len)
+    assert torch.equal(s1, summed) and torch.equal(s2, summed)
+    assert got1.view(B * Hkv, k).tolist() == want
+    assert got2.view(B * Hkv, k).tolist() == want
+    for r in range(B * Hkv):  # the compared values themselves, element by element
+        for slot in range(limit):
+            den = np.float32(input_pos_after - max(int(flat_p[r, slot]), prefill_len - 1))
+            assert compared.view(B * Hkv, limit)[r, slot].item() == float(np.float32(flat_s[r, slot]) / den)
+    # the plausible mistakes give another answer on this data (sets, not only order)
+    wrong_clamp = _normalised_choice_by_loop(flat_s, flat_p, limit, k, input_pos_after, prefill_len, clamp_shift=0)
+    wrong_pos = _normalised_choice_by_loop(flat_s, flat_p, limit, k, input_pos_after, prefill_len, pos_shift=q_len)
+    assert any(set(a) != set(b) for a, b in zip(want, wrong_clamp)), "data does not tell prefill_len from prefill_len - 1"
+    assert any(set(a) != set(b) for a, b in zip(want, wrong_pos)), "data does not tell input_pos before from after the advance"
+
+
+def test_normalised_cache_steps_against_a_per_token_model():
+    """Cache level: which input_pos and which prefill length reach the division. The model keeps a
+    dict token -> cumulative score per (b, h) and never sees a slot; after every step on a full cache
+    the oracle's next_index, read back through its token positions, must be the tokens with the
+    smallest score / (tokens seen so far, this step's included, - max(token, prefill_length - 1))."""
+    B, Hq, Hkv, L, D, chunk = 1, 4, 2, 40, 8, 4
+    n0 = 28  # prefill shorter than the cache: slots filled later are not clamped
+    steps = (4, 4, 4, 3, 4, 1, 4, 2)
+    q, k, v = _inputs(31, B, Hq, Hkv, n0 + sum(steps), D)
+    ora = P.PolicyCacheOracle(B, Hq, Hkv, L, D, max_chunk_size=chunk, normalize_scores=True)
+    ora.prefill(q[:, :, :n0], k[:, :, :n0], v[:, :, :n0])
+    model = [[{t: 0.0 for t in range(n0)} for _ in range(Hkv)] for _ in range(B)]
+    pos = n0
+    checked = 0
+    for num in steps:
+        before_tp = ora.token_pos.clone()
+        was_full = ora.current_length == L
+        _, w, index = ora.forward(q[:, :, pos : pos + num], k[:, :, pos : pos + num], v[:, :, pos : pos + num])
+        pos += num
+        for b in range(B):
+            for h in range(Hkv):
+                m = model[b][h]
+                if was_full:
+                    for t in before_tp[b, h, index[b, h]].tolist():
+                        del m[t]
+                for t in range(pos - num, pos):
+                    m[t] = 0.0
+                tp = ora.token_pos[b, h, : ora.current_length].tolist()
+                assert sorted(tp) == sorted(m)
+                for slot, t in enumerate(tp):
+                    m[t] = float(np.float32(m[t]) + np.float32(w[b, h, slot].item()))
+                if ora.current_length == L:
+                    ranked = sorted((np.float32(s) / np.float32(pos - max(t, n0 - 1)), tp.index(t)) for t, s in m.items())
+                    kk = ora.next_index.shape[-1]
+                    assert [slot for _, slot in ranked[:kk]] == ora.next_index[b, h].tolist()
+                    checked += 1
+    assert checked >= 4 * B * Hkv
