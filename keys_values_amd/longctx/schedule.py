@@ -1,32 +1,50 @@
-"""Chunk schedule of the long-context forward pass."""
+"""Chunk schedule of the long-context forward pass.
+
+Contract (``create_chunk_sizes`` with ``randomize_chunk_sizes=False``, keys_values/long_context.py:45-121,
+checked there by ``_assert_chunk_sizes``, :123-160):
+
+* the first chunk is the prefill: the smallest ``max_prefill_length`` of the caches;
+* every cache length that the sequence reaches is the end of a chunk, so that a cache is never filled
+  up in the middle of a chunk;
+* between two such cuts the tokens go in chunks of ``chunk_size``; what is left before a cut makes one
+  more chunk, unless it is ``ABSORB`` tokens or fewer, in which case the chunk before it takes them;
+* behind the last cut: chunks of ``chunk_size`` and one remainder.
+"""
 from typing import List, Sequence
 
-CLOSEBY_THRESHOLD = 4  # keys_values/long_context.py:40
+ABSORB = 4  # a chunk that would end this close to a cut ends on it (CLOSEBY_THRESHOLD, keys_values/long_context.py:40)
+
+
+def _cover(span: int, chunk_size: int, ends_on_cut: bool) -> List[int]:
+    """Chunk sizes for ``span`` tokens that start on a chunk boundary."""
+    if span <= 0:
+        return []
+    if not ends_on_cut:
+        whole, rest = divmod(span, chunk_size)
+        return [chunk_size] * whole + ([rest] if rest else [])
+    # whole chunks as long as more than chunk_size + ABSORB tokens remain; the last chunk takes the rest
+    whole = max(0, -((chunk_size + ABSORB - span) // chunk_size))
+    return [chunk_size] * whole + [span - whole * chunk_size]
 
 
 def create_chunk_sizes(max_prefill_length: int, cache_lengths: Sequence[int], seq_length: int, chunk_size: int) -> List[int]:
-    """Deterministic branch (``randomize_chunk_sizes=False``) of ``create_chunk_sizes``,
-    keys_values/long_context.py:45-121: the first chunk has the smallest ``max_prefill_length`` of
-    the caches, later chunks have ``chunk_size`` tokens, and no cache length falls inside a chunk (a
-    chunk that would end within ``CLOSEBY_THRESHOLD`` tokens of one, or beyond it, ends exactly there).
-
-    ``max_prefill_length``: min over the caches; ``cache_lengths``: the caches' lengths."""
+    """``max_prefill_length``: minimum over the caches; ``cache_lengths``: the caches' lengths.
+    Returns the chunk sizes, which add up to ``seq_length``."""
     if seq_length <= 0 or chunk_size <= 0 or max_prefill_length <= 0:
         raise ValueError("seq_length, chunk_size and max_prefill_length must be positive")
-    mpl = max_prefill_length
-    points_to_cover = sorted(set(c for c in cache_lengths if c <= seq_length))
-    if not points_to_cover:
-        return [seq_length] if mpl >= seq_length else [mpl, seq_length - mpl]
-    chunk_sizes = [mpl]
-    num_done = mpl
-    while num_done < seq_length:
-        c_size = min(chunk_size, seq_length - num_done)
-        next_pt = num_done + c_size
-        if points_to_cover and next_pt >= points_to_cover[0] - CLOSEBY_THRESHOLD:
-            c_size = points_to_cover.pop(0) - num_done
-        if c_size > 0:
-            chunk_sizes.append(c_size)
-        num_done += c_size
-    if sum(chunk_sizes) != seq_length:
-        raise AssertionError(f"chunk sizes {chunk_sizes} do not add up to {seq_length}")
-    return chunk_sizes
+    reached = sorted({int(c) for c in cache_lengths if c <= seq_length})
+    if not reached:
+        # no cache fills up: the prefill and, if the sequence is longer, all the rest in one chunk
+        # (keys_values/long_context.py:81-86)
+        first = min(max_prefill_length, seq_length)
+        return [first] + ([seq_length - first] if seq_length > first else [])
+    if reached[0] < max_prefill_length:
+        raise ValueError(f"cache length {reached[0]} is below the prefill length {max_prefill_length}")
+    sizes = [max_prefill_length]
+    at = max_prefill_length
+    for cut in reached:
+        sizes += _cover(cut - at, chunk_size, ends_on_cut=True)
+        at = cut
+    sizes += _cover(seq_length - at, chunk_size, ends_on_cut=False)
+    assert sum(sizes) == seq_length
+    return sizes

@@ -22,7 +22,10 @@ How each function is pinned (tests/test_oracle.py):
   blocks over heads), hand-computed vectors and packed bytes, and bit-equality with the scalar C
   restatement (IEEE float32 primitives only).
 * ``h2o_update_select`` / ``cache_write`` / ``H2OCacheOracle``: brute-force python loops on small caches
-  and the bookkeeping checks of test/kvcache/test_h2o.py:109-137,227-343.
+  and the bookkeeping checks of test/kvcache/test_h2o.py:109-137,227-343; the normalised selection
+  (scores divided by residency, keys_values/kvcache/h2o.py:183-196) by per-slot loops in numpy float32
+  on data that tells the clamp at prefill_length - 1 and the already advanced input_pos from their
+  off-by-one neighbours, and at cache level by a per-token model (tests/test_policy_oracle.py).
 * Tie order of ``torch.argsort`` / ``torch.topk(sorted=False)`` is implementation-defined in the
   reference (keys_values/kvcache/attn_weights.py:773-783): parity unpinned for ties; this oracle and
   the kernels both break ties towards the lower slot and tests compare sets away from ties.

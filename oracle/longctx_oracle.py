@@ -9,7 +9,12 @@ a float64 evaluation; the rotary encoding against its invariants (it preserves t
 (d, d + D/2) pair, position 0 is the identity, and q.k after rotation depends on the position
 difference only) and against the explicit per-pair 2x2 rotation; the chunk schedule against the
 properties its reference asserts (keys_values/long_context.py:123-160: sizes add up, the first chunk is
-the prefill length, no cache length inside a chunk). The MLP is litgpt's LLaMAMLP
+the prefill length, no cache length inside a chunk) and the reference's cursor walk on random cases;
+``qk_norm_rope`` row by row against the pinned pieces (which head gets which weight, each token its own
+position, values untouched) and against scalar arithmetic with both bf16 roundings written out;
+``PrefillOracle`` by zero output projections (the stack must reduce to the final norm of the
+embeddings) and by one block on tiny widths recomputed token by token with explicit matrix-vector
+products, the pinned row functions and a cache oracle of its own. The MLP is litgpt's LLaMAMLP
 (``proj(silu(fc_1 x) * fc_2 x)``); litgpt is not part of the reference tree (unpinned dependency of
 it), so that formula is restated from its published source: parity unpinned.
 """

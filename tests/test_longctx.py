@@ -39,6 +39,36 @@ def test_chunk_sizes_config5():
     assert sizes == [16384] + [1024] * 112
 
 
+def _schedule_by_walk(mpl, lengths, seq, chunk):
+    """Checker: the reference's cursor walk (keys_values/long_context.py:72-113, deterministic branch)."""
+    cuts = sorted(set(c for c in lengths if c <= seq))
+    if not cuts:
+        return [seq] if mpl >= seq else [mpl, seq - mpl]
+    out, done = [mpl], mpl
+    while done < seq:
+        size = min(chunk, seq - done)
+        if cuts and done + size >= cuts[0] - 4:
+            size = cuts.pop(0) - done
+        if size > 0:
+            out.append(size)
+        done += size
+    return out
+
+
+def test_chunk_sizes_equal_the_cursor_walk_on_random_cases():
+    import random
+
+    rnd = random.Random(7)
+    for _ in range(3000):
+        chunk = rnd.choice([1, 2, 3, 4, 5, 7, 16, 64, 100, 1024])
+        mpl = rnd.randint(1, 300)
+        lengths = [mpl + rnd.randint(0, 400) for _ in range(rnd.randint(1, 4))]
+        seq = rnd.randint(1, 1500)
+        assert create_chunk_sizes(mpl, lengths, seq, chunk) == _schedule_by_walk(mpl, lengths, seq, chunk), (mpl, lengths, seq, chunk)
+    with pytest.raises(ValueError):
+        create_chunk_sizes(100, [50], 200, 16)
+
+
 def test_rmsnorm_oracle_closed_forms():
     w = torch.linspace(0.5, 1.5, 64)
     # constant row c: |x|/sqrt(n) = |c|  ->  y = c / (|c| + eps) * w
@@ -88,6 +118,155 @@ def test_rope_oracle_invariants():
     assert dot(10, 3) == pytest.approx(dot(1010, 1003), rel=1e-3, abs=1e-3)
     # and agrees with the rotary encoding used to build the attention benchmark inputs
     torch.testing.assert_close(y, O.apply_rope(x, torch.arange(100, 100 + T)), rtol=1e-5, atol=1e-5)
+
+
+def _bf16_round(x: float) -> float:
+    """Round-to-nearest-even of a Python float to bfloat16, by hand on the fp32 bit pattern."""
+    import struct
+
+    bits = struct.unpack("<I", struct.pack("<f", x))[0]
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return struct.unpack("<f", struct.pack("<I", bits))[0]
+
+
+def test_qk_norm_rope_oracle_against_per_head_loops():
+    """keys_values/model.py:686-775: the projection's output holds, per token, n_head query heads, then
+    n_query_groups key heads, then as many value heads; queries are normalised with norm_q, keys with
+    norm_k (per head, over head_size), the result is rounded to the activations' type, then rotated by
+    the token's own position input_pos + t, and rounded again; values pass through."""
+    B, num, Hq, Hkv, D, input_pos, eps = 2, 5, 4, 2, 16, 37, 1e-6
+    gen = torch.Generator().manual_seed(8)
+    qkv = (torch.randn(B, num, (Hq + 2 * Hkv) * D, generator=gen) * 2).to(torch.bfloat16)
+    qw, kw = torch.rand(D, generator=gen) + 0.5, torch.rand(D, generator=gen) + 0.5
+    cos, sin = LO.rope_tables(256, D, 1e4)
+    q, k, v = LO.qk_norm_rope(qkv, Hq, Hkv, D, qw, kw, eps, cos, sin, input_pos)
+    assert q.shape == (B, Hq, num, D) and k.shape == (B, Hkv, num, D) and v.shape == (B, Hkv, num, D)
+    # (1) composition from the pinned pieces, one (token, head) row at a time
+    for b in range(B):
+        for t in range(num):
+            p = input_pos + t
+            for h in range(Hq + 2 * Hkv):
+                row = qkv[b, t, h * D : (h + 1) * D]
+                if h < Hq:
+                    want = LO.apply_rope(LO.rmsnorm(row.view(1, D), qw, eps), cos[p : p + 1], sin[p : p + 1])[0]
+                    assert torch.equal(q[b, h, t], want), (b, t, h)
+                elif h < Hq + Hkv:
+                    want = LO.apply_rope(LO.rmsnorm(row.view(1, D), kw, eps), cos[p : p + 1], sin[p : p + 1])[0]
+                    assert torch.equal(k[b, h - Hq, t], want), (b, t, h)
+                else:
+                    assert torch.equal(v[b, h - Hq - Hkv, t], row), (b, t, h)
+    # (2) scalar arithmetic in Python floats with both roundings written out, for every element of a few rows
+    worst = 0.0
+    differs_without_middle_round = False
+    for (b, t, h) in ((0, 0, 0), (1, 3, 2), (0, 4, Hq), (1, 1, Hq + 1)):
+        row = [float(x) for x in qkv[b, t, h * D : (h + 1) * D]]
+        wt = qw if h < Hq else kw
+        rms = math.sqrt(sum(x * x for x in row)) / math.sqrt(D)
+        exact = [x / (rms + eps) * float(wt[d]) for d, x in enumerate(row)]
+        normed = [_bf16_round(x) for x in exact]
+        p = input_pos + t
+        got = (q[b, h, t] if h < Hq else k[b, h - Hq, t]).tolist()
+        for src, check in ((normed, True), (exact, False)):
+            for d in range(D):
+                j = d % (D // 2)
+                ang = p * (1e4 ** (-2.0 * j / D))
+                other = -src[d + D // 2] if d < D // 2 else src[d - D // 2]
+                val = _bf16_round(src[d] * math.cos(ang) + other * math.sin(ang))
+                if check:
+                    worst = max(worst, abs(val - got[d]) / max(abs(val), 1e-3))
+                elif val != got[d]:
+                    differs_without_middle_round = True
+    assert worst <= 2 ** -7, worst  # at most the last bf16 bit (fp32 cos/sin against float64 here)
+    assert differs_without_middle_round, "the rounding between normalisation and rotation must be visible in the data"
+
+
+def _tiny_prefill_setup(quantized, zero_out=False, seed=3):
+    from types import SimpleNamespace
+
+    cfg = SimpleNamespace(n_layer=1, n_embd=16, n_head=2, n_query_groups=1, head_size=8, intermediate_size=24, vocab_size=50,
+                          rope_base=1e4, norm_eps=1e-5)
+    gen = torch.Generator().manual_seed(seed)
+
+    def w(o, i, std=0.3):
+        return (torch.randn(o, i, generator=gen) * std).to(torch.bfloat16)
+
+    d = cfg.head_size
+    layer = dict(qkv=w((cfg.n_head + 2 * cfg.n_query_groups) * d, cfg.n_embd), proj=w(cfg.n_embd, cfg.n_head * d),
+                 fc_1=w(cfg.intermediate_size, cfg.n_embd), fc_2=w(cfg.intermediate_size, cfg.n_embd),
+                 mlp_proj=w(cfg.n_embd, cfg.intermediate_size), norm_1=torch.rand(cfg.n_embd, generator=gen) + 0.5,
+                 norm_2=torch.rand(cfg.n_embd, generator=gen) + 0.5, norm_q=torch.rand(d, generator=gen) + 0.5,
+                 norm_k=torch.rand(d, generator=gen) + 0.5)
+    if zero_out:
+        layer["proj"].zero_()
+        layer["mlp_proj"].zero_()
+    wte = w(cfg.vocab_size, cfg.n_embd, 1.0)
+    ln_f = torch.rand(cfg.n_embd, generator=gen) + 0.5
+    L, chunk = 8, 2
+    ora = LO.PrefillOracle(cfg, wte, [layer], ln_f, L, chunk, 1, quantized, 64)
+    ids = torch.randint(0, cfg.vocab_size, (1, L + 3 * chunk), generator=gen)
+    return cfg, layer, wte, ln_f, L, chunk, ora, ids
+
+
+def test_prefill_oracle_with_zero_output_projections_is_the_final_norm_of_the_embeddings():
+    # both residual branches add exactly zero: the stack reduces to ln_f(wte[ids])
+    cfg, layer, wte, ln_f, L, chunk, ora, ids = _tiny_prefill_setup(False, zero_out=True)
+    start = 0
+    for n in (L, chunk, chunk, chunk):
+        sl = ids[:, start : start + n]
+        assert torch.equal(ora.forward_chunk(sl), LO.rmsnorm(wte[sl], ln_f, cfg.norm_eps))
+        start += n
+    assert ora.input_pos == L + 3 * chunk and ora.caches[0].input_pos == ora.input_pos
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+def test_prefill_oracle_one_layer_token_by_token(quantized):
+    """One block on tiny widths recomputed token by token: explicit matrix-vector products in fp32
+    rounded to bf16, the pinned row functions, and a cache oracle of its own fed chunk by chunk
+    (Block.forward, keys_values/model.py:560-584, non-parallel residual: x += attn(norm_1 x);
+    x += mlp(norm_2 x); CausalSelfAttention.forward, :686-811)."""
+    cfg, layer, wte, ln_f, L, chunk, ora, ids = _tiny_prefill_setup(quantized)
+    Hq, Hkv, D = cfg.n_head, cfg.n_query_groups, cfg.head_size
+    cos, sin = LO.rope_tables(64, D, cfg.rope_base)
+    cache = O.H2OCacheOracle(1, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=chunk)
+
+    def matvec(W, x):  # bf16 weights and activations, fp32 accumulation, one rounding
+        return torch.tensor([sum(float(a) * float(b) for a, b in zip(rowW, x)) for rowW in W.float()]).to(torch.bfloat16)
+
+    def stored(x):
+        return O.dequantize_rows(*O.quantize_rows(x)) if quantized else x
+
+    start = 0
+    for ci, n in enumerate((L, chunk, chunk, chunk)):
+        sl = ids[:, start : start + n]
+        got = ora.forward_chunk(sl)
+        xs = [wte[int(i)] for i in sl[0]]
+        q = torch.empty(1, Hq, n, D, dtype=torch.bfloat16)
+        k = torch.empty(1, Hkv, n, D, dtype=torch.bfloat16)
+        v = torch.empty(1, Hkv, n, D, dtype=torch.bfloat16)
+        for t, x in enumerate(xs):
+            qkv = matvec(layer["qkv"], LO.rmsnorm(x.view(1, -1), layer["norm_1"], cfg.norm_eps)[0])
+            p = start + t
+            for h in range(Hq):
+                q[0, h, t] = LO.apply_rope(LO.rmsnorm(qkv[h * D : (h + 1) * D].view(1, D), layer["norm_q"], cfg.norm_eps), cos[p : p + 1], sin[p : p + 1])[0]
+            for h in range(Hkv):
+                o = (Hq + h) * D
+                k[0, h, t] = LO.apply_rope(LO.rmsnorm(qkv[o : o + D].view(1, D), layer["norm_k"], cfg.norm_eps), cos[p : p + 1], sin[p : p + 1])[0]
+                v[0, h, t] = qkv[o + Hkv * D : o + Hkv * D + D]
+        if ci == 0:
+            att = cache.prefill(q, k, v, stored(k), stored(v))
+        else:
+            att, _, _ = cache.forward(q, stored(k), stored(v))
+        for t, x in enumerate(xs):
+            y = torch.cat([att[0, h, t] for h in range(Hq)])  # heads side by side, keys_values/attention/base.py:378-380
+            x = x + matvec(layer["proj"], y)
+            xn = LO.rmsnorm(x.view(1, -1), layer["norm_2"], cfg.norm_eps)[0]
+            g, u = matvec(layer["fc_1"], xn), matvec(layer["fc_2"], xn)
+            act = (g.float() / (1.0 + torch.exp(-g.float()))).to(torch.bfloat16)  # silu, rounded as an op of its own
+            x = x + matvec(layer["mlp_proj"], act * u)
+            want = LO.rmsnorm(x.view(1, -1), ln_f, cfg.norm_eps)[0]
+            torch.testing.assert_close(got[0, t].float(), want.float(), rtol=2 ** -6, atol=2 ** -7)
+        assert torch.equal(cache.token_pos, ora.caches[0].token_pos) and torch.equal(cache.scores, ora.caches[0].scores)
+        start += n
 
 
 # ---- GPU ------------------------------------------------------------------------------------------------
