@@ -22,6 +22,10 @@ Inputs are resident in HBM before the timed region.
 `--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
                        launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
+The default run also times, after the headline workload, the decode + H2O step, the quantiser and the
+long-context prefill on their own configurations and reports them under `config.secondary`
+(`--no-secondary` skips them).
+
 Prints ONE JSON line (see the keys below). `roofline` describes the dominant kernel, timed with
 events on the launch stream inside the timed steps; `cpu_baseline` times the CPU oracle (the
 reference's eager op sequence restated) on a bounded sample of the same workload.
@@ -59,6 +63,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="default workload only: skip the decode, quantiser and long-context legs that are reported under config.secondary")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
     ap.add_argument("--tokens", type=int, default=131072, help="longctx: prompt length")
@@ -623,8 +629,31 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fn = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib}[args.workload]
-    res = fn(args, torch, dev)
+    fns = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib}
+    res = fns[args.workload](args, torch, dev)
+    if args.workload == "prefill" and args.kv == "bf16" and not args.no_secondary:
+        # The other kernels with a target of their own, each on its own configuration, in the same run: the
+        # headline fields above stay what they are, these go under config.secondary.
+        import copy
+        import gc
+
+        secondary = {}
+        for name, steps, warmup in (("decode", 20, 5), ("quantize", 20, 5), ("longctx", 1, 1)):
+            sub = copy.copy(args)
+            sub.workload, sub.steps, sub.warmup = name, steps, warmup
+            gc.collect()
+            torch.cuda.empty_cache()
+            t0 = time.perf_counter()
+            try:
+                r = fns[name](sub, torch, dev)
+                secondary[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                                   "steps": r["steps"], "warmup": r["warmup"], "dtype": r["dtype"], "workload": r["config"]["workload"],
+                                   "detail": {k: v for k, v in r["config"].items() if k != "workload"},
+                                   "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"],
+                                   "wall_s": round(time.perf_counter() - t0, 1)}
+            except Exception as ex:  # a failing secondary leg must not take the headline measurement with it
+                secondary[name] = {"error": f"{type(ex).__name__}: {ex}"}
+        res["config"]["secondary"] = secondary
     print(json.dumps(res), flush=True)
 
 

@@ -182,10 +182,11 @@ __global__ __launch_bounds__(256) void update_argmin_kernel(const kvx_h2o_args a
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int i0 = base + it * 1024 + threadIdx.x * 4;
-    if (i0 + 3 < a.kv_len && ((a.sc_stride_h | a.sc_stride_b) & 3) == 0) {
+    // 16-byte loads need 16-byte aligned rows: the score rows by their strides, the rows of w (kv_len long) by kv_len
+    if (i0 + 3 < a.kv_len && ((a.sc_stride_h | a.sc_stride_b) & 3) == 0 && (!w || (a.kv_len & 3) == 0)) {
       f32x4_t s = *(const f32x4_t*)(sc + i0);
       if (w) {
-        const f32x4_t ww = *(const f32x4_t*)(w + i0);  // rows of w are kv_len long: aligned only if kv_len % 4 == 0
+        const f32x4_t ww = *(const f32x4_t*)(w + i0);
         s += ww;
         *(f32x4_t*)(sc + i0) = s;
       }

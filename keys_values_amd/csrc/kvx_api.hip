@@ -75,6 +75,10 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
     if (need_v_o) KVX_REQUIRE(a->v_scale && a->v_zp, KVX_ERR_INVALID, "%s: quantised cache needs v_scale and v_zp", who);
   }
   KVX_REQUIRE(a->num_splits >= 0, KVX_ERR_INVALID, "%s: num_splits must be >= 0", who);
+  // the tiled kernels address a tile's rows with 32-bit byte offsets from the tile's base: 64 rows of the slot stride
+  constexpr int64_t kMaxSlotStride = (int64_t)1 << 25;
+  KVX_REQUIRE(a->k_stride_t <= kMaxSlotStride && (!need_v_o || a->v_stride_t <= kMaxSlotStride), KVX_ERR_UNSUPPORTED,
+              "%s: slot strides above 2^25 elements are not supported", who);
   return KVX_OK;
 }
 
@@ -121,6 +125,7 @@ int kvx_sdpa_prefill(const kvx_sdpa_args* a, void* stream) {
   int rc = check_sdpa_common(a, "kvx_sdpa_prefill", true);
   if (rc != KVX_OK) return rc;
   KVX_REQUIRE(a->q_len <= a->kv_len, KVX_ERR_INVALID, "kvx_sdpa_prefill: q_len=%d exceeds kv_len=%d", a->q_len, a->kv_len);
+  KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_prefill: workspace must be 16-byte aligned");
   return launch_sdpa_prefill(*a, (hipStream_t)stream);
 }
 
@@ -137,6 +142,7 @@ int kvx_sdpa_prefill_weights(const kvx_sdpa_args* a, void* stream) {
   KVX_REQUIRE(a->q_len <= a->kv_len, KVX_ERR_INVALID, "kvx_sdpa_prefill_weights: q_len=%d exceeds kv_len=%d", a->q_len,
               a->kv_len);
   KVX_REQUIRE(a->lse && a->w, KVX_ERR_INVALID, "kvx_sdpa_prefill_weights: lse and w must be given");
+  KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_prefill_weights: workspace must be 16-byte aligned");
   rc = launch_sdpa_prefill(*a, (hipStream_t)stream);
   if (rc != KVX_OK) return rc;
   return launch_score_sum(*a, (hipStream_t)stream);

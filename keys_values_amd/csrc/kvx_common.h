@@ -112,7 +112,7 @@ __device__ __forceinline__ uint32_t quant_code(float x, float inv, float zf, flo
 // scale and zero point of a row from its min and max (IEEE division, no fast-math).
 __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, int32_t& zp, float qmax = 255.0f) {
   float s = (mx - mn) / qmax;
-  s = fmaxf(s, 1.1920929e-07f);
+  s = s < 1.1920929e-07f ? 1.1920929e-07f : s;  // torch.clamp(min=eps): a NaN stays a NaN (fmaxf would drop it)
   scale = s;
   zp = 0 - (int32_t)__builtin_rintf(mn / s);
 }

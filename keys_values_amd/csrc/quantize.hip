@@ -35,6 +35,98 @@ __device__ __forceinline__ float row_min(float v) {
   return v;
 }
 
+// Does one of the 8 values hold a NaN? The reference takes a row's extremes with torch.aminmax
+// (keys_values/kvcache/quantize/pytorch.py:90), which returns NaN for a row that holds one: such a row
+// gets a NaN scale and dequantises to NaN throughout (fminf / fmaxf would drop the NaN).
+__device__ __forceinline__ bool has_nan8(const float (&x)[8]) {
+  return __builtin_isunordered(x[0], x[1]) | __builtin_isunordered(x[2], x[3]) | __builtin_isunordered(x[4], x[5]) |
+         __builtin_isunordered(x[6], x[7]);
+}
+
+// True in all LPR lanes of a row if one of them says `bad`. The wavefront's ballot is a scalar: rows
+// with a NaN are rare, and the test costs a scalar compare when there is none.
+template <int LPR>
+__device__ __forceinline__ bool row_any(bool bad) {
+  const unsigned long long m = __ballot(bad);
+  if (m == 0) return false;
+  const int first = (int)(__lane_id() & ~(unsigned)(LPR - 1));
+  return ((m >> first) & ((1ull << LPR) - 1ull)) != 0;
+}
+
+// Codes of 4 values packed into a dword, byte e = clamp(rint(x[e] * inv) + zf, 0, 255). The sum is an
+// integer-valued float, so the conversion's rounding does not matter; v_cvt_pk_u8_f32 saturates to
+// [0, 255] (a NaN gives 0) and places the byte, which is the clamp, the cast and the packing in one.
+__device__ __forceinline__ uint32_t codes4_u8(float x0, float x1, float x2, float x3, float inv, float zf) {
+  uint32_t w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(x0 * inv) + zf, 0, 0);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(x1 * inv) + zf, 1, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(x2 * inv) + zf, 2, w);
+  return __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(x3 * inv) + zf, 3, w);
+}
+// The same with codes clamped to [0, 15] (4-bit store).
+__device__ __forceinline__ uint32_t codes4_u4(float x0, float x1, float x2, float x3, float inv, float zf) {
+  uint32_t w = __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_rintf(x0 * inv) + zf, 15.0f), 0, 0);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_rintf(x1 * inv) + zf, 15.0f), 1, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_rintf(x2 * inv) + zf, 15.0f), 2, w);
+  return __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_rintf(x3 * inv) + zf, 15.0f), 3, w);
+}
+
+template <int LPR>
+__device__ __forceinline__ void row_extremes(u32x4_t raw, float (&x)[8], float& mn, float& mx) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = bf16_lo(raw[e]);
+    x[2 * e + 1] = bf16_hi(raw[e]);
+  }
+  mn = x[0];
+  mx = x[0];
+#pragma unroll
+  for (int e = 1; e < 8; ++e) {
+    mn = fminf(mn, x[e]);
+    mx = fmaxf(mx, x[e]);
+  }
+  mn = row_min<LPR>(mn);
+  mx = row_max<LPR>(mx);
+  if (row_any<LPR>(has_nan8(x))) mn = mx = __builtin_nanf("");
+}
+
+// The ROWS_PER_THREAD rows a lane works on at once share the per-row arithmetic (three IEEE divisions):
+// all lanes of a row hold its extremes, so lane c of a quad works out the scale and zero point of row
+// c only, and the others fetch 1 / scale and the zero point from it with a quad broadcast. Returns the
+// codes of row i in c[i] (bytes), and in (scale, zp) the state of row (lane & 3).
+template <int LPR, int BITS>
+__device__ __forceinline__ void quantize_rows_in_flight(const u32x4_t (&raw)[ROWS_PER_THREAD], u32x2_t (&c)[ROWS_PER_THREAD], float& scale,
+                                                        int32_t& zp) {
+  static_assert(ROWS_PER_THREAD == 4, "one row per lane of a quad");
+  float x[ROWS_PER_THREAD][8], mn[ROWS_PER_THREAD], mx[ROWS_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) row_extremes<LPR>(raw[i], x[i], mn[i], mx[i]);
+  const int mine = (int)(__lane_id() & 3u);
+  const float my_mn = mine == 0 ? mn[0] : mine == 1 ? mn[1] : mine == 2 ? mn[2] : mn[3];
+  const float my_mx = mine == 0 ? mx[0] : mine == 1 ? mx[1] : mine == 2 ? mx[2] : mx[3];
+  quant_params(my_mn, my_mx, scale, zp, BITS == 8 ? 255.0f : 15.0f);
+  const int inv_bits = __builtin_bit_cast(int, 1.0f / scale);
+  const int zf_bits = __builtin_bit_cast(int, (float)zp);
+  float inv[ROWS_PER_THREAD], zf[ROWS_PER_THREAD];
+  inv[0] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(inv_bits, 0x00, 0xf, 0xf, true));  // quad_perm [0,0,0,0]
+  inv[1] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(inv_bits, 0x55, 0xf, 0xf, true));  // quad_perm [1,1,1,1]
+  inv[2] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(inv_bits, 0xAA, 0xf, 0xf, true));  // quad_perm [2,2,2,2]
+  inv[3] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(inv_bits, 0xFF, 0xf, 0xf, true));  // quad_perm [3,3,3,3]
+  zf[0] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(zf_bits, 0x00, 0xf, 0xf, true));
+  zf[1] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(zf_bits, 0x55, 0xf, 0xf, true));
+  zf[2] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(zf_bits, 0xAA, 0xf, 0xf, true));
+  zf[3] = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(zf_bits, 0xFF, 0xf, 0xf, true));
+#pragma unroll
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) {
+    if constexpr (BITS == 8) {
+      c[i][0] = codes4_u8(x[i][0], x[i][1], x[i][2], x[i][3], inv[i], zf[i]);
+      c[i][1] = codes4_u8(x[i][4], x[i][5], x[i][6], x[i][7], inv[i], zf[i]);
+    } else {
+      c[i][0] = codes4_u4(x[i][0], x[i][1], x[i][2], x[i][3], inv[i], zf[i]);
+      c[i][1] = codes4_u4(x[i][4], x[i][5], x[i][6], x[i][7], inv[i], zf[i]);
+    }
+  }
+}
+
 // Quantise the 8 values of this lane's share of a row; every lane of the row returns the same
 // scale / zero point.
 template <int LPR>
@@ -53,6 +145,7 @@ __device__ __forceinline__ u32x2_t quantize8(u32x4_t raw, float& scale, int32_t&
   }
   mn = row_min<LPR>(mn);
   mx = row_max<LPR>(mx);
+  if (row_any<LPR>(has_nan8(x))) mn = mx = __builtin_nanf("");  // aminmax propagates NaN, fminf / fmaxf drop it
   quant_params(mn, mx, scale, zp);
   const float inv = 1.0f / scale;
   const float zf = (float)zp;
@@ -78,19 +171,20 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t*
     const int64_t r = row0 + (int64_t)i * RPB;
     raw[i] = r < rows ? __builtin_nontemporal_load((const u32x4_t*)(x + r * x_row_stride + col * 8)) : u32x4_t{0, 0, 0, 0};
   }
+  u32x2_t c[ROWS_PER_THREAD];
+  float s;
+  int32_t z;
+  quantize_rows_in_flight<LPR, 8>(raw, c, s, z);  // executed by all lanes: the DPP exchanges need them
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
-    float s;
-    int32_t z;
-    const u32x2_t c = quantize8<LPR>(raw[i], s, z);  // executed by all lanes: the DPP reduction needs them
-    if (r < rows) {
-      *(u32x2_t*)(codes + r * D + col * 8) = c;
-      if (col == 0) {
-        scale[r] = s;
-        zp[r] = z;
-      }
-    }
+    if (r < rows) *(u32x2_t*)(codes + r * D + col * 8) = c[i];
+  }
+  // lane `col` of a row's first quad holds the state of row `col` of the four
+  const int64_t r_mine = row0 + (int64_t)col * RPB;
+  if (col < ROWS_PER_THREAD && r_mine < rows) {
+    scale[r_mine] = s;
+    zp[r_mine] = z;
   }
 }
 
@@ -141,6 +235,7 @@ __device__ __forceinline__ u32x2_t quantize4(u32x4_t raw, float& scale, int32_t&
   }
   mn = row_min<LPR>(mn);
   mx = row_max<LPR>(mx);
+  if (row_any<LPR>(has_nan8(x))) mn = mx = __builtin_nanf("");  // aminmax propagates NaN, fminf / fmaxf drop it
   quant_params(mn, mx, scale, zp, 15.0f);
   const float inv = 1.0f / scale;
   const float zf = (float)zp;
@@ -168,20 +263,20 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows4_kernel(const uint16_t
     const int64_t r = row0 + (int64_t)i * RPB;
     raw[i] = r < rows ? __builtin_nontemporal_load((const u32x4_t*)(x + r * x_row_stride + col * 8)) : u32x4_t{0, 0, 0, 0};
   }
+  u32x2_t c[ROWS_PER_THREAD];
+  float s;
+  int32_t z;
+  quantize_rows_in_flight<LPR, 4>(raw, c, s, z);  // executed by all lanes: the reductions and the exchanges need them
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
-    float s;
-    int32_t z;
-    const u32x2_t c = quantize4<LPR>(raw[i], s, z);  // executed by all lanes: the reductions and the exchange need them
-    const uint32_t p0 = __shfl_xor(c[0], LPR / 2, 64), p1 = __shfl_xor(c[1], LPR / 2, 64);
-    if (r < rows && col < LPR / 2) {
-      *(u32x2_t*)(codes + r * (D / 2) + col * 8) = u32x2_t{(c[0] << 4) | p0, (c[1] << 4) | p1};
-      if (col == 0) {
-        scale[r] = s;
-        zp[r] = z;
-      }
-    }
+    const uint32_t p0 = __shfl_xor(c[i][0], LPR / 2, 64), p1 = __shfl_xor(c[i][1], LPR / 2, 64);
+    if (r < rows && col < LPR / 2) *(u32x2_t*)(codes + r * (D / 2) + col * 8) = u32x2_t{(c[i][0] << 4) | p0, (c[i][1] << 4) | p1};
+  }
+  const int64_t r_mine = row0 + (int64_t)col * RPB;
+  if (col < ROWS_PER_THREAD && r_mine < rows) {
+    scale[r_mine] = s;
+    zp[r_mine] = z;
   }
 }
 
@@ -241,17 +336,19 @@ __global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_blo
   const int cps = a.D / 8;  // chunks of 8 values per segment
   const int nchunks = a.nseg * cps;
   auto chunk = [&](int c) { return *(const u32x4_t*)(base + (int64_t)(c / cps) * a.x_stride_seg + (c % cps) * 8); };
-  float mn = INFINITY, mx = -INFINITY;
+  float mn = INFINITY, mx = -INFINITY, bad = 0.0f;
   for (int c = lane; c < nchunks; c += 64) {
     const u32x4_t raw = chunk(c);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       mn = fminf(mn, fminf(bf16_lo(raw[e]), bf16_hi(raw[e])));
       mx = fmaxf(mx, fmaxf(bf16_lo(raw[e]), bf16_hi(raw[e])));
+      bad = __builtin_isunordered(bf16_lo(raw[e]), bf16_hi(raw[e])) ? 1.0f : bad;
     }
   }
   mn = wave_min(mn);
   mx = wave_max(mx);
+  if (wave_max(bad) != 0.0f) mn = mx = __builtin_nanf("");  // as torch.aminmax: a NaN in the block is the block's extreme
   constexpr float qmax = BITS == 8 ? 255.0f : 15.0f;
   float s;
   int32_t z;

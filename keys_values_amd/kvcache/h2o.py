@@ -97,9 +97,9 @@ class H2OKVCache:
         # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
         self.dequantize_chunk_rows = dequantize_chunk_rows
         # overlap_select: launch the score update + eviction choice of a chunk step on a second stream, so
-        # that it runs beside whatever the caller enqueues next; the next forward waits for it. The scores,
-        # the next slots and token_pos must then not be read from the caller's stream before
-        # wait_for_selection() (the properties of this class do that).
+        # that it runs beside whatever the caller enqueues next; the next forward and next_positions() wait
+        # for it. The attributes scores, token_pos and _next_index are plain tensors: a caller that reads
+        # them directly calls wait_for_selection() first.
         self._overlap = bool(overlap_select)
         self._side_stream = None
         self._select_done = None

@@ -55,6 +55,39 @@ def test_quantize_rows_bit_exact(kvx, gpu, rows, D):
     assert torch.equal(out.cpu(), O.dequantize_rows(c_ref, s_ref, z_ref, torch.bfloat16)), "dequantised rows differ"
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantize_row_with_nan(kvx, gpu, bits):
+    """torch.aminmax gives NaN extremes for a row that holds a NaN (keys_values/kvcache/quantize/pytorch.py:90),
+    so the row's scale is NaN and the row dequantises to NaN throughout; what its zero point and codes are
+    is a float-to-integer conversion of NaN, which the reference leaves to the platform: not compared.
+    Rows without a NaN are untouched by their neighbours."""
+    rows, D = 64, 128
+    x = outlier_rows(5, rows, D)
+    x[3, 17] = float("nan")
+    x[40, 0] = float("nan")
+    x[41, D - 1] = -float("nan")
+    bad = torch.tensor([3, 40, 41])
+    good = torch.tensor([r for r in range(rows) if r not in (3, 40, 41)])
+    c_ref, s_ref, z_ref = O.quantize_rows(x, bits)
+    assert torch.isnan(s_ref[bad]).all() and not torch.isnan(s_ref[good]).any()
+    xg = x.to(gpu)
+    codes = torch.empty((rows, D if bits == 8 else D // 2), dtype=torch.uint8, device=gpu)
+    sc = torch.empty(rows, dtype=torch.float32, device=gpu)
+    zp = torch.empty(rows, dtype=torch.int32, device=gpu)
+    fn = kvx.kvx_quantize_rows if bits == 8 else kvx.kvx_quantize_rows4
+    _lib.check(fn(xg.data_ptr(), D, rows, D, codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), _lib.stream_ptr(gpu)))
+    out = torch.empty((rows, D), dtype=torch.bfloat16, device=gpu)
+    dq = kvx.kvx_dequantize_rows if bits == 8 else kvx.kvx_dequantize_rows4
+    _lib.check(dq(codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), rows, D, out.data_ptr(), D, _lib.stream_ptr(gpu)))
+    torch.cuda.synchronize()
+    assert torch.isnan(sc.cpu()[bad]).all()
+    assert torch.isnan(out.cpu()[bad].float()).all()
+    want_codes = O.compress4(c_ref) if bits == 4 else c_ref
+    assert torch.equal(sc.cpu()[good], s_ref[good]) and torch.equal(zp.cpu()[good], z_ref[good])
+    assert torch.equal(codes.cpu()[good], want_codes[good])
+    assert torch.equal(out.cpu()[good], O.dequantize_rows(c_ref, s_ref, z_ref)[good])
+
+
 def test_quantize_empty_and_strided(kvx, gpu):
     assert kvx.kvx_quantize_rows(None, 128, 0, 128, None, None, None, None) == 0
     x = outlier_rows(4, 300, 256).to(gpu)  # rows of 128 inside rows of 256

@@ -379,6 +379,7 @@ def test_prefill_model_vs_oracle(gpu, quantized):
             forced = []
             for li, cache in enumerate(model.caches):
                 want = ref.caches[li].next_index
+                cache.wait_for_selection()  # the choice runs on a second stream
                 got = cache._next_index[:B].cpu().long()
                 for h in range(cfg.n_query_groups):
                     a, r = set(got[0, h, :chunk].tolist()), set(want[0, h, :chunk].tolist())
