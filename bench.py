@@ -206,8 +206,7 @@ def bench_prefill(args, torch, dev):
         cache.batch_size, cache.current_length, cache.prefill_length = B, T, T
         cache._input_pos = T
         cache._use_initial_rule = False
-        cache._next_index.copy_(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
-        cache._have_next = True
+        cache.set_next_positions(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
         kn, vn = k[:, :, -q_len:].contiguous(), v[:, :, -q_len:].contiguous()
         for _ in range(3):
             cache.forward(q, kn, vn)
@@ -366,8 +365,7 @@ def bench_decode(args, torch, dev):
     cache.batch_size, cache.current_length, cache.prefill_length = B, L, L
     cache._input_pos = L
     cache._use_initial_rule = False
-    cache._next_index.zero_()
-    cache._have_next = True
+    cache.set_next_positions(torch.zeros((B, Hkv, 1), dtype=torch.int32, device=dev))
     n = args.steps + args.warmup
     qs = torch.randn((n, B, Hq, 1, D), generator=gen, device=dev).to(torch.bfloat16)
     ks = torch.randn((n, B, Hkv, 1, D), generator=gen, device=dev).to(torch.bfloat16)
@@ -539,8 +537,7 @@ def bench_policy(args, torch, dev):
         cache._input_pos = T
         cache._use_initial_rule = False
         cache.next_grace_pos = T - cache.grace_period if cache.grace_period else None
-        cache._next_index.copy_(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
-        cache._have_next = True
+        cache.set_next_positions(torch.arange(q_len, dtype=torch.int32, device=dev).view(1, 1, q_len).expand(B, Hkv, q_len))
         for _ in range(max(args.warmup, 2)):
             cache.forward(q, kn, vn)
         torch.cuda.synchronize()

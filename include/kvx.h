@@ -289,7 +289,9 @@ int kvx_cache_write(const kvx_cache_write_args* args, void* stream);
  * the same set in unspecified order. limit = cache_length - grace_period: the ring is never evicted.
  * With normalize != 0 the value compared is
  * scores / (input_pos - max(token_pos, prefill_len - 1)) (keys_values/kvcache/h2o.py:183-196);
- * token_pos then must be given. 1 <= k <= min(limit, 4096); limit <= kv_len.
+ * token_pos then must be given. 1 <= k <= limit <= kv_len; up to 4096 slots are chosen per kernel launch,
+ * a longer selection (up to the whole argsort, k = limit) takes ceil(k / 4096) launches and 8 bytes of
+ * workspace per row.
  * scores rows at scores + b*sc_stride_b + h*sc_stride_h; w contiguous (B, Hkv, kv_len).
  * next_index: int32 (B, Hkv, k) contiguous.
  *

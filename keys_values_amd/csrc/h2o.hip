@@ -236,8 +236,17 @@ __global__ void argmin_finish_kernel(const unsigned long long* best, int32_t* ne
 
 // CACHED: the row's ordered keys live in LDS after the first pass (rows of up to ~36K slots), so the
 // radix passes and the gather never go back to global memory.
+// Selections of more than MAX_PASS_K slots run as several launches: each takes the next a.k smallest
+// (value, slot) keys above `bound` (the last key of the launch before, per row) and leaves its own last
+// key there. out_off / out_stride place the launch's slots inside the row of next_index.
+struct SelectPass {
+  unsigned long long* bound;  // per row, or nullptr: a single launch
+  int lower;                  // 1: only keys above bound[row] take part
+  int out_off, out_stride;
+};
+
 template <bool CACHED>
-__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a, int kpad, const float* stats) {
+__global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2o_args a, int kpad, const float* stats, const SelectPass ps) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   unsigned long long* cand = (unsigned long long*)dyn_lds;    // kpad entries
   uint32_t* keys = (uint32_t*)(dyn_lds + (size_t)kpad * 8);   // a.limit entries (CACHED only)
@@ -253,6 +262,15 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
   const float* w = a.w ? a.w + (int64_t)row * a.kv_len : nullptr;
   const int32_t* tpr = a.token_pos ? a.token_pos + b * a.tp_stride_b + hh * a.tp_stride_h : nullptr;
   const Modify md = load_modify(a, stats, b, hh);
+  // keys at or below the bound were taken by an earlier launch: they get the largest key and so never
+  // come before a key still to be taken
+  const unsigned long long bound = ps.lower ? ps.bound[row] : 0ull;
+  const uint32_t bound_u = (uint32_t)(bound >> 32), bound_i = (uint32_t)bound;
+  auto live_key = [&](float v, int i) -> uint32_t {
+    const uint32_t u = ordered_bits(select_value(v, a, tpr, i, md));
+    if (ps.lower && (u < bound_u || (u == bound_u && (uint32_t)i <= bound_i))) return 0xffffffffu;
+    return u;
+  };
 
   // pass 0: scores += w (every later pass of this thread touches the slots it wrote here) and the keys
   // One workgroup walks the whole row: batches of 8 loads per array are issued before anything is
@@ -277,12 +295,12 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
         v += wv[j];
         sc[i] = v;
       }
-      if (CACHED && i < a.limit) keys[i] = ordered_bits(select_value(v, a, tpr, i, md));
+      if (CACHED && i < a.limit) keys[i] = live_key(v, i);
     }
   }
   auto key_of = [&](int i) -> uint32_t {
     if constexpr (CACHED) return keys[i];
-    else return ordered_bits(select_value(sc[i], a, tpr, i, md));
+    else return live_key(sc[i], i);
   };
 
   for (int i = tid; i < kpad; i += SEL_THREADS) cand[i] = ~0ull;
@@ -441,13 +459,18 @@ __global__ __launch_bounds__(SEL_THREADS) void update_select_kernel(const kvx_h2
       else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     }
   __syncthreads();
-  for (int j = tid; j < a.k; j += SEL_THREADS) a.next_index[(int64_t)row * a.k + j] = (int32_t)(cand[j] & 0xffffffffull);
+  for (int j = tid; j < a.k; j += SEL_THREADS) a.next_index[(int64_t)row * ps.out_stride + ps.out_off + j] = (int32_t)(cand[j] & 0xffffffffull);
+  if (ps.bound && tid == 0) ps.bound[row] = cand[a.k - 1];
 }
 
 }  // namespace
 
 static bool is_variant(const kvx_h2o_args& a) { return a.v_norm != nullptr || a.q_errors != nullptr; }
-static size_t best_bytes(const kvx_h2o_args& a) { return a.k == 1 ? ((size_t)a.B * a.Hkv * sizeof(unsigned long long) + 15) / 16 * 16 : 0; }
+constexpr int MAX_PASS_K = 4096;  // slots one launch of update_select_kernel sorts in LDS
+// per row one 64-bit key: the running minimum of k == 1, or the bound handed from launch to launch when k > MAX_PASS_K
+static size_t best_bytes(const kvx_h2o_args& a) {
+  return (a.k == 1 || a.k > MAX_PASS_K) ? ((size_t)a.B * a.Hkv * sizeof(unsigned long long) + 15) / 16 * 16 : 0;
+}
 
 size_t h2o_workspace(const kvx_h2o_args& a) { return best_bytes(a) + (a.q_errors ? (size_t)a.B * a.Hkv * 4 * sizeof(float) : 0); }
 
@@ -477,19 +500,31 @@ int launch_h2o_update_select(const kvx_h2o_args& a_in, hipStream_t st) {
     KVX_HIP(hipGetLastError());
     return KVX_OK;
   }
-  int kpad = 1;
-  while (kpad < a.k) kpad <<= 1;
-  // keys in LDS when the row fits beside the candidates (144 KB of the 160 KB of a compute unit)
-  constexpr size_t kDynLimit = 144 * 1024;
-  const size_t cached_bytes = (size_t)kpad * 8 + (size_t)a.limit * 4;
-  if (cached_bytes <= kDynLimit) {
-    if (cached_bytes > 48 * 1024)  // beyond the default dynamic LDS allowance (the setting is per device and kernel)
-      KVX_HIP(hipFuncSetAttribute((const void*)update_select_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLimit));
-    hipLaunchKernelGGL(update_select_kernel<true>, dim3(rows), dim3(SEL_THREADS), cached_bytes, st, a, kpad, (const float*)stats);
-  } else {
-    hipLaunchKernelGGL(update_select_kernel<false>, dim3(rows), dim3(SEL_THREADS), (size_t)kpad * 8, st, a, kpad, (const float*)stats);
+  // up to MAX_PASS_K slots per launch; a longer selection (the reference keeps the whole argsort when no chunk
+  // size is set, keys_values/kvcache/attn_weights.py:773-774) continues above the last key of the launch before
+  const int k_total = a.k;
+  SelectPass ps;
+  ps.bound = k_total > MAX_PASS_K ? (unsigned long long*)a.workspace : nullptr;
+  ps.out_stride = k_total;
+  for (int done = 0; done < k_total; done += MAX_PASS_K) {
+    a.k = min(MAX_PASS_K, k_total - done);
+    ps.lower = done > 0;
+    ps.out_off = done;
+    int kpad = 1;
+    while (kpad < a.k) kpad <<= 1;
+    // keys in LDS when the row fits beside the candidates (144 KB of the 160 KB of a compute unit)
+    constexpr size_t kDynLimit = 144 * 1024;
+    const size_t cached_bytes = (size_t)kpad * 8 + (size_t)a.limit * 4;
+    if (cached_bytes <= kDynLimit) {
+      if (cached_bytes > 48 * 1024)  // beyond the default dynamic LDS allowance (the setting is per device and kernel)
+        KVX_HIP(hipFuncSetAttribute((const void*)update_select_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLimit));
+      hipLaunchKernelGGL(update_select_kernel<true>, dim3(rows), dim3(SEL_THREADS), cached_bytes, st, a, kpad, (const float*)stats, ps);
+    } else {
+      hipLaunchKernelGGL(update_select_kernel<false>, dim3(rows), dim3(SEL_THREADS), (size_t)kpad * 8, st, a, kpad, (const float*)stats, ps);
+    }
+    KVX_HIP(hipGetLastError());
+    a.w = nullptr;  // the scores are updated once
   }
-  KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
 

@@ -280,7 +280,7 @@ static int check_h2o(const kvx_h2o_args* a, const char* who) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "%s: h2o args is NULL", who);
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->kv_len > 0, KVX_ERR_INVALID, "%s: sizes must be positive", who);
   KVX_REQUIRE(a->limit > 0 && a->limit <= a->kv_len, KVX_ERR_INVALID, "%s: limit=%d must be in [1, kv_len=%d]", who, a->limit, a->kv_len);
-  KVX_REQUIRE(a->k >= 1 && a->k <= a->limit && a->k <= 4096, KVX_ERR_INVALID, "%s: k=%d must be in [1, min(limit, 4096)]", who, a->k);
+  KVX_REQUIRE(a->k >= 1 && a->k <= a->limit, KVX_ERR_INVALID, "%s: k=%d must be in [1, limit=%d]", who, a->k, a->limit);
   KVX_REQUIRE(a->scores && a->next_index, KVX_ERR_INVALID, "%s: NULL pointer", who);
   KVX_REQUIRE(!a->normalize || a->token_pos, KVX_ERR_INVALID, "%s: normalize needs token_pos", who);
   KVX_REQUIRE(!(a->v_norm && a->w) || a->q_len > 0, KVX_ERR_INVALID, "%s: v_norm needs q_len > 0", who);

@@ -28,7 +28,7 @@ the Q-Hitter combination with the quantisation error (``QuantizedH2OKVCache`` /
 keys_values/kvcache/factory.py:50-66. With ``switch_replay_logging(True)`` the cache records the token
 chunks and the slot every later token went to (keys_values/kvcache/attn_weights.py:43-204,939-966).
 
-Not covered (raises): fp16/fp32 caches, bitsandbytes stores, quantisation blocks over heads in the cache object.
+Not covered (raises): fp32 caches, bitsandbytes stores, quantisation blocks over heads in the cache object.
 """
 import ctypes
 from dataclasses import dataclass
@@ -42,7 +42,10 @@ from .replay import DEFAULT_REPLAY_LOG_BLOCKSIZE, AttnWeightsReplayLog, ReplayAr
 
 DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
 DEFAULT_COMBINATION_CONSTANT = 0.5  # keys_values/kvcache/qh2o.py:25
-MAX_SELECT = 4096  # largest k of kvx_h2o_update_select
+# Slots one launch of the selection kernel chooses. A step on a full cache chooses min(this, what the
+# cache may be asked for); a later request for more (a chunk longer than this with no max_chunk_size) is
+# served by selecting again, from the same scores, as many slots as it needs.
+EAGER_SELECT = 4096
 # Query rows (tokens x heads per KV head) of a chunk from which dequantising the store once per chunk
 # is faster than dequantising it inside the attention kernels (every 256 rows walk the whole store):
 # the copy costs two passes over the store, the kernels gain in proportion to the rows.
@@ -146,7 +149,10 @@ class H2OKVCache:
             max_chunk_size = None
         self.max_chunk_size = max_chunk_size
         limit = self.cache_length - grace_period
-        self._select_k = min(limit, MAX_SELECT) if max_chunk_size is None else min(max_chunk_size, limit, MAX_SELECT)
+        # what next_positions may be asked for on a full cache: the whole argsort when no chunk size is set
+        # (keys_values/kvcache/attn_weights.py:773-783)
+        self._select_k = limit if max_chunk_size is None else min(max_chunk_size, limit)
+        self._next_count = 0  # leading entries of _next_index that hold the current choice
         self._keep_initial_fraction = keep_initial_fraction
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         if self.device.type != "cuda":
@@ -170,7 +176,8 @@ class H2OKVCache:
         if grace_period > 0:  # the ring twice over: any wrap-around run of up to grace_period slots is one view of it
             ring = torch.arange(length - grace_period, length, dtype=torch.int32, device=self.device)
             self._ring_twice = torch.cat((ring, ring))
-        self._next_index = torch.zeros((b, h, self._select_k), dtype=torch.int32, device=self.device)
+        # the current choice: (batch, heads, _next_count) slots, packed at the start of this buffer
+        self._next_flat = torch.zeros(b * h * self._select_k, dtype=torch.int32, device=self.device)
         self._have_next = False
         self._use_initial_rule = None
         self._input_pos = 0
@@ -197,7 +204,7 @@ class H2OKVCache:
             result = min(result, diff)
         if self.max_chunk_size is not None:
             result = min(result, self.max_chunk_size)
-        return min(result, self._select_k) if diff == 0 else result
+        return result
 
     def token_positions(self) -> torch.Tensor:
         if self.current_length is None:
@@ -209,6 +216,24 @@ class H2OKVCache:
         if self._select_done is not None:
             torch.cuda.current_stream(self.device).wait_event(self._select_done)
             self._select_done, self._select_keep = None, None
+
+    @property
+    def _next_index(self) -> torch.Tensor:
+        """(max_batch_size, n_query_groups, _next_count) view of the slots chosen last."""
+        c = max(self._next_count, 1)
+        n = self.max_batch_size * self.n_query_groups * c
+        return self._next_flat[:n].view(self.max_batch_size, self.n_query_groups, c)
+
+    def set_next_positions(self, index: torch.Tensor):
+        """Replace the choice of the next slots to write by ``index`` (batch, n_query_groups, num): for
+        callers that decide the eviction themselves, and for tests that keep two caches in step."""
+        b, h, num = index.shape
+        if h != self.n_query_groups or b > self.max_batch_size or not 1 <= num <= self._select_k:
+            raise ValueError(f"index.shape = {tuple(index.shape)} does not fit the cache")
+        self.wait_for_selection()
+        self._next_count = num
+        self._next_index[:b].copy_(index.to(device=self.device, dtype=torch.int32))
+        self._have_next = True
 
     def next_positions(self, num: int) -> Optional[torch.Tensor]:
         """Slots the next ``forward`` writes to, int64 (batch, n_query_groups, num), or None
@@ -274,7 +299,25 @@ class H2OKVCache:
             return torch.arange(n0, n0 + num, dtype=torch.int32, device=self.device).view(1, 1, -1).expand(b, h, -1).contiguous()
         if not self._have_next:
             return None
+        if num > self._next_count:
+            self._select_more(num)
         return self._next_index[:b, :, :num]
+
+    def _select_more(self, num: int):
+        """The step before chose fewer slots than are asked for now (it could not know): choose ``num`` from
+        the same scores. Nothing is added to them (no weights), so the first entries come out as before."""
+        if num > self._select_k:
+            raise ValueError(f"num = {num} exceeds what a full cache hands out ({self._select_k})")
+        a = self._h2o_args(True, num)
+        a.next_index = self._next_flat.data_ptr()
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            nbytes = lib.kvx_h2o_workspace_bytes(ctypes.byref(a))
+            ws = _lib.workspace(self.device, nbytes)
+            a.workspace = _lib.ptr(ws)
+            a.workspace_bytes = 0 if ws is None else ws.numel()
+            _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
+        self._next_count = num
 
     # -- the step (keys_values/kvcache/base.py:554-595) -----------------------------------------
 
@@ -434,11 +477,11 @@ class H2OKVCache:
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
 
-    def _h2o_args(self, full: bool) -> _lib.H2OArgs:
+    def _h2o_args(self, full: bool, k: int = 1) -> _lib.H2OArgs:
         a = _lib.H2OArgs()
         a.B, a.Hkv, a.kv_len = self.batch_size, self.n_query_groups, self.current_length
         a.limit = self.cache_length - self.grace_period if full else self.current_length
-        a.k = self._select_k if full else 1
+        a.k = k if full else 1
         a.normalize = int(self.normalize_scores and full)
         a.input_pos = self._input_pos
         a.prefill_len = self.prefill_length
@@ -454,13 +497,15 @@ class H2OKVCache:
     def _decode_h2o_step(self, query, kc, vc, quant) -> torch.Tensor:
         """``self.mha(...)`` and ``self._update(...)`` of keys_values/kvcache/base.py:583-595 for one new
         token and a full cache, as the single fused call ``kvx_sdpa_decode_h2o`` (selection size 1)."""
-        if self._select_k != 1 or self.v_length or self.q_hitter:
+        if self.v_length or self.q_hitter:
             out, w, _ = ops.decode_core(query, kc, vc, self.scale_factor, return_weights=True, quant=quant)
-            self._update(w, 1)
+            self._update(w, 1, select=1)
             return out
+        # the lowest-score slot only: a following single-token step needs no more, anything longer selects again
         launch, out = self._decode_h2o_prepare(query, kc, vc, quant)
         launch()
         self._have_next = True
+        self._next_count = 1
         return out
 
     def _decode_h2o_prepare(self, query, kc, vc, quant):
@@ -476,8 +521,8 @@ class H2OKVCache:
             ops._fill_common(a, query, kc, vc, self.scale_factor, self.current_length - 1, None, quant, 0)
             a.o = o_view.data_ptr()
             a.o_stride_b, a.o_stride_h, a.o_stride_t = o_view.stride(0), o_view.stride(1), o_view.stride(2)
-            h = self._h2o_args(True)
-            h.next_index = self._next_index.data_ptr()
+            h = self._h2o_args(True, 1)
+            h.next_index = self._next_flat.data_ptr()
             nb_a = lib.kvx_sdpa_decode_h2o_workspace_bytes(ctypes.byref(a))
             nb_h = (lib.kvx_h2o_workspace_bytes(ctypes.byref(h)) + 255) // 256 * 256
             ws = _lib.workspace(dev, nb_a + nb_h)
@@ -492,8 +537,9 @@ class H2OKVCache:
         launch.keepalive = (query, kc, vc, quant, out, ws)
         return launch, out
 
-    def _update(self, attn_weights: torch.Tensor, query_length: int):
-        """keys_values/kvcache/attn_weights.py:721-783 with keys_values/kvcache/h2o.py:146-199."""
+    def _update(self, attn_weights: torch.Tensor, query_length: int, select: Optional[int] = None):
+        """keys_values/kvcache/attn_weights.py:721-783 with keys_values/kvcache/h2o.py:146-199. ``select``: how
+        many slots to choose now (default: as many as a next step may take, at most EAGER_SELECT)."""
         if not isinstance(attn_weights, torch.Tensor):
             raise TypeError("attn_weights argument needs to be torch.Tensor")
         if not isinstance(query_length, int) or query_length <= 0:
@@ -506,13 +552,14 @@ class H2OKVCache:
         _lib.require_gpu(attn_weights)
         attn_weights = attn_weights.contiguous()
         full = self.current_length == self.cache_length
-        a = self._h2o_args(full)
+        k_now = min(self._select_k, EAGER_SELECT) if select is None else min(select, self._select_k)
+        a = self._h2o_args(full, k_now)
         a.w = attn_weights.data_ptr()
         a.q_len = query_length
         lib = _lib.load()
         with torch.cuda.device(self.device):
             if full:
-                nxt = self._next_index
+                nxt = self._next_flat
             else:  # only the accumulation matters while slots are free; the choice is discarded
                 nxt = torch.empty((self.batch_size, self.n_query_groups, 1), dtype=torch.int32, device=self.device)
             a.next_index = nxt.data_ptr()
@@ -542,6 +589,7 @@ class H2OKVCache:
                 nxt.record_stream(self._side_stream)
                 self._select_keep = (attn_weights, nxt)
         self._have_next = full
+        self._next_count = k_now if full else 0
 
 
 class VLengthH2OKVCache(H2OKVCache):

@@ -205,6 +205,8 @@ def gpu_h2o(kvx, gpu, scores, w, kv_len, limit, k, normalize=False, token_pos=No
 @pytest.mark.parametrize("B,Hkv,L,kv_len,limit,k", [
     (2, 3, 300, 300, 300, 1), (8, 8, 5000, 5000, 5000, 1), (1, 2, 1024, 1024, 1024, 128), (2, 2, 4097, 4000, 3999, 1000),
     (1, 8, 16384, 16384, 16384, 1024), (1, 1, 64, 64, 64, 64), (1, 2, 131072, 131072, 131072, 4096), (2, 2, 10001, 10001, 10001, 1),
+    # more than one launch of 4096 slots, up to the whole argsort (keys_values/kvcache/attn_weights.py:773-774)
+    (1, 2, 20000, 20000, 20000, 9000), (2, 1, 8192, 8192, 8192, 8192), (1, 2, 131072, 131072, 131000, 131000), (1, 1, 5000, 4999, 4500, 4097),
 ])
 def test_h2o_update_select(kvx, gpu, B, Hkv, L, kv_len, limit, k):
     gen = torch.Generator().manual_seed(L + k)
@@ -229,6 +231,52 @@ def test_h2o_select_ties_and_no_weights(kvx, gpu):
         s_gpu, n_gpu = gpu_h2o(kvx, gpu, scores, None, 999, 999, k)
         assert torch.equal(n_gpu.long(), n_ref)
         assert torch.equal(s_gpu, scores)
+
+
+def test_h2o_select_ties_across_launches(kvx, gpu):
+    # a selection of several launches whose cuts fall inside long runs of equal scores: the order within a
+    # run is by slot, and a run is continued, not repeated, by the next launch
+    gen = torch.Generator().manual_seed(8)
+    scores = torch.randint(0, 4, (2, 2, 12000), generator=gen).float()
+    for k in (4096, 4097, 9000, 12000):
+        s_ref = scores.clone()
+        n_ref = O.h2o_update_select(s_ref, None, 12000, 12000, k)
+        _, n_gpu = gpu_h2o(kvx, gpu, scores, None, 12000, 12000, k)
+        assert torch.equal(n_gpu.long(), n_ref), k
+
+
+def test_cache_selects_again_when_asked_for_more(gpu):
+    """No max_chunk_size: the reference keeps the whole argsort and serves any chunk up to the cache length
+    (keys_values/kvcache/attn_weights.py:501-508,773-774). The cache chooses one slot after a single-token
+    step and selects again when a longer chunk follows."""
+    B, Hq, Hkv, L, D = 1, 2, 1, 10000, 64
+    gen = torch.Generator().manual_seed(12)
+    total = L + 1 + 1 + 6000 + 1
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=None)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=None, device=gpu)
+    ref.prefill(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L])
+    cache.forward(qs[:, :, :L].to(gpu), ks[:, :, :L].to(gpu), vs[:, :, :L].to(gpu))
+    pos = L
+    for num in (1, 1, 6000, 1):
+        assert cache.max_forward_length() == L
+        sl = slice(pos, pos + num)
+        had = ref.next_index is not None
+        if had:
+            want = ref.next_index[:, :, :num]
+            got = cache.next_positions(num).cpu()
+            assert got.shape == want.shape
+            _sets_equal_away_from_ties(got, want, ref.scores, num)
+            cache.set_next_positions(want)  # stay on the oracle's slots
+        o_ref, _, _ = ref.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        assert rel_err(o.float().cpu().view(B, num, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+        assert torch.equal(cache.token_pos.cpu(), ref.token_pos)
+        torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
+        pos += num
 
 
 def test_h2o_select_normalized(kvx, gpu):
@@ -291,7 +339,7 @@ def test_h2o_cache_steps_vs_oracle(gpu, quantized):
         if step > 0:
             # write to the oracle's slots so that the two caches stay comparable step after step
             # (the GPU's own choice is checked below)
-            cache._next_index[:B, :, :chunk] = index.to(torch.int32).to(gpu)
+            cache.set_next_positions(index)
         o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
         torch.cuda.synchronize()
         assert cache.input_pos == ref.input_pos
@@ -495,7 +543,7 @@ def test_chunk_over_dequantised_copy_equals_fused_dequantisation(gpu, bits):
         torch.testing.assert_close(copy.scores, fused.scores, rtol=1e-3, atol=1e-6)
         assert torch.equal(copy.k, fused.k) and torch.equal(copy.v, fused.v) and torch.equal(copy.token_pos, fused.token_pos)
         if copy._have_next:
-            fused._next_index.copy_(copy._next_index)  # keep the two in step where scores tie in the last bits
+            fused.set_next_positions(copy._next_index)  # keep the two in step where scores tie in the last bits
         pos += num
 
 

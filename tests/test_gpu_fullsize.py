@@ -155,8 +155,7 @@ def test_256_decode_steps_at_8_x_131072_slots(kvx, gpu):
     cache.token_pos.copy_(torch.arange(L, dtype=torch.int32, device=gpu).expand(B, Hkv, L))
     cache.batch_size, cache.current_length, cache.prefill_length = B, L, L
     cache._input_pos, cache._use_initial_rule = L, False
-    cache._next_index.zero_()  # step 0 writes slot 0
-    cache._have_next = True
+    cache.set_next_positions(torch.zeros((B, Hkv, 1), dtype=torch.int32, device=gpu))  # step 0 writes slot 0
     ones = torch.ones(B, Hkv, device=gpu)
     q = k = v = None
     for t in range(steps):

@@ -52,7 +52,7 @@ def _run_steps(gpu, cache, ref, q, k, v, n_prefill, steps):
         o_ref, w_ref, index = ref.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
         if had_choice:
             # evict the oracle's slots so that both caches stay comparable (the GPU's own choice was checked below)
-            cache._next_index[:B, :, :num] = index.to(torch.int32).to(gpu)
+            cache.set_next_positions(index)
         o = cache.forward(q[:, :, sl].to(gpu), k[:, :, sl].to(gpu), v[:, :, sl].to(gpu))
         torch.cuda.synchronize()
         assert cache.input_pos == ref.input_pos and cache.current_length == ref.current_length
@@ -67,9 +67,12 @@ def _run_steps(gpu, cache, ref, q, k, v, n_prefill, steps):
         if cache.q_errors is not None:
             torch.testing.assert_close(cache.q_errors.cpu(), ref.buffers["q_errors"], rtol=1e-5, atol=1e-6)
         if ref.next_index is not None:
-            kk_sel = cache._select_k
-            assert kk_sel == ref.next_index.shape[-1]
-            got = cache._next_index[:B].cpu().long()
+            # the cache chooses as many slots as the step after may need at once (one after a single token)
+            # and selects again when asked for more; the oracle keeps the reference's whole list
+            assert cache._select_k == ref.next_index.shape[-1]
+            kk_sel = cache._next_count
+            assert 1 <= kk_sel <= cache._select_k
+            got = cache._next_index[:B, :, :kk_sel].cpu().long()
             assert int(got.max()) < cache.cache_length - cache.grace_period, "a ring slot was chosen for eviction"
             _sets_equal_away_from_ties(got, ref.next_index, ref.compared, kk_sel)
         pos += num
@@ -314,7 +317,7 @@ def test_replay_log(gpu, kwargs):
         had_choice = ref.next_index is not None
         _, _, index = ref.forward(q[:, :, sl], k[:, :, sl], v[:, :, sl])
         if had_choice:
-            cache._next_index[:B, :, :num] = index.to(torch.int32).to(gpu)
+            cache.set_next_positions(index)
         cache.forward(q[:, :, sl].to(gpu), k[:, :, sl].to(gpu), v[:, :, sl].to(gpu), tokens[:, sl].to(gpu))
         if pos >= L:
             used.append(index)

@@ -384,7 +384,7 @@ def test_prefill_model_vs_oracle(gpu, quantized):
                 for h in range(cfg.n_query_groups):
                     a, r = set(got[0, h, :chunk].tolist()), set(want[0, h, :chunk].tolist())
                     assert len(a ^ r) <= 4, f"layer {li} head {h}: selections differ in {len(a ^ r)} slots"
-                cache._next_index[:B, :, :chunk] = want[:, :, :chunk].to(torch.int32).to(gpu)
+                cache.set_next_positions(want[:, :, :chunk])
                 forced.append(None)
         h_ref = ref.forward_chunk(sl, forced)
         h_gpu = model.forward_chunk(sl.to(gpu)).cpu()
