@@ -259,7 +259,7 @@ typedef struct kvx_cache_write_args {
   float* v_scale;
   int32_t* v_zp;
   int64_t qs_stride_b, qs_stride_h;
-  int32_t* token_pos; /* (B, Hkv, cache_len) */
+  int32_t* token_pos; /* (B, Hkv, cache_len), or NULL: rows only (DefaultKVCacheBuffers.set_slots, no position bookkeeping) */
   int64_t tp_stride_b, tp_stride_h;
   float* scores; /* (B, Hkv, cache_len) or NULL */
   int64_t sc_stride_b, sc_stride_h;

@@ -9,4 +9,4 @@ from .ops import (  # noqa: F401
     sdpa_prefill_fused,
     sdpa_prefill_fused_v2,
 )
-from .sdpa import HipSDPA, can_do_hip_sdpa, get_hip_sdpa  # noqa: F401
+from .sdpa import HipMultiHeadSelfAttention, HipSDPA, can_do_hip_sdpa, get_hip_sdpa  # noqa: F401

@@ -37,14 +37,15 @@ def _pad_head_size(query, key, value):
     return pad(query), pad(key), pad(value), diff
 
 
-def sdpa_check_args(query, key, value):
-    """keys_values/attention/sdpa_wrapper.py:24-47."""
+def sdpa_check_args(query, key, value, packed4: bool = False):
+    """keys_values/attention/sdpa_wrapper.py:24-47. ``packed4``: key / value are rows of the 4-bit store, two
+    codes per byte, so their last axis is half the head size."""
     if query.ndim != 4 or key.ndim != 4 or value.ndim != 4:
         raise ValueError("query, key, value must be 4D tensors")
     if key.shape != value.shape:
         raise ValueError("key, value must have same shape")
     batch_size, n_head, q_len, head_size = query.shape
-    if key.shape[0] != batch_size or key.shape[-1] != head_size:
+    if key.shape[0] != batch_size or key.shape[-1] != (head_size // 2 if packed4 else head_size):
         raise ValueError(f"key.shape = {key.shape}, must be ({batch_size}, _, _, {head_size})")
     _, n_query_groups, kv_len, _ = key.shape
     if not (0 < q_len <= kv_len):
@@ -86,7 +87,8 @@ class HipSDPA:
             raise ValueError("input_pos must be int scalar")
         if input_pos <= 0:
             raise ValueError("input_pos must be positive. Don't use for square prefill")
-        batch_size, n_head, n_query_groups, q_len, kv_len, head_size = sdpa_check_args(query, key, value)
+        packed4 = quant is not None and key.ndim == 4 and query.ndim == 4 and key.shape[-1] * 2 == query.shape[-1]
+        batch_size, n_head, n_query_groups, q_len, kv_len, head_size = sdpa_check_args(query, key, value, packed4)
         if token_positions is not None and token_positions.shape != key.shape[:-1]:
             raise ValueError(f"token_positions.shape = {token_positions.shape}, key.shape = {key.shape}: Not compatible")
         if scale_factor is None:
@@ -120,6 +122,47 @@ class HipSDPA:
         if head_size_diff is not None:
             attn_outputs = attn_outputs[:, :, :, :head_size]
         return attn_outputs, attn_weights
+
+
+class HipMultiHeadSelfAttention:
+    """The call surface of ``MultiHeadSelfAttention.__call__`` (keys_values/attention/base.py:287-380) for the
+    configurations the HIP kernels serve (no sliding window, no logit soft-capping): the cache passes the
+    queries and a ``KeysAndValues`` holder and gets ``(attn_outputs (B, q_len, n_head * hs), attn_weights)``.
+    ``input_pos`` 0 / None is the causal first chunk (no weights, keys_values/kvcache/base.py:567-581). A holder
+    of a quantised store (``key_codes`` / ``value_codes`` / ``quant``) is read in place by the kernels."""
+
+    def __init__(self, scale_factor: Optional[float] = None):
+        self.scale_factor = scale_factor
+        self._sdpa = get_hip_sdpa()
+
+    def __call__(self, query: torch.Tensor, k_and_v, block_idx: int = 0, input_pos: Optional[int] = None,
+                 return_attn_weights: bool = False, token_positions: Optional[torch.Tensor] = None):
+        is_causal = input_pos is None or input_pos == 0
+        if not is_causal and token_positions is None:
+            raise ValueError("token_positions must be given if input_pos > 0")
+        quant = getattr(k_and_v, "quant", None)
+        if quant is not None:
+            key, value = k_and_v.key_codes, k_and_v.value_codes
+        else:
+            key, value = k_and_v.keys(), k_and_v.values()
+        batch_size, _, q_len, head_size = query.shape
+        scale = self.scale_factor if self.scale_factor is not None else 1.0 / math.sqrt(head_size)
+        if is_causal:
+            if return_attn_weights:
+                raise ValueError("attention weights are not returned for the first chunk (input_pos = 0)")
+            if key.shape[2] != q_len:
+                raise ValueError(f"first chunk: kv_len = {key.shape[2]} must equal q_len = {q_len}")
+            if quant is None:
+                query, key, value, diff = _pad_head_size(query, key, value)
+            else:
+                diff = None
+            out, _, _ = ops.prefill_core(query, key, value, scale, 0, None, return_weights=False, output_transposed=True, quant=quant)
+            if diff is not None:
+                out = out[..., :head_size]
+            return out.reshape(batch_size, q_len, -1), None
+        out, w = self._sdpa.scaled_dot_product_attention(query, key, value, scale, input_pos, token_positions, return_attn_weights,
+                                                         output_transposed=True, quant=quant)
+        return out.reshape(batch_size, q_len, -1), w
 
 
 _hip_sdpa = None

@@ -251,7 +251,8 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4, KVX_ERR_UNSUPPORTED,
               "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
   KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
-  KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache && a->token_pos, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
+  KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
+  KVX_REQUIRE(a->token_pos || a->grace_num == 0, KVX_ERR_INVALID, "kvx_cache_write: the ring move needs token_pos");
   KVX_REQUIRE(aligned16(a->key) && aligned16(a->value) && mult8(a->key_stride_b) && mult8(a->key_stride_h) &&
                   mult8(a->key_stride_t) && mult8(a->value_stride_b) && mult8(a->value_stride_h) && mult8(a->value_stride_t),
               KVX_ERR_INVALID, "kvx_cache_write: key/value must be 16-byte aligned with strides that are multiples of 8");

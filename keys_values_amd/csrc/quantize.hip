@@ -543,7 +543,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
       put(krow, vrow, slot, mv, false);
     }
     if (mv && col == 0) {
-      a.token_pos[tp_row + slot] = a.input_pos - a.grace_period + j;
+      if (a.token_pos) a.token_pos[tp_row + slot] = a.input_pos - a.grace_period + j;
       if (a.scores) a.scores[sc_row + slot] = a.scores[sc_row + ring];
       if (a.v_norm) a.v_norm[sc_row + slot] = a.v_norm[sc_row + ring];
       if (a.q_errors) a.q_errors[sc_row + slot] = a.q_errors[sc_row + ring];
@@ -567,7 +567,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
         (uint32_t)slot;
   }
   if (ok && col == 0) {
-    a.token_pos[tp_row + wslot] = a.input_pos + src;
+    if (a.token_pos) a.token_pos[tp_row + wslot] = a.input_pos + src;
     if (a.scores) a.scores[sc_row + wslot] = 0.0f;
     if (a.v_norm) a.v_norm[sc_row + wslot] = vnorm;
     if (a.q_errors) a.q_errors[sc_row + wslot] = qerr;
