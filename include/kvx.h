@@ -11,7 +11,7 @@
  *
  * Conventions
  *   B      batch size                 Hq     query heads          Hkv   key/value heads
- *   G      Hq / Hkv (group size)      D      head size (64 or 128)
+ *   G      Hq / Hkv (group size)      D      head size (64, 128 or 256; quantised stores: 64 or 128)
  *   q_len  queries per call           kv_len cache slots visible to the call
  *   Tensors are addressed as base + b*stride_b + h*stride_h + t*stride_t + d with the head
  *   dimension contiguous; strides are in ELEMENTS of the tensor's own type. This covers both the
@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define KVX_VERSION 101 /* major*10000 + minor*100 + patch */
+#define KVX_VERSION 102 /* major*10000 + minor*100 + patch */
 
 enum kvx_status {
   KVX_OK = 0,
@@ -53,6 +53,9 @@ enum kvx_kv_dtype {
                       "torch-quantized8" store, keys_values/kvcache/quantize/pytorch.py:281-295);
                       rows are dequantised inside the kernel exactly as
                       keys_values/kvcache/quantize/pytorch.py:143-154,467-478 would, i.e. to bf16 */
+  KVX_KV_F16 = 3,  /* float16 rows; q and o are then float16 as well (the reference's extension takes float16 and
+                      bfloat16, keys_values/csrc/bindings.cpp:207, keys_values/attention/flashinfer_wrapper.py:311-319).
+                      Every other value of this enum goes with bfloat16 q and o. */
   KVX_KV_U4 = 2    /* the 4-bit store of the same quantiser ("torch-quantized4"): rows of D/2 bytes, byte j =
                       code[j] << 4 | code[j + D/2] (keys_values/kvcache/quantize/pytorch.py:384-393,457-465),
                       same per-row state; strides of k / v count bytes */
@@ -66,9 +69,9 @@ typedef struct kvx_sdpa_args {
   float sm_scale;      /* softmax scale, e.g. 1/sqrt(D) */
   int32_t num_splits;  /* KV splits for prefill/decode; 0 = library heuristic */
 
-  const void* q;       /* bf16 (B, Hq, q_len, D) by strides */
+  const void* q;       /* bf16 (fp16 with KVX_KV_F16) (B, Hq, q_len, D) by strides */
   int64_t q_stride_b, q_stride_h, q_stride_t;
-  const void* k;       /* bf16 or uint8 (B, Hkv, kv_len, D) by strides */
+  const void* k;       /* bf16, fp16 or uint8 (B, Hkv, kv_len, D) by strides */
   int64_t k_stride_b, k_stride_h, k_stride_t;
   const void* v;
   int64_t v_stride_b, v_stride_h, v_stride_t;
@@ -82,7 +85,7 @@ typedef struct kvx_sdpa_args {
   const int32_t* token_positions; /* (B, Hkv, kv_len) or NULL */
   int64_t tp_stride_b, tp_stride_h;
 
-  void* o;             /* bf16 (B, Hq, q_len, D) by strides */
+  void* o;             /* bf16 (fp16 with KVX_KV_F16) (B, Hq, q_len, D) by strides */
   int64_t o_stride_b, o_stride_h, o_stride_t;
   float* lse;          /* fp32 (B, q_len, Hq) contiguous, base 2; output of prefill/decode, input of score_sum */
   float* w;            /* fp32 (B, Hkv, kv_len) contiguous score-sums, or NULL */

@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libkvx.so")
 
 KVX_OK, KVX_ERR_INVALID, KVX_ERR_UNSUPPORTED, KVX_ERR_HIP, KVX_ERR_WORKSPACE = 0, 1, 2, 3, 4
-KVX_KV_BF16, KVX_KV_U8, KVX_KV_U4 = 0, 1, 2
+KVX_KV_BF16, KVX_KV_U8, KVX_KV_U4, KVX_KV_F16 = 0, 1, 2, 3
 
 
 class SdpaArgs(ctypes.Structure):

@@ -21,7 +21,9 @@ import torch
 
 from .. import _lib
 
-ALLOWED_HEAD_SIZES = (64, 128)  # keys_values/attention/flashinfer_wrapper.py:276 allows 256 as well
+ALLOWED_HEAD_SIZES = (64, 128, 256)  # keys_values/attention/flashinfer_wrapper.py:276
+QUANTIZED_HEAD_SIZES = (64, 128)    # the kernels that read codes
+ALLOWED_DTYPES = (torch.bfloat16, torch.float16)  # keys_values/attention/flashinfer_wrapper.py:311-319
 
 
 class QuantState(NamedTuple):
@@ -98,7 +100,7 @@ def _fill_common(a: _lib.SdpaArgs, query, key, value, scale, input_pos, token_po
         a.v_scale, a.v_zp = quant.v_scale.data_ptr(), quant.v_zp.data_ptr()
         a.qs_stride_b, a.qs_stride_h = quant.k_scale.stride(0), quant.k_scale.stride(1)
     else:
-        a.kv_dtype = _lib.KVX_KV_BF16
+        a.kv_dtype = _lib.KVX_KV_F16 if query.dtype == torch.float16 else _lib.KVX_KV_BF16
     if token_positions is not None:
         a.token_positions = token_positions.data_ptr()
         a.tp_stride_b, a.tp_stride_h = token_positions.stride(0), token_positions.stride(1)
@@ -110,11 +112,11 @@ def _row_len(D: int, key: torch.Tensor, quant) -> int:
 
 
 def _check_dtypes(query, key, value, quant):
-    if query.dtype != torch.bfloat16:
-        # the reference takes fp16 and bf16 (keys_values/attention/flashinfer_wrapper.py:311-319);
-        # the MFMA kernels here are bf16 only
-        raise NotImplementedError(f"query.dtype must be torch.bfloat16, got {query.dtype}")
-    want = torch.uint8 if quant is not None else torch.bfloat16
+    if query.dtype not in ALLOWED_DTYPES:
+        raise NotImplementedError(f"query.dtype must be torch.bfloat16 or torch.float16, got {query.dtype}")
+    if quant is not None and query.dtype != torch.bfloat16:
+        raise NotImplementedError("the quantised stores dequantise to bfloat16: query.dtype must be torch.bfloat16")
+    want = torch.uint8 if quant is not None else query.dtype
     for name, t in (("key", key), ("value", value)):
         if t is not None and t.dtype != want:
             raise NotImplementedError(f"{name}.dtype must be {want}, got {t.dtype}")
@@ -162,8 +164,8 @@ def prefill_core(
         raise ValueError(f"Must have 0 < q_len = {q_len} <= kv_len = {T}")
     if Hkv <= 0 or Hq % Hkv != 0:
         raise ValueError(f"n_head = {Hq} must be a positive multiple of n_query_groups = {Hkv}")
-    if D not in ALLOWED_HEAD_SIZES:
-        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES}")
+    if D not in (ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES):
+        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES}")
     token_positions = _token_positions_i32(token_positions, B, Hkv, T)
     dev = query.device
     lib = _lib.load()
@@ -203,8 +205,8 @@ def score_sum_core(query, key, lse, scale, input_pos, token_positions=None, quan
     Hkv, T = key.shape[1], key.shape[2]
     if lse.shape != (B, q_len, Hq) or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError(f"lse must be contiguous float32 {(B, q_len, Hq)}, got {tuple(lse.shape)} {lse.dtype}")
-    if D not in ALLOWED_HEAD_SIZES:
-        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES}")
+    if D not in (ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES):
+        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES}")
     token_positions = _token_positions_i32(token_positions, B, Hkv, T)
     dev = query.device
     with torch.cuda.device(dev):
@@ -243,8 +245,8 @@ def decode_core(
         raise ValueError(f"key.shape = {tuple(key.shape)}, value.shape = {tuple(value.shape)} do not fit query {tuple(query.shape)}")
     if Hkv <= 0 or Hq % Hkv != 0:
         raise ValueError(f"n_head = {Hq} must be a positive multiple of n_query_groups = {Hkv}")
-    if D not in ALLOWED_HEAD_SIZES:
-        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES}")
+    if D not in (ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES):
+        raise NotImplementedError(f"head size {D} not in {ALLOWED_HEAD_SIZES if quant is None else QUANTIZED_HEAD_SIZES}")
     dev = query.device
     lib = _lib.load()
     with torch.cuda.device(dev):

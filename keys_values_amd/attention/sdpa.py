@@ -20,7 +20,7 @@ _PAD_TO = ops.ALLOWED_HEAD_SIZES
 
 def can_do_hip_sdpa(head_size: int, dtype: torch.dtype, return_attn_weights: bool = False) -> bool:
     """Gate with the meaning of ``can_do_flashinfer`` (keys_values/attention/flashinfer_wrapper.py:311-319)."""
-    return dtype == torch.bfloat16 and 0 < head_size <= _PAD_TO[-1] and ops.is_available()
+    return dtype in ops.ALLOWED_DTYPES and 0 < head_size <= _PAD_TO[-1] and ops.is_available()
 
 
 def _pad_head_size(query, key, value):
@@ -93,11 +93,11 @@ class HipSDPA:
             raise ValueError(f"token_positions.shape = {token_positions.shape}, key.shape = {key.shape}: Not compatible")
         if scale_factor is None:
             scale_factor = 1.0 / math.sqrt(head_size)
-        if query.dtype != torch.bfloat16 or head_size > _PAD_TO[-1]:
+        if query.dtype not in ops.ALLOWED_DTYPES or head_size > _PAD_TO[-1]:
             raise NotImplementedError(
                 "HipSDPA needs these conditions:\n"
                 f"- head_size <= {_PAD_TO[-1]}, but is {head_size}\n"
-                f"- query.dtype == torch.bfloat16, but is {query.dtype}"
+                f"- query.dtype in (torch.bfloat16, torch.float16), but is {query.dtype}"
             )
         use_decode_kernel = q_len == 1
         if use_decode_kernel and kv_len == 1:
@@ -106,8 +106,8 @@ class HipSDPA:
             query, key, value, head_size_diff = _pad_head_size(query, key, value)
         else:
             head_size_diff = None
-            if head_size not in _PAD_TO:
-                raise NotImplementedError(f"quantised cache needs head_size in {_PAD_TO}")
+            if head_size not in ops.QUANTIZED_HEAD_SIZES:
+                raise NotImplementedError(f"quantised cache needs head_size in {ops.QUANTIZED_HEAD_SIZES}")
 
         if use_decode_kernel:
             # the single new token is the newest: it sees every slot, positions are not needed

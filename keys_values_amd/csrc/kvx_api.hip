@@ -49,9 +49,10 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
               "%s: sizes must be positive (B=%d Hq=%d Hkv=%d q_len=%d kv_len=%d)", who, a->B, a->Hq, a->Hkv, a->q_len,
               a->kv_len);
   KVX_REQUIRE(a->Hq % a->Hkv == 0, KVX_ERR_INVALID, "%s: Hq=%d must be a multiple of Hkv=%d", who, a->Hq, a->Hkv);
-  KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, a->D);
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4, KVX_ERR_UNSUPPORTED,
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4 || a->kv_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED,
               "%s: unknown kv_dtype %d", who, a->kv_dtype);
+  KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
+              "%s: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", who, a->D);
   const int row_elems = a->kv_dtype == KVX_KV_U4 ? a->D / 2 : a->D;  // elements of the cache's own type per row
   KVX_REQUIRE(a->input_pos >= 0, KVX_ERR_INVALID, "%s: input_pos=%d must be >= 0", who, a->input_pos);
   KVX_REQUIRE(a->sm_scale > 0.0f, KVX_ERR_INVALID, "%s: sm_scale must be positive", who);
@@ -70,7 +71,7 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
                 "%s: o must be 16-byte aligned with strides that are multiples of 8 elements", who);
     KVX_REQUIRE(a->v_stride_t >= row_elems, KVX_ERR_INVALID, "%s: bad v slot stride", who);
   }
-  if (a->kv_dtype != KVX_KV_BF16) {
+  if (!kv_is_plain(a->kv_dtype)) {
     KVX_REQUIRE(a->k_scale && a->k_zp, KVX_ERR_INVALID, "%s: quantised cache needs k_scale and k_zp", who);
     if (need_v_o) KVX_REQUIRE(a->v_scale && a->v_zp, KVX_ERR_INVALID, "%s: quantised cache needs v_scale and v_zp", who);
   }
@@ -247,9 +248,10 @@ int kvx_dequantize_blocks(const kvx_block_quant_args* a, void* stream) {
 int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");
-  KVX_REQUIRE(a->D == 64 || a->D == 128, KVX_ERR_UNSUPPORTED, "kvx_cache_write: head size %d not in {64, 128}", a->D);
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4, KVX_ERR_UNSUPPORTED,
+  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4 || a->kv_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED,
               "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
+  KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
+              "kvx_cache_write: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a->D);
   KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
   KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
   KVX_REQUIRE(a->token_pos || a->grace_num == 0, KVX_ERR_INVALID, "kvx_cache_write: the ring move needs token_pos");
@@ -259,7 +261,7 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(aligned16(a->k_cache) && aligned16(a->v_cache) && mult8(a->kc_stride_b) && mult8(a->kc_stride_h) &&
                   mult8(a->kc_stride_t) && mult8(a->vc_stride_b) && mult8(a->vc_stride_h) && mult8(a->vc_stride_t),
               KVX_ERR_INVALID, "kvx_cache_write: caches must be 16-byte aligned with strides that are multiples of 8");
-  if (a->kv_dtype != KVX_KV_BF16)
+  if (!kv_is_plain(a->kv_dtype))
     KVX_REQUIRE(a->k_scale && a->k_zp && a->v_scale && a->v_zp, KVX_ERR_INVALID, "kvx_cache_write: quantised cache needs scale / zero-point arrays");
   KVX_REQUIRE((int64_t)a->input_pos + a->num < INT32_MAX && a->input_pos >= 0, KVX_ERR_INVALID, "kvx_cache_write: bad input_pos");
   KVX_REQUIRE(a->grace_num >= 0 && a->grace_num <= a->num, KVX_ERR_INVALID, "kvx_cache_write: grace_num=%d must be in [0, num=%d]", a->grace_num, a->num);
@@ -271,7 +273,7 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   }
   KVX_REQUIRE(!a->replay_log || (a->log_blocksize > 0 && a->log_pos >= 0), KVX_ERR_INVALID,
               "kvx_cache_write: replay log needs log_blocksize > 0 and log_pos >= 0");
-  KVX_REQUIRE(!a->q_errors || a->kv_dtype != KVX_KV_BF16, KVX_ERR_INVALID, "kvx_cache_write: q_errors needs a quantised cache");
+  KVX_REQUIRE(!a->q_errors || !kv_is_plain(a->kv_dtype), KVX_ERR_INVALID, "kvx_cache_write: q_errors needs a quantised cache");
   return launch_cache_write(*a, (hipStream_t)stream);
 }
 

@@ -82,6 +82,38 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
+// ---- the two 16-bit element types of q / k / v / o: bf16 and, with KVX_KV_F16, fp16 -----------------
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// plain rows of the query's own type (no codes)
+constexpr bool kv_is_plain(int kv) { return kv == KVX_KV_BF16 || kv == KVX_KV_F16; }
+
+// D = A B + C on one 32x32x16 tile, operands as four dwords of eight 16-bit values
+template <bool F16>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(u32x4_t a, u32x4_t b, f32x16_t c) {
+  if constexpr (F16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// two fp32 -> packed pair of the element type, round to nearest even (lo = a, hi = b)
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_pair(float a, float b) {
+  if constexpr (F16) {
+    const f16x2_t r = __builtin_convertvector(f32x2_t{a, b}, f16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    return pack_bf16(a, b);
+  }
+}
+
+// acc + x.lo * y.lo + x.hi * y.hi on packed pairs of the element type
+template <bool F16>
+__device__ __forceinline__ float dot2_acc(uint32_t x, uint32_t y, float acc) {
+  if constexpr (F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, x), __builtin_bit_cast(f16x2_t, y), acc, false);
+  else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, y), acc, false);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -416,18 +416,27 @@ __device__ __forceinline__ float row_sum(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
-  if constexpr (LPR == 16)
+  if constexpr (LPR >= 16)
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+  if constexpr (LPR == 32) v += __shfl_xor(v, 16, 64);  // the other DPP row of the group
   return v;
 }
 
-// |row|_2 of a bf16 row spread over LPR lanes, accumulated in fp32.
-template <int LPR>
+// |row|_2 of a bf16 (F16: fp16) row spread over LPR lanes, accumulated in fp32.
+template <int LPR, bool F16 = false>
 __device__ __forceinline__ float row_norm(u32x4_t raw) {
   float ss = 0.0f;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const float a = bf16_lo(raw[e]), b = bf16_hi(raw[e]);
+    float a, b;
+    if constexpr (F16) {
+      const f16x2_t hv = __builtin_bit_cast(f16x2_t, (uint32_t)raw[e]);
+      a = (float)hv[0];
+      b = (float)hv[1];
+    } else {
+      a = bf16_lo(raw[e]);
+      b = bf16_hi(raw[e]);
+    }
     ss += a * a;
     ss += b * b;
   }
@@ -459,7 +468,7 @@ __device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, flo
 // read's data is consumed before the write is issued.
 template <int D, int KV>
 __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
-  constexpr bool U8 = KV != KVX_KV_BF16;  // a quantised store: codes + row state
+  constexpr bool U8 = !kv_is_plain(KV);  // a quantised store: codes + row state
   constexpr bool U4 = KV == KVX_KV_U4;    // two codes per byte: only the lanes of the first half of a row store
   constexpr int LPR = D / 8;
   const int64_t gid = (int64_t)blockIdx.x * NTHREADS + threadIdx.x;
@@ -560,7 +569,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
     qerr = put(kr, vr, wslot, ok, a.q_errors != nullptr);
   }
   float vnorm = 0.0f;
-  if (a.v_norm) vnorm = row_norm<LPR>(vr);  // uniform branch: every lane takes part in the reduction
+  if (a.v_norm) vnorm = row_norm<LPR, KV == KVX_KV_F16>(vr);  // uniform branch: every lane takes part in the reduction
   if (live && col == 0 && a.replay_log) {  // the slot as consumed, valid or not: the log mirrors index
     const int64_t lp = a.log_pos + j;
     a.replay_log[(lp / a.log_blocksize) * a.log_stride_block + b * a.log_stride_b + hh * a.log_stride_h + lp % a.log_blocksize] =
@@ -652,13 +661,18 @@ int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st) {
   const int64_t total = (int64_t)a.B * a.Hkv * a.num * (a.D / 8);
   if (total == 0) return KVX_OK;
   const unsigned grid = (unsigned)((total + NTHREADS - 1) / NTHREADS);
-  if (a.D == 128) {
+  if (a.D == 256) {  // plain rows only (checked by the caller)
+    if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<256, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else hipLaunchKernelGGL((cache_write_kernel<256, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  } else if (a.D == 128) {
     if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
     else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
     else hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
   } else {
     if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
     else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    else if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
     else hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
   }
   KVX_HIP(hipGetLastError());

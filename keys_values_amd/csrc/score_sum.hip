@@ -141,7 +141,8 @@ struct QLoader {
 };
 
 template <int D, int KV>
-__global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParams p) {
+__global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
+  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q and k
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,19 +154,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
   const int key0 = blockIdx.y * BK + wave * NW;
 
   // K fragments (B operand): lane holds key column n of tile nt, d = 16 j + 8 h .. +8
-  bf16x8_t kf[2][D / 16];
+  u32x4_t kf[2][D / 16];
   int32_t tpk[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
     const int key = key0 + nt * 32 + n;
     const bool ok = key < p.kv_len;
     tpk[nt] = ok ? (p.tp ? p.tp[b * p.tp_sb + kvh * p.tp_sh + key] : key) : INT_MAX;
-    if constexpr (KV == KVX_KV_BF16) {
+    if constexpr (kv_is_plain(KV)) {
       const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st;
 #pragma unroll
       for (int j = 0; j < D / 16; ++j) {
         u32x4_t t = ok ? *(const u32x4_t*)(kp + 16 * j + 8 * h) : u32x4_t{0, 0, 0, 0};
-        kf[nt][j] = as_bf16x8(t);
+        kf[nt][j] = t;
       }
     } else {
       const uint8_t* kp = (const uint8_t*)p.k + b * p.k_sb + kvh * p.k_sh + (int64_t)key * p.k_st;
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
         } else {
           cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
         }
-        kf[nt][j] = as_bf16x8(dequant_words(cc[0], cc[1], zp, sc));
+        kf[nt][j] = dequant_words(cc[0], cc[1], zp, sc);
       }
     }
   }
@@ -207,9 +208,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void score_sum_kernel(const ScoreParam
       for (int nt = 0; nt < 2; ++nt) {
         if (j == 0) {
           const f32x16_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], zero, 0, 0, 0);
+          s[nt] = mfma_32x32x16<F16>(qq, kf[nt][j], zero);
         } else {
-          s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(qq), kf[nt][j], s[nt], 0, 0, 0);
+          s[nt] = mfma_32x32x16<F16>(qq, kf[nt][j], s[nt]);
         }
       }
     }
@@ -334,13 +335,17 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
   if (a.D == 128) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st);
     return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
   }
   if (a.D == 64) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, st);
     return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
   }
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128}", a.D);
+  if (a.D == 256 && kv_is_plain(a.kv_dtype))
+    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, st) : launch_t<256, KVX_KV_BF16>(p, st);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
 }
 
 }  // namespace kvx

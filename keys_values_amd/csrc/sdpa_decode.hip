@@ -57,8 +57,9 @@ __device__ __forceinline__ float dpp_add(float x) {
 }
 template <int LPR>
 __device__ __forceinline__ float row_group_sum(float x) {
-  static_assert(LPR == 16 || LPR == 8, "row groups of 8 or 16 lanes");
-  if constexpr (LPR == 16) {
+  static_assert(LPR == 32 || LPR == 16 || LPR == 8, "row groups of 8, 16 or 32 lanes");
+  if constexpr (LPR == 32) x += __shfl_xor(x, 16, 64);  // the other DPP row of the group
+  if constexpr (LPR >= 16) {
     x = dpp_add<0x128>(x);  // row_ror:8
     x = dpp_add<0x124>(x);  // row_ror:4
   } else {
@@ -74,6 +75,7 @@ constexpr float kRescaleSlack = 8.0f;  // the running maximum moves only when a 
 
 template <int D, int G, int KV>
 __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p) {
+  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q, k, v, o
   constexpr int LPR = D / 8;     // lanes per row: a lane owns 8 consecutive d
   constexpr int RPI = 64 / LPR;  // rows per load instruction of a wavefront
   constexpr int U = 4;           // load instructions per step and tensor (even: rows pair up for dot2)
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     for (int e = 0; e < 4; ++e) qv[g][e] = t[e];
   }
   // Rows are addressed as a uniform base plus a 32-bit byte offset (the host checks the range).
-  constexpr bool U8 = KV != KVX_KV_BF16;  // codes + row state (8-bit or 4-bit store)
+  constexpr bool U8 = !kv_is_plain(KV);  // codes + row state (8-bit or 4-bit store)
   constexpr bool U4 = KV == KVX_KV_U4;
   constexpr int ES = U8 ? 1 : 2;
   const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t kw = kx[e];  // a bit_cast applied to the vector element itself reads element 0
-          a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, kw), __builtin_bit_cast(bf16x2_t, qv[g][e]), a, false);
+          a = dot2_acc<F16>(kw, qv[g][e], a);
         }
         a = row_group_sum<LPR>(a) * p.c;
         s[u][g] = valid ? a : -INFINITY;
@@ -211,22 +213,22 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
         xa = dq8(xa[0], xa[1], r.vz[u], r.vs[u]);
         xb = dq8(xb[0], xb[1], r.vz[u + 1], r.vs[u + 1]);
       }
-      bf16x2_t pg[G];
+      uint32_t pg[G];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const float pa = fast_exp2(s[u][g] - m_run[g]);
         const float pb = fast_exp2(s[u + 1][g] - m_run[g]);
         l_run[g] += pa + pb;
-        pg[g] = __builtin_bit_cast(bf16x2_t, pack_bf16(pa, pb));
+        pg[g] = pack_pair<F16>(pa, pb);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bf16x2_t lo = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(xb[e], xa[e], 0x05040100u));
-        const bf16x2_t hi = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(xb[e], xa[e], 0x07060302u));
+        const uint32_t lo = __builtin_amdgcn_perm(xb[e], xa[e], 0x05040100u);
+        const uint32_t hi = __builtin_amdgcn_perm(xb[e], xa[e], 0x07060302u);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-          acc[g][2 * e] = __builtin_amdgcn_fdot2_f32_bf16(lo, pg[g], acc[g][2 * e], false);
-          acc[g][2 * e + 1] = __builtin_amdgcn_fdot2_f32_bf16(hi, pg[g], acc[g][2 * e + 1], false);
+          acc[g][2 * e] = dot2_acc<F16>(lo, pg[g], acc[g][2 * e]);
+          acc[g][2 * e + 1] = dot2_acc<F16>(hi, pg[g], acc[g][2 * e + 1]);
         }
       }
     }
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 
 // Combine the splits of one (b, query head): 4 groups of D threads each take a quarter of the
 // splits, then the groups are added through LDS. Also produces the base-2 log-sum-exp.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams p) {
   __shared__ float red[4][D + 1];
   __shared__ float sM;
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
     const float l4 = red[0][D] + red[1][D] + red[2][D] + red[3][D];
     const float r = a4 / l4;
     const float other = __shfl_xor(r, 1, 64);
-    if ((d & 1) == 0) *(uint32_t*)(p.o + b * p.o_sb + hqi * p.o_sh + d) = pack_bf16(r, other);
+    if ((d & 1) == 0) *(uint32_t*)(p.o + b * p.o_sb + hqi * p.o_sh + d) = pack_pair<F16>(r, other);
     if (d == 0) {
       const float lse = M + fast_log2(l4);
       p.lse_ws[bh] = lse;
@@ -475,11 +477,15 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
 template <int D, int G>
 int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
-  if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p);
-  else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p);
-  else hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p);
+  if constexpr (D <= 128) {
+    if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p);
+    else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p);
+  }
+  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p);
+  else if (kv == KVX_KV_BF16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p);
   KVX_HIP(hipGetLastError());
-  hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
+  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_merge_kernel<D, true>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
+  else hipLaunchKernelGGL((decode_merge_kernel<D, false>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
   KVX_HIP(hipGetLastError());
   const dim3 wgrid((p.kv_len + 4095) / 4096, p.Hkv, p.B);
   if (hh) {
@@ -515,7 +521,7 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   const Plan pl = make_plan(a, hh != nullptr);
   KVX_REQUIRE(a.workspace && a.workspace_bytes >= pl.total, KVX_ERR_WORKSPACE,
               "kvx_sdpa_decode: workspace of %zu bytes needed, %zu given", pl.total, a.workspace_bytes);
-  const int64_t es = a.kv_dtype != KVX_KV_BF16 ? 1 : 2;
+  const int64_t es = kv_is_plain(a.kv_dtype) ? 2 : 1;
   KVX_REQUIRE((int64_t)a.kv_len * a.k_stride_t * es < (1ll << 32) && (int64_t)a.kv_len * a.v_stride_t * es < (1ll << 32), KVX_ERR_UNSUPPORTED,
               "kvx_sdpa_decode: one (batch, head) row set of K or V must span less than 4 GiB (kv_len %d, slot strides %lld / %lld)",
               a.kv_len, (long long)a.k_stride_t, (long long)a.v_stride_t);
@@ -543,7 +549,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   if (a.D == 128) return launch_d<128>(p, pl.G, a.kv_dtype, hh, st);
   if (a.D == 64) return launch_d<64>(p, pl.G, a.kv_dtype, hh, st);
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128}", a.D);
+  if (a.D == 256 && kv_is_plain(a.kv_dtype)) return launch_d<256>(p, pl.G, a.kv_dtype, hh, st);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
 }
 
 }  // namespace kvx

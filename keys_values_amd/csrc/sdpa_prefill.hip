@@ -31,7 +31,7 @@ constexpr float kSlackLog2 = 8.0f;  // see the running-maximum update in the ker
 // Wavefronts per workgroup, 32 rows each. The uint8 cache takes 8: a tile is dequantised once per
 // workgroup, so twice the rows halve that vector work per row (-13 % kernel time); for bf16 tiles the
 // two sizes run alike and the smaller one leaves more workgroups for short chunks.
-constexpr int nwaves(int kv) { return kv != 0 ? 8 : 4; }  // kv: enum kvx_kv_dtype
+constexpr int nwaves(int kv) { return kv_is_plain(kv) ? 4 : 8; }  // kv: enum kvx_kv_dtype
 constexpr int BN = 64;   // keys per tile
 
 struct PrefillParams {
@@ -63,7 +63,7 @@ struct PrefillParams {
 //   V, ds_read_b64_tr_b16:  4 consecutive rows x chunks {c, c + 1}   -> bits 1..2 of swz_v distinct over r % 4
 // Both depend on r % 16 only, so they repeat for the row groups a wavefront loads (16 or 32 rows apart).
 template <int CPR>
-__device__ __forceinline__ int swz_k(int r) { return CPR == 16 ? (r & 15) : ((r >> 1) & 7); }
+__device__ __forceinline__ int swz_k(int r) { return CPR >= 16 ? (r & 15) : ((r >> 1) & 7); }
 template <int CPR>
 __device__ __forceinline__ int swz_v(int r) { return ((r & 3) << 1) | ((r >> 2) & 1); }
 
@@ -124,11 +124,11 @@ __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp
 // tile ahead like the DMA), are dequantised to bf16 and written to the same LDS layout.
 template <int D, int KV>
 struct Loader {
-  static constexpr bool U8 = KV != KVX_KV_BF16;  // codes through registers (8-bit or 4-bit store)
+  static constexpr bool U8 = !kv_is_plain(KV);  // codes through registers (8-bit or 4-bit store)
   static constexpr bool U4 = KV == KVX_KV_U4;
   static constexpr int CPR = D / 8;
   static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
-  static constexpr int NWAVES = nwaves(U8);
+  static constexpr int NWAVES = nwaves(KV);
   static constexpr int NTHREADS = 64 * NWAVES;
   static constexpr int NI = BN / RPW / NWAVES;     // instructions per wavefront per operand: 4 / 2
   static constexpr int ESZ = U8 ? 1 : 2;
@@ -142,7 +142,8 @@ struct Loader {
   uint32_t koff, voff;          // byte offset of this lane's chunk of row group 0 inside a tile (source side swizzled)
   int64_t k_tile_bytes, v_tile_bytes, k_st, v_st;
   int64_t k_step, v_step;       // bytes between this wavefront's consecutive row groups (NWAVES RPW rows)
-  int wave, lane, kv_len, rl, cgk, cgv;
+  int wave, lane, kv_len, rl;
+  int cgk[NI], cgv[NI];         // the source chunk that belongs at this lane's LDS position, per row group
   int shk, shv;                 // 4-bit store: nibble of this lane's K / V chunk (4 = high)
   uint32_t lds_k, lds_v;        // LDS addresses of the K and V buffers (wavefront-uniform)
   uint32_t lds_kw, lds_vw;      // the same plus this wavefront's row-group offset
@@ -175,23 +176,27 @@ struct Loader {
     tp = p.tp ? p.tp + b * p.tp_sb + kvh * p.tp_sh : nullptr;
     k_tile_bytes = (int64_t)BN * p.k_st * ESZ;
     v_tile_bytes = (int64_t)BN * p.v_st * ESZ;
-    // row groups of one wavefront are NWAVES RPW rows apart, a multiple of 16: the XOR keys and with them
-    // the source chunks are the same for all of them
-    const int r = row_of(0);
-    cgk = (lane % CPR) ^ swz_k<CPR>(r);  // the chunk that belongs at LDS position lane % CPR of row r
-    cgv = (lane % CPR) ^ swz_v<CPR>(r);
-    koff = (uint32_t)(r * p.k_st * ESZ + chunk_off(cgk));
-    voff = (uint32_t)(r * p.v_st * ESZ + chunk_off(cgv));
-    shk = u4_shift<D>(cgk);
-    shv = u4_shift<D>(cgv);
+    // row groups of one wavefront are NWAVES RPW rows apart: a multiple of 16 (the XOR keys and with them the
+    // source chunks are then the same for all of them) except for D = 256 with four wavefronts (8 rows apart)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = row_of(i);
+      cgk[i] = (lane % CPR) ^ swz_k<CPR>(r);  // the chunk that belongs at LDS position lane % CPR of row r
+      cgv[i] = (lane % CPR) ^ swz_v<CPR>(r);
+    }
+    const int r0 = row_of(0);
+    koff = (uint32_t)(r0 * p.k_st * ESZ + chunk_off(cgk[0]));
+    voff = (uint32_t)(r0 * p.v_st * ESZ + chunk_off(cgv[0]));
+    shk = u4_shift<D>(cgk[0]);  // quantised stores: D <= 128, all row groups share their chunk
+    shv = u4_shift<D>(cgv[0]);
     k_step = (int64_t)NWAVES * RPW * p.k_st * ESZ;
     v_step = (int64_t)NWAVES * RPW * p.v_st * ESZ;
     lds_kw = lds_k + (uint32_t)(wave * RPW * CPR * 16);
     lds_vw = lds_v + (uint32_t)(wave * RPW * CPR * 16);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      koffs[i] = koff + (uint32_t)(i * k_step);
-      voffs[i] = voff + (uint32_t)(i * v_step);
+      koffs[i] = (uint32_t)(row_of(i) * p.k_st * ESZ + chunk_off(cgk[i]));
+      voffs[i] = (uint32_t)(row_of(i) * p.v_st * ESZ + chunk_off(cgv[i]));
     }
   }
 
@@ -227,7 +232,7 @@ struct Loader {
       for (int i = 0; i < NI; ++i) {
         if constexpr (!U8) {
           const uint32_t dst = (IS_K ? lds_k : lds_v) + (uint32_t)((buf * BN + (NWAVES * i + wave) * RPW) * CPR * 16);
-          dma16(tb + i * step, off0, dst);
+          dma16(tb, IS_K ? koffs[i] : voffs[i], dst);
         } else {
           const int key = key0 + row_of(i);
           const u32x2_t c = *(const u32x2_t*)(tb + i * step + off0);
@@ -241,7 +246,7 @@ struct Loader {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int key = min(key0 + row_of(i), kv_len - 1);
-        const uint32_t off = (uint32_t)((int64_t)(key - key0) * st * ESZ) + chunk_off(IS_K ? cgk : cgv);
+        const uint32_t off = (uint32_t)((int64_t)(key - key0) * st * ESZ) + chunk_off(IS_K ? cgk[i] : cgv[i]);
         if constexpr (!U8) {
           const uint32_t dst = (IS_K ? lds_k : lds_v) + (uint32_t)((buf * BN + (NWAVES * i + wave) * RPW) * CPR * 16);
           dma16(tb, off, dst);
@@ -301,7 +306,8 @@ struct Loader {
 };
 
 template <int D, int KV>
-__global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(64 * nwaves(KV), (kv_is_plain(KV) && D <= 128) ? 2 : 1) void sdpa_prefill_kernel(const PrefillParams p) {
+  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q, k, v, o
   constexpr int BM = 32 * nwaves(KV);  // rows per workgroup
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;  // k-steps of the first product
@@ -329,13 +335,13 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
   const int qpos_min_w = p.input_pos + min(row0w, p.R - 1) / p.G;
 
   // Q fragments (B operand): lane holds row n, d = 16 j + 8 h .. +8
-  bf16x8_t qf[KS];
+  u32x4_t qf[KS];
   {
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)(kvh * p.G + g) * p.q_sh + (int64_t)qi * p.q_st;
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
       u32x4_t t = row_ok ? *(const u32x4_t*)(qp + 16 * j + 8 * h) : u32x4_t{0, 0, 0, 0};
-      qf[j] = as_bf16x8(t);
+      qf[j] = t;
     }
   }
 
@@ -403,7 +409,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const u32x4_t kk = *(const u32x4_t*)(kb + ka[j] + mt * 32 * CPR * 16);
-        s[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kk), qf[j], s[mt], 0, 0, 0);
+        s[mt] = mfma_32x32x16<F16>(kk, qf[j], s[mt]);
       }
   };
   // mask (only tiles that hold a position some row of this wavefront may not see)
@@ -439,11 +445,11 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
 #pragma unroll
     for (int i = FIRST_I; i < FIRST_I + COUNT; ++i) {
       const int mt = i / (2 * DT), j = (i / DT) % 2, dt = i % DT;
-      const bf16x8_t pf = as_bf16x8(u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]});
+      const u32x4_t pf = u32x4_t{pb[mt][4 * j], pb[mt][4 * j + 1], pb[mt][4 * j + 2], pb[mt][4 * j + 3]};
       const int rb = (32 * mt + 16 * j) * CPR * 16;
       const u32x2_t lo = lds_read_tr16(vl[dt] + rb);
       const u32x2_t hi = lds_read_tr16(vl[dt] + rb + 8 * CPR * 16);
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]}), pf, o[dt], 0, 0, 0);
+      o[dt] = mfma_32x32x16<F16>(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pf, o[dt]);
     }
   };
   auto pv = [&](const uint32_t (&pb)[2][8], int buf) {
@@ -473,7 +479,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr int cur = decltype(cur_tag)::value;
     // STEADY: tiles t and t + 1 are full and tile t + 1 belongs to this walk
-    constexpr bool STEADY = decltype(steady_tag)::value && KV == KVX_KV_BF16;
+    constexpr bool STEADY = decltype(steady_tag)::value && kv_is_plain(KV);
     uint32_t (&pb_prev)[2][8] = pbs[cur ^ 1];
     uint32_t (&pb)[2][8] = pbs[cur];
     const bool has1 = STEADY || t + 1 < tile_end;
@@ -519,7 +525,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
         const float p1 = fast_exp2(fmaf(s[mt][i + 1], p.c, -mc));
         rs0 += p0;
         rs1 += p1;
-        pb[mt][i >> 1] = pack_bf16(p0, p1);
+        pb[mt][i >> 1] = pack_pair<F16>(p0, p1);
       }
     l += rs0 + rs1;
     if constexpr (!FIRST) {
@@ -597,8 +603,8 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
           u32x2_t w2;
-          w2[0] = pack_bf16(o[dt][4 * a] * inv, o[dt][4 * a + 1] * inv);
-          w2[1] = pack_bf16(o[dt][4 * a + 2] * inv, o[dt][4 * a + 3] * inv);
+          w2[0] = pack_pair<F16>(o[dt][4 * a] * inv, o[dt][4 * a + 1] * inv);
+          w2[1] = pack_pair<F16>(o[dt][4 * a + 2] * inv, o[dt][4 * a + 3] * inv);
           *(u32x2_t*)(op + dt * 32 + 8 * a + 4 * h) = w2;
         }
       if (p.lse && h == 0) p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] = m * p.c + fast_log2(lt);
@@ -623,7 +629,7 @@ __global__ __launch_bounds__(64 * nwaves(KV), KV != 0 ? 1 : 2) void sdpa_prefill
 }
 
 // Combine the per-split partials of a row: one workgroup of D/4 threads... one thread per 4 d.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(const PrefillParams p) {
   constexpr int TPR = D / 4;              // threads per row
   constexpr int ROWS = 256 / TPR;         // rows per workgroup
@@ -650,8 +656,8 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(const PrefillPa
   const float inv = L > 0.0f ? 1.0f / L : 0.0f;
   uint16_t* op = p.o + b * p.o_sb + (int64_t)(kvh * p.G + g) * p.o_sh + (int64_t)qi * p.o_st + dq * 4;
   u32x2_t w2;
-  w2[0] = pack_bf16(acc[0] * inv, acc[1] * inv);
-  w2[1] = pack_bf16(acc[2] * inv, acc[3] * inv);
+  w2[0] = pack_pair<F16>(acc[0] * inv, acc[1] * inv);
+  w2[1] = pack_pair<F16>(acc[2] * inv, acc[3] * inv);
   *(u32x2_t*)op = w2;
   if (p.lse && dq == 0) p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] = Mu + fast_log2(L);
 }
@@ -661,7 +667,7 @@ int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
   // Aim for one resident round of workgroups (2 per compute unit, 1 with the uint8 cache): more
   // splits only add partials to write, merge and re-read. At least 8 key tiles per split.
   const int64_t base = (int64_t)a.B * a.Hkv * m_blocks;
-  const int target = (a.kv_dtype != KVX_KV_BF16 ? 1 : 2) * num_cus();
+  const int target = ((kv_is_plain(a.kv_dtype) && a.D <= 128) ? 2 : 1) * num_cus();
   int s = (int)((target + base - 1) / base);
   s = max(1, min(s, num_tiles / 8));
   return max(1, min(s, 64));
@@ -717,7 +723,7 @@ int launch_t(PrefillParams& p, hipStream_t st) {
   if (p.num_splits > 1) {
     constexpr int ROWS = 256 / (D / 4);
     const int64_t total_rows = (int64_t)p.B * p.Hkv * p.R;
-    hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D>), dim3((unsigned)((total_rows + ROWS - 1) / ROWS)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D, KV == KVX_KV_F16>), dim3((unsigned)((total_rows + ROWS - 1) / ROWS)), dim3(256), 0, st, p);
     KVX_HIP(hipGetLastError());
   }
   return KVX_OK;
@@ -744,13 +750,17 @@ int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {
   }
   if (a.D == 128) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st);
     return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
   }
   if (a.D == 64) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, st);
     return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
   }
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_prefill: head size %d not in {64, 128}", a.D);
+  if (a.D == 256 && kv_is_plain(a.kv_dtype))
+    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, st) : launch_t<256, KVX_KV_BF16>(p, st);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_prefill: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
 }
 
 }  // namespace kvx

@@ -174,8 +174,9 @@ class HipKVCacheBuffers(KVCacheBuffers):
         super().__init__(params, cache_length)
         if num_bits not in (None, 4, 8):
             raise ValueError(f"num_bits = {num_bits}, must be None, 4 or 8")
-        if params.head_size not in ops.ALLOWED_HEAD_SIZES:
-            raise NotImplementedError(f"head_size = {params.head_size} not in {ops.ALLOWED_HEAD_SIZES}")
+        sizes = ops.ALLOWED_HEAD_SIZES if num_bits is None else ops.QUANTIZED_HEAD_SIZES
+        if params.head_size not in sizes:
+            raise NotImplementedError(f"head_size = {params.head_size} not in {sizes}")
         if self.dtype is not None and self.dtype not in (torch.bfloat16, torch.float16):
             raise NotImplementedError(f"dtype {self.dtype}: the kernels take bfloat16 or float16 rows")
         if num_bits is not None and self.dtype not in (None, torch.bfloat16):
@@ -276,7 +277,7 @@ class HipKVCacheBuffers(KVCacheBuffers):
             value = value.contiguous()
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, d, self.cache_length
-        a.kv_dtype = {None: _lib.KVX_KV_BF16, 8: _lib.KVX_KV_U8, 4: _lib.KVX_KV_U4}[self.num_bits]
+        a.kv_dtype = {None: _lib.KVX_KV_F16 if self.dtype == torch.float16 else _lib.KVX_KV_BF16, 8: _lib.KVX_KV_U8, 4: _lib.KVX_KV_U4}[self.num_bits]
         a.index, a.index_stride_b, a.index_stride_h = index.data_ptr(), index.stride(0), index.stride(1)
         a.key, a.key_stride_b, a.key_stride_h, a.key_stride_t = key.data_ptr(), key.stride(0), key.stride(1), key.stride(2)
         a.value, a.value_stride_b, a.value_stride_h, a.value_stride_t = value.data_ptr(), value.stride(0), value.stride(1), value.stride(2)

@@ -123,10 +123,12 @@ class H2OKVCache:
             raise TypeError("the quantisation-error policy needs the quantised store")
         if not (0 <= combination_constant <= 1):  # keys_values/kvcache/qh2o.py:97-100
             raise ValueError(f"combination_constant = {combination_constant}, must be in [0, 1]")
-        if params.dtype not in (None, torch.bfloat16):
-            raise NotImplementedError(f"cache dtype {params.dtype}: the kernels take bfloat16")
-        if params.head_size not in (64, 128):
-            raise NotImplementedError(f"head_size = {params.head_size} not in (64, 128)")
+        if params.dtype not in (None, torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"cache dtype {params.dtype}: the kernels take bfloat16 or float16")
+        if quantized and params.dtype == torch.float16:
+            raise NotImplementedError("the quantised stores dequantise to bfloat16")
+        if params.head_size not in (ops.QUANTIZED_HEAD_SIZES if quantized else ops.ALLOWED_HEAD_SIZES):
+            raise NotImplementedError(f"head_size = {params.head_size} not in {ops.QUANTIZED_HEAD_SIZES if quantized else ops.ALLOWED_HEAD_SIZES}")
         if params.n_head % params.n_query_groups != 0:
             raise ValueError("n_head must be a multiple of n_query_groups")
         self.params = params
@@ -135,7 +137,7 @@ class H2OKVCache:
         self.n_head = params.n_head
         self.cache_length = params.cache_length
         self.head_size = params.head_size
-        self.dtype = torch.bfloat16
+        self.dtype = params.dtype if params.dtype is not None else torch.bfloat16
         self.grace_period = grace_period
         self.next_grace_pos = None
         self.v_length = v_length
@@ -158,7 +160,7 @@ class H2OKVCache:
         if self.device.type != "cuda":
             raise RuntimeError(f"H2OKVCache buffers live on a ROCm device, not on {self.device}: there is no CPU path")
         b, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
-        kv_dtype = torch.uint8 if quantized else torch.bfloat16
+        kv_dtype = torch.uint8 if quantized else self.dtype
         row = d // 2 if (quantized and num_bits == 4) else d  # the 4-bit store packs two codes per byte
         # K and V (and their row states) are the two halves of one allocation each: one launch can walk both
         self._kv = torch.zeros((2, b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
@@ -420,14 +422,14 @@ class H2OKVCache:
         self._use_initial_rule = num == self.cache_length
         self._have_next = False
         self._input_pos = num
-        out, _, _ = ops.prefill_core(query, key.to(torch.bfloat16), value.to(torch.bfloat16), self.scale_factor, 0, None,
+        out, _, _ = ops.prefill_core(query, key.to(self.dtype), value.to(self.dtype), self.scale_factor, 0, None,
                                      return_weights=False, output_transposed=True)
         return out.reshape(b, num, hq * d)
 
     def _write(self, index: torch.Tensor, key: torch.Tensor, value: torch.Tensor, input_pos: int):
         b, h, num = index.shape
-        key = key.to(torch.bfloat16)
-        value = value.to(torch.bfloat16)
+        key = key.to(self.dtype)
+        value = value.to(self.dtype)
         if key.stride(-1) != 1:
             key = key.contiguous()
         if value.stride(-1) != 1:
@@ -435,7 +437,8 @@ class H2OKVCache:
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, self.head_size, self.cache_length
         a.input_pos = input_pos
-        a.kv_dtype = (_lib.KVX_KV_U4 if self.num_bits == 4 else _lib.KVX_KV_U8) if self.quantized else _lib.KVX_KV_BF16
+        a.kv_dtype = ((_lib.KVX_KV_U4 if self.num_bits == 4 else _lib.KVX_KV_U8) if self.quantized
+                      else (_lib.KVX_KV_F16 if self.dtype == torch.float16 else _lib.KVX_KV_BF16))
         a.index = index.data_ptr()
         a.index_stride_b, a.index_stride_h = index.stride(0), index.stride(1)
         a.key = key.data_ptr()

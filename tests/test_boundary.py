@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(kvx):
     assert sorted(_lib.SYMBOLS) == names, "ctypes table and header disagree"
     for n in names:
         assert hasattr(kvx, n), f"libkvx.so does not export {n}"
-    assert kvx.kvx_version() == 101
+    assert kvx.kvx_version() == 102
 
 
 def test_struct_layouts_match_c(tmp_path):
@@ -66,8 +66,11 @@ def test_validation_answers_without_a_gpu(kvx):
     with pytest.raises(ValueError):
         _lib.check(rc)
     a.Hq = 8
-    a.D = 256
+    a.D = 512
     assert kvx.kvx_sdpa_prefill(ctypes.byref(a), None) == _lib.KVX_ERR_UNSUPPORTED
+    a.D, a.kv_dtype = 256, _lib.KVX_KV_U8  # heads of 256 only with plain rows
+    assert kvx.kvx_sdpa_prefill(ctypes.byref(a), None) == _lib.KVX_ERR_UNSUPPORTED
+    a.kv_dtype = _lib.KVX_KV_BF16
     h = _lib.H2OArgs()
     h.B, h.Hkv, h.kv_len, h.limit, h.k = 1, 1, 16, 16, 17
     assert kvx.kvx_h2o_update_select(ctypes.byref(h), None) == _lib.KVX_ERR_INVALID
@@ -209,8 +212,11 @@ def test_hip_sdpa_keeps_reference_errors():
         s.scaled_dot_product_attention(torch.zeros(1, 3, 2, 64, dtype=torch.bfloat16), k, k, None, 6, None)
     with pytest.raises(ValueError, match="Not compatible"):
         s.scaled_dot_product_attention(q, k, k, None, 6, torch.zeros(1, 2, 7, dtype=torch.int32))
-    with pytest.raises(NotImplementedError):
-        s.scaled_dot_product_attention(q.half(), k.half(), k.half(), None, 6, None)
+    with pytest.raises(NotImplementedError):  # float32 is not served (float16 and bfloat16 are, as in the reference)
+        s.scaled_dot_product_attention(q.float(), k.float(), k.float(), None, 6, None)
+    with pytest.raises(NotImplementedError, match="head_size <= 256"):
+        s.scaled_dot_product_attention(torch.zeros(1, 4, 2, 264, dtype=torch.bfloat16), torch.zeros(1, 2, 8, 264, dtype=torch.bfloat16),
+                                       torch.zeros(1, 2, 8, 264, dtype=torch.bfloat16), None, 6, None)
     with pytest.raises(NotImplementedError, match="q_len=1, kv_len=1"):
         s.scaled_dot_product_attention(q[:, :, :1], k[:, :, :1], k[:, :, :1], None, 6, None)
 

@@ -251,3 +251,99 @@ def test_prefill_and_decode_random_shapes(gpu, case):
     torch.cuda.synchronize()
     assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
     torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
+
+
+# ---- float16 queries / keys / values and head size 256 (keys_values/attention/flashinfer_wrapper.py:276,311-319) ----
+
+TYPED_CASES = [
+    # dtype, B, Hq, Hkv, q_len, T, D, input_pos, scattered, splits
+    (torch.float16, 1, 8, 2, 128, 1024, 64, 896, True, 2),
+    (torch.float16, 2, 8, 2, 100, 333, 128, 233, False, 3),
+    (torch.float16, 1, 4, 4, 37, 700, 128, 1000, True, 0),
+    (torch.float16, 1, 4, 2, 70, 300, 256, 400, True, 2),
+    (torch.bfloat16, 1, 8, 2, 128, 1024, 256, 896, True, 0),
+    (torch.bfloat16, 2, 4, 1, 33, 200, 256, 167, False, 1),
+    (torch.bfloat16, 1, 4, 2, 300, 300, 256, 0, False, 2),  # square causal prefill
+]
+
+
+@pytest.mark.parametrize("dtype,B,Hq,Hkv,q_len,T,D,input_pos,scattered,splits", TYPED_CASES)
+def test_prefill_decode_fp16_and_head_size_256(gpu, dtype, B, Hq, Hkv, q_len, T, D, input_pos, scattered, splits):
+    q, k, v, gen = make_qkv(200 + T + q_len + D, B, Hq, Hkv, q_len, T, D, dtype=dtype)
+    tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len) if scattered else None
+    if tp is None and input_pos != T - q_len:
+        tp = (torch.arange(T, dtype=torch.int32) + (input_pos - (T - q_len))).view(1, 1, T).expand(B, Hkv, T).contiguous()
+    scale = 1.0 / math.sqrt(D)
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, None if tp is None else tp.to(torch.int64))
+    l_ref = O.lse2(q, k, scale, input_pos, tp)
+    out, w, lse = ops.prefill_core(q.to(gpu), k.to(gpu), v.to(gpu), scale, input_pos, None if tp is None else tp.to(gpu),
+                                   return_weights=True, return_lse=True, output_transposed=False, num_splits=splits)
+    torch.cuda.synchronize()
+    assert out.dtype == dtype
+    check_o(out, o_ref)
+    torch.testing.assert_close(lse.cpu(), l_ref, rtol=1e-4, atol=1e-3)
+    check_w(w, w_ref, q_len)
+    # the score-sum kernel alone, fed the oracle's log-sum-exp
+    w2 = ops.score_sum_core(q.to(gpu), k.to(gpu), l_ref.to(gpu), scale, input_pos, None if tp is None else tp.to(gpu))
+    check_w(w2, w_ref, q_len)
+    # one new token over the same cache
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], k, v, scale, 10 * T, None)
+    out1, w1, lse1 = ops.decode_core(q[:, :, :1].to(gpu), k.to(gpu), v.to(gpu), scale, return_weights=True, return_lse=True)
+    torch.cuda.synchronize()
+    assert out1.dtype == dtype
+    check_o(out1.unsqueeze(2), o1_ref)
+    check_w(w1, w1_ref, 1)
+    torch.testing.assert_close(lse1.cpu(), O.lse2(q[:, :, :1], k, scale, 10 * T, None), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float16, 128), (torch.bfloat16, 256), (torch.float16, 256)])
+def test_h2o_cache_steps_fp16_and_head_size_256(gpu, dtype, D):
+    """The cache object with float16 rows / heads of 256: prefill, chunk steps and a single-token step
+    against the oracle (the slot write is a copy of 16-bit rows, the V-norm policy reads them as float16)."""
+    from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
+
+    B, Hq, Hkv, L, chunk = 1, 4, 2, 256, 32
+    gen = torch.Generator().manual_seed(D)
+    total = L + 2 * chunk + 1
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(dtype)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(dtype)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(dtype)
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=dtype, max_chunk_size=chunk)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq, dtype), max_chunk_size=chunk, device=gpu)
+    ref.prefill(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L])
+    cache.forward(qs[:, :, :L].to(gpu), ks[:, :, :L].to(gpu), vs[:, :, :L].to(gpu))
+    pos = L
+    for num in (chunk, chunk, 1):
+        sl = slice(pos, pos + num)
+        had = ref.next_index is not None
+        o_ref, _, index = ref.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        if had:
+            cache.set_next_positions(index)
+        o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        assert o.dtype == dtype
+        assert rel_err(o.float().cpu().view(B, num, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+        assert torch.equal(cache.k.cpu(), ref.k) and torch.equal(cache.v.cpu(), ref.v)
+        assert torch.equal(cache.token_pos.cpu(), ref.token_pos)
+        torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
+        pos += num
+
+
+def test_gate_mirrors_the_reference(gpu):
+    from keys_values_amd.attention.sdpa import can_do_hip_sdpa
+
+    # keys_values/attention/flashinfer_wrapper.py:311-319: float16 or bfloat16, head sizes up to 256
+    for dtype in (torch.float16, torch.bfloat16):
+        for hs in (1, 48, 64, 100, 128, 200, 256):
+            assert can_do_hip_sdpa(hs, dtype, True) and can_do_hip_sdpa(hs, dtype, False)
+        assert not can_do_hip_sdpa(257, dtype)
+    assert not can_do_hip_sdpa(128, torch.float32)
+    # zero-padding from 129..255 to 256
+    B, Hq, Hkv, q_len, T, D = 1, 4, 2, 9, 70, 200
+    q, k, v, gen = make_qkv(43, B, Hq, Hkv, q_len, T, D, dtype=torch.float16)
+    tp = scattered_positions(gen, B, Hkv, T, 100, q_len)
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, 1 / math.sqrt(D), 100, tp.to(torch.int64))
+    out, w = HipSDPA().scaled_dot_product_attention(q.to(gpu), k.to(gpu), v.to(gpu), None, 100, tp.to(gpu), return_attn_weights=True)
+    assert out.shape == (B, Hq, q_len, D) and out.dtype == torch.float16
+    check_o(out, o_ref)
+    check_w(w, w_ref, q_len)
