@@ -1336,6 +1336,12 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
       // element (an exponential's result may not be read by the very next instruction)
       // (each result passes through an empty volatile statement: without it the compiler sinks the whole
       // computation below the step's last matrix instruction, where nothing overlaps it)
+      // (the row sum takes the element of the slot before: an exponential's result may not be read by the very
+      // next instruction)
+      if constexpr (SL >= 1) {
+        lrow[(SL - 1) >> 4] += ((SL - 1) & 1) ? po : pe;
+        asm volatile("" : "+v"(lrow[(SL - 1) >> 4]));
+      }
       if constexpr (SL >= 2 && (SL & 1) == 0) {
         constexpr int E = (SL - 2) & 15, ERB = (SL - 2) >> 4;
         uint32_t pk = pack_pair<F16>(pe, po);
@@ -1346,7 +1352,6 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
         constexpr int E = SL & 15, ERB = SL >> 4;
         float pv = fast_exp2(fmaf(s[ERB][E], p.c, -mc[ERB]));
         asm volatile("" : "+v"(pv));
-        lrow[ERB] += pv;
         if constexpr (E & 1) po = pv;
         else pe = pv;
       }
@@ -1360,6 +1365,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
     };
     unroll_seq<0, 32>(slot);
     {
+      lrow[1] += po;
       uint32_t pk = pack_pair<F16>(pe, po);
       asm volatile("" : "+v"(pk));
       pb[PAR][1][1][3] = pk;
