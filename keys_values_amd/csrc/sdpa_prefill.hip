@@ -58,15 +58,16 @@ struct PrefillParams {
 // K and V tiles in LDS: [key][16-byte chunk], rows unpadded (D * 2 bytes), chunk c of row r stored at
 // position c ^ key(r). Unpadded rows are what the global -> LDS DMA writes (a wavefront fills 1024
 // contiguous bytes per instruction); the XOR then has to spread what one LDS phase touches over
-// the 64 banks (measured on gfx950: a ds_read_b128 phase serves 16 lanes, a ds_read_b64_tr_b16
-// phase 16 lanes):
+// the 64 banks (256 bytes per cycle; measured on gfx950 with the LDS bank-conflict counter):
 //   K, ds_read_b128:        16 consecutive rows, the same chunk      -> swz_k distinct over 16 rows
-//   V, ds_read_b64_tr_b16:  4 consecutive rows x chunks {c, c + 1}   -> bits 1..2 of swz_v distinct over r % 4
+//   V, ds_read_b64_tr_b16:  half a wavefront reads 4 consecutive rows x 4 chunks (64 bytes a row): rows of 256
+//                           bytes or more start at the same bank, so bits 2..3 of swz_v are distinct over r % 4
+//                           (with bits 1..2, as for 128-byte rows, every such read took a 2-way conflict)
 // Both depend on r % 16 only, so they repeat for the row groups a wavefront loads (16 or 32 rows apart).
 template <int CPR>
 __device__ __forceinline__ int swz_k(int r) { return CPR >= 16 ? (r & 15) : ((r >> 1) & 7); }
 template <int CPR>
-__device__ __forceinline__ int swz_v(int r) { return ((r & 3) << 1) | ((r >> 2) & 1); }
+__device__ __forceinline__ int swz_v(int r) { return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 1)) : (((r & 3) << 1) | ((r >> 2) & 1)); }
 
 template <int D>
 struct alignas(16) Smem {
