@@ -19,6 +19,7 @@
 //   K/V tiles travel global -> LDS by DMA (global_load_lds_dwordx4, no registers), double-buffered,
 //   rows unpadded and XOR-swizzled against bank conflicts. The loop is software-pipelined: the
 //   matrix cores add V(t-1) P(t-1) to O while the vector ALU turns S(t) into P(t).
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -1527,9 +1528,16 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(const PrefillPa
   if (p.lse && dq == 0) p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] = Mu + fast_log2(L);
 }
 
-// The 64-row kernel serves plain rows with D = 128 once a (batch, KV head) pair has a workgroup's worth of rows.
+// The 64-row kernel can serve plain rows with D = 128 once a (batch, KV head) pair has a workgroup's worth of
+// rows. It halves the LDS traffic per matrix instruction but runs one wavefront per SIMD, whose instruction
+// issue then bounds it; on the measured shapes it ends a few percent behind the 32-row kernel, so it is chosen
+// only when the environment asks for it (KVX_PREFILL_ROWS64=1, looked up at every call).
+bool rows64_requested() {
+  const char* e = getenv("KVX_PREFILL_ROWS64");
+  return e && e[0] == '1';
+}
 bool use_w64(const kvx_sdpa_args& a) {
-  return a.D == 128 && kv_is_plain(a.kv_dtype) && (int64_t)a.q_len * (a.Hq / a.Hkv) >= W64_BM;
+  return rows64_requested() && a.D == 128 && kv_is_plain(a.kv_dtype) && (int64_t)a.q_len * (a.Hq / a.Hkv) >= W64_BM;
 }
 
 int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
