@@ -500,7 +500,7 @@ def bench_longctx(args, torch, dev):
         "config": {"workload": f"BASELINE.json configs[4]: random-init Qwen3-4B-shaped stack, {cfg.n_layer} layers, {seq} random tokens, "
                                f"chunks {sizes[0]} + {len(sizes) - 1} x {chunk}, uint8 H2O caches of {L} slots, seed 4",
                    "ms_per_step_gpu_events": round(ms_gpu, 2), "flops_attention_score_sums": attn, "flops_dense_layers": dense,
-                   "tflops_total": round((attn + dense) / (ms_step * 1e-3) / 1e12, 1), "library_gemms": "tuned (TunableOp)" if args.tune_gemms else "default"},
+                   "tflops_total": round((attn + dense) / (ms_step * 1e-3) / 1e12, 1), "library_gemms": "tuned (TunableOp)" if args.tune_gemms else ("committed per-shape table" if model.gemm_table else "library default")},
         "roofline": {"bound": "mfma", "kernel": "whole prefill (attention + score-sum kernels and library GEMMs)",
                      "achieved": round((attn + dense) / (ms_gpu * 1e-3) / 1e12, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round((attn + dense) / (ms_gpu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None},

@@ -9,6 +9,8 @@ keys_values/kvcache/base.py:554-595). Weights are random (normal, std 0.02, as
 keys_values/model.py:294-301); the linear layers are plain library GEMMs through PyTorch, everything
 else runs on the HIP kernels of this package. There is no CPU path.
 """
+import os
+import tempfile
 from dataclasses import dataclass
 from typing import List, Optional
 
@@ -57,10 +59,35 @@ class _Layer:
         self.norm_k = torch.ones(d, dtype=torch.float32, device=device) if cfg.norm_qk else None
 
 
+GEMM_TABLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_table_gfx950.csv")
+
+
+def use_gemm_table(path: str = GEMM_TABLE) -> bool:
+    """The linear layers are plain library GEMMs, and which kernel serves a shape is the library's choice; its
+    default is a poor one for some of the shapes of this stack. The table next to this file records, per shape
+    (Qwen3-4B widths, chunks of 1024 and 16384 tokens), the kernel PyTorch's TunableOp measured as fastest on
+    gfx950; it is read with tuning switched off, so nothing is measured at run time and the choice is the same in
+    every run. The file names the library versions it was made with: PyTorch refuses it under other versions,
+    and the library's default choice stays in place (returns False). Process-wide, like TunableOp itself."""
+    import torch.cuda.tunable as tunable
+
+    if not os.path.exists(path):
+        return False
+    try:
+        tunable.enable(True)
+        tunable.tuning_enable(False)
+        tunable.record_untuned_enable(False)
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), "kvx_tunableop_results.csv"))  # never into the caller's directory
+        return bool(tunable.read_file(path))
+    except Exception:  # a PyTorch without TunableOp, or a table it cannot parse: the default choice stays
+        return False
+
+
 class LongContextPrefillModel:
     def __init__(self, cfg: PrefillConfig, cache_length: int, chunk_size: int, max_batch_size: int = 1, quantized: bool = True,
-                 max_context: int = 131072, seed: int = 4, device: Optional[torch.device] = None):
+                 max_context: int = 131072, seed: int = 4, device: Optional[torch.device] = None, gemm_table: bool = True):
         self.cfg = cfg
+        self.gemm_table = use_gemm_table() if gemm_table else False
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         if self.device.type != "cuda":
             raise RuntimeError("LongContextPrefillModel runs on a ROCm device only")
