@@ -19,6 +19,10 @@ Inputs are resident in HBM before the timed region.
 `--workload policy`  : the same 1024-token chunk through the cache object (write with the ring move, attention,
                        score-sum, score update, choice of the next 1024 slots) for each eviction-policy variant
                        (grace period, normalised scores, V-norm weighting, Q-Hitter); ms per chunk step.
+`--workload ceiling` : runs the stand-alone probe built next to the library (keys_values_amd/mfma_probe): what the
+                       matrix cores sustain (clock, TFLOP/s) alone and with vector work beside them, and how fast
+                       a single wavefront issues; prints the probe's table on stderr and the sustained pure-matrix
+                       figure as the JSON line.
 `--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
                        launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
@@ -61,7 +65,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib"])
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib", "ceiling"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
                     help="default workload only: skip the decode, quantiser and long-context legs that are reported under config.secondary")
@@ -613,6 +617,32 @@ def bench_calib(args, torch, dev):
             "config": {"workload": "elementwise negate, 1 GiB read + 1 GiB written per launch", "bytes_read": 2 * n, "bytes_written": 2 * n}}
 
 
+def bench_ceiling(args, torch, dev):
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keys_values_amd", "mfma_probe")
+    if not os.path.exists(exe):
+        raise RuntimeError("keys_values_amd/mfma_probe is not built: run `python -m keys_values_amd.build`")
+    t0 = time.perf_counter()
+    out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300).stdout
+    print(out, file=sys.stderr, flush=True)
+    rows = []
+    for line in out.splitlines():
+        if "TFLOP/s" not in line:
+            continue
+        f = line.split()
+        i = f.index("wave/SIMD")
+        rows.append({"what": " ".join(f[: i - 1]), "waves_per_simd": int(f[i - 1]), "operands": f[i + 1], "ms": float(f[i + 2]),
+                     "ghz": float(f[i + 4]), "cycles_per_round": float(f[i + 6]), "tflops": float(f[i + 8])})
+    pure = [r for r in rows if r["what"] == "matrix instruction only" and r["operands"] == "random"]
+    best = max(pure, key=lambda r: r["tflops"])
+    return {"metric": "sustained bf16 MFMA TFLOP/s, matrix instructions only, random operands", "value": best["tflops"], "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": 1, "warmup": 1, "ms_per_step": best["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "keys_values_amd/mfma_probe: v_mfma_f32_32x32x16_bf16 loops over the whole device", "shader_clock_ghz": best["ghz"],
+                       "frac_of_nominal_peak": round(best["tflops"] / 2500.0, 3), "rows": rows, "wall_s": round(time.perf_counter() - t0, 1)}}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -626,7 +656,8 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fns = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib}
+    fns = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib,
+           "ceiling": bench_ceiling}
     res = fns[args.workload](args, torch, dev)
     if args.workload == "prefill" and args.kv == "bf16" and not args.no_secondary:
         # The other kernels with a target of their own, each on its own configuration, in the same run: the
