@@ -37,12 +37,14 @@ struct DecodeParams {
   uint16_t* o;
   float* lse_out;  // user (B, 1, Hq) or NULL
   float* w;        // user (B, Hkv, kv_len) or NULL
-  float* logits;   // (B, Hkv, Tpad, G)
+  float* logits;   // (B, Hkv, Tpad, G), G the padded group size
   float* part_o;   // (B, Hq, S, D)
   float* part_ml;  // (B, Hq, S, 2)
   float* lse_ws;   // (B, Hq)
   unsigned long long* best;  // fused H2O form: (value, slot) minimum per (b, kvh) row, else NULL
   int32_t B, Hq, Hkv, kv_len, Tpad, num_splits, keys_per_split;
+  int32_t Gr;  // query heads per KV head; the kernels' G is Gr rounded up to a power of two (heads Gr .. G - 1 are
+               // dummies: zero queries, nothing of theirs is stored, their logits count for nothing)
   float c;
   int64_t q_sb, q_sh, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, qs_sb, qs_sh;
 };
@@ -96,7 +98,8 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
   uint32_t qv[G][4];  // bf16 pairs of q[head][8 dc .. 8 dc + 8]
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    const u32x4_t t = *(const u32x4_t*)(p.q + b * p.q_sb + (int64_t)(kvh * G + g) * p.q_sh + 8 * dc);
+    u32x4_t t = {0u, 0u, 0u, 0u};
+    if (g < p.Gr) t = *(const u32x4_t*)(p.q + b * p.q_sb + (int64_t)(kvh * p.Gr + g) * p.q_sh + 8 * dc);
 #pragma unroll
     for (int e = 0; e < 4; ++e) qv[g][e] = t[e];
   }
@@ -290,6 +293,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
   __syncthreads();
   for (int i = tid; i < G * D; i += NTHREADS) {
     const int g = i / D, d = i % D;
+    if (g >= p.Gr) continue;
     float M = rml[0][g][0];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) M = fmaxf(M, rml[w][g][0]);
@@ -300,7 +304,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
       x += red[w][g][d] * sc;
       l += rml[w][g][1] * sc;
     }
-    const int64_t o = ((int64_t)b * p.Hq + kvh * G + g) * p.num_splits + split;
+    const int64_t o = ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits + split;
     p.part_o[o * D + d] = x;
     if (d == 0) {
       p.part_ml[o * 2] = M;
@@ -373,7 +377,7 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams 
   const int kvh = blockIdx.y, b = blockIdx.z;
   float lse[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) lse[g] = p.lse_ws[(int64_t)b * p.Hq + kvh * G + g];
+  for (int g = 0; g < G; ++g) lse[g] = g < p.Gr ? p.lse_ws[(int64_t)b * p.Hq + kvh * p.Gr + g] : INFINITY;  // exp2(x - inf) = 0
   const float* lgrow = p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G;
   float* wr = p.w ? p.w + ((int64_t)b * p.Hkv + kvh) * p.kv_len : nullptr;
   float* sc = H2O ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
@@ -400,7 +404,7 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams 
       else x = t[it][0][0];
       acc += fast_exp2(x - lse[g]);
     }
-    acc *= 1.0f / (float)G;
+    acc *= 1.0f / (float)p.Gr;
     if (wr) wr[k] = acc;
     if constexpr (H2O) {
       float val = sc[k] + acc;
@@ -444,7 +448,8 @@ struct Plan {
 
 Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
-  pl.G = a.Hq / a.Hkv;
+  const int gr = a.Hq / a.Hkv;
+  pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : 8));
   // About 16 workgroups per compute unit over the whole grid, each with at least 1024 keys.
   int splits = a.num_splits;
   if (splits <= 0) {
@@ -460,7 +465,7 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   pl.Tpad = ((a.kv_len + 63) / 64) * 64;
   size_t off = 0;
   pl.off_logits = off;
-  off += (a.w || fused_h2o) ? (size_t)a.B * a.Hq * pl.Tpad * 4 : 0;
+  off += (a.w || fused_h2o) ? (size_t)a.B * a.Hkv * pl.G * pl.Tpad * 4 : 0;
   pl.off_part_o = off;
   off += (size_t)a.B * a.Hq * pl.num_splits * a.D * 4;
   pl.off_part_ml = off;
@@ -510,7 +515,7 @@ int launch_d(const DecodeParams& p, int G, int kv, const kvx_h2o_args* hh, hipSt
     case 4: return launch_dg<D, 4>(p, kv, hh, st);
     case 8: return launch_dg<D, 8>(p, kv, hh, st);
   }
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in {1, 2, 4, 8}", G);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);
 }
 
 }  // namespace
@@ -540,6 +545,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.lse_ws = (float*)(ws + pl.off_lse);
   p.best = hh ? (unsigned long long*)(ws + pl.off_best) : nullptr;
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
+  p.Gr = a.Hq / a.Hkv;
+  KVX_REQUIRE(p.Gr <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);
   p.num_splits = pl.num_splits; p.keys_per_split = pl.keys_per_split;
   p.c = a.sm_scale * kLog2e;
   p.q_sb = a.q_stride_b; p.q_sh = a.q_stride_h;

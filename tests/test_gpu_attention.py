@@ -143,6 +143,10 @@ DECODE_CASES = [
     (1, 8, 1, 5000, 128, 3),
     (2, 4, 2, 17, 64, 0),
     (1, 8, 2, 9000, 64, 2),
+    (2, 6, 2, 700, 128, 0),        # group sizes that are not powers of two: 3, 7 (Qwen2-7B: 28 / 4), 5, 6
+    (1, 28, 4, 3000, 128, 2),
+    (1, 5, 1, 513, 64, 1),
+    (2, 12, 2, 260, 128, 0),
 ]
 
 
@@ -208,7 +212,7 @@ def _random_cases(n, seed):
     rnd = random.Random(seed)
     cases = []
     for _ in range(n):
-        G = rnd.choice([1, 2, 4, 8])
+        G = rnd.choice([1, 2, 3, 4, 5, 6, 7, 8])
         Hkv = rnd.choice([1, 2, 3])
         D = rnd.choice([64, 128])
         T = rnd.choice([1, 2, 63, 64, 65, 127, 200, 333, 512, 777, 1025, 2049])

@@ -355,9 +355,11 @@ def test_h2o_cache_steps_vs_oracle(gpu, quantized):
         pos += chunk
 
 
-def test_h2o_cache_decode_steps(gpu):
-    # single-token steps: argmin selection, slot reuse, scores = running sum (test/kvcache/test_h2o.py:109-137)
-    B, Hq, Hkv, L, D = 2, 8, 2, 256, 128
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (6, 2), (7, 1)])
+def test_h2o_cache_decode_steps(gpu, Hq, Hkv):
+    # single-token steps: argmin selection, slot reuse, scores = running sum (test/kvcache/test_h2o.py:109-137);
+    # group sizes 4, 3 and 7 (the fused decode step pads the last two to 4 and 8 heads inside the kernel)
+    B, L, D = 2, 256, 128
     gen = torch.Generator().manual_seed(3)
     total = L + 6
     qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
@@ -414,6 +416,8 @@ def test_attention_over_uint8_cache(kvx, gpu):
     (1, 4, 4, 777, 64, 700, True, False),
     (2, 8, 1, 4096 + 33, 128, 4096, True, True),
     (1, 2, 1, 17, 64, 17, False, True),
+    (2, 6, 2, 600, 128, 600, False, False),
+    (1, 5, 1, 300, 64, 256, True, True),
 ])
 def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, B, Hq, Hkv, T, D, limit, normalize, quantized):
     """kvx_sdpa_decode_h2o == kvx_sdpa_decode (with weights) followed by kvx_h2o_update_select(k=1),
