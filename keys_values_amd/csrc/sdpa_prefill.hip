@@ -20,6 +20,7 @@
 //   rows unpadded and XOR-swizzled against bank conflicts. The loop is software-pipelined: the
 //   matrix cores add V(t-1) P(t-1) to O while the vector ALU turns S(t) into P(t).
 #include <cstdlib>
+#include <cstring>
 #include <type_traits>
 #include <utility>
 
@@ -930,10 +931,13 @@ __device__ __forceinline__ void zero_o(f32x16_t& o) {
                  "s_nop 1" : "={a[112:127]}"(o));
 }
 // wait states that pass all of O through: whatever reads it afterwards depends on these
-__device__ __forceinline__ void settle_o(f32x16_t (&o)[4][2]) {
+__device__ __forceinline__ void settle_o(f32x16_t (&o)[8]) {
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7"
-               : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[1][0]), "+{a[48:63]}"(o[1][1]), "+{a[64:79]}"(o[2][0]),
-                 "+{a[80:95]}"(o[2][1]), "+{a[96:111]}"(o[3][0]), "+{a[112:127]}"(o[3][1]));
+               : "+{a[0:15]}"(o[0]), "+{a[16:31]}"(o[1]), "+{a[32:47]}"(o[2]), "+{a[48:63]}"(o[3]), "+{a[64:79]}"(o[4]),
+                 "+{a[80:95]}"(o[5]), "+{a[96:111]}"(o[6]), "+{a[112:127]}"(o[7]));
+}
+__device__ __forceinline__ void settle_o(f32x16_t (&o)[4]) {
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" : "+{a[0:15]}"(o[0]), "+{a[16:31]}"(o[1]), "+{a[32:47]}"(o[2]), "+{a[48:63]}"(o[3]));
 }
 // maxima without the canonicalising copies the compiler puts in front of fmaxf (the scores hold no signalling NaN)
 __device__ __forceinline__ float max3_raw(float a, float b, float c) {
@@ -985,7 +989,9 @@ __device__ __forceinline__ void unroll_seq(F& f) {
   unroll_seq_impl(f, std::make_integer_sequence<int, N>{});
 }
 __device__ __forceinline__ void pin_s(f32x16_t (&s)[2]) { asm volatile("" : "+v"(s[0]), "+v"(s[1])); }
+__device__ __forceinline__ void pin_s(f32x16_t (&s)[1]) { asm volatile("" : "+v"(s[0])); }
 __device__ __forceinline__ void pin_p(u32x4_t (&pp)[2][2]) { asm volatile("" : "+v"(pp[0][0]), "+v"(pp[0][1]), "+v"(pp[1][0]), "+v"(pp[1][1])); }
+__device__ __forceinline__ void pin_p(u32x4_t (&pp)[1][2]) { asm volatile("" : "+v"(pp[0][0]), "+v"(pp[0][1])); }
 
 constexpr int W64_BM = 256;  // rows per workgroup of the 64-row kernel
 
@@ -1083,14 +1089,16 @@ struct TileSender {
   }
 };
 
-template <int KV>
-__global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillParams p) {
+template <int KV, int NRB>
+__global__ __launch_bounds__(256, NRB == 1 ? 2 : 1) void sdpa_prefill_slots_kernel(const PrefillParams p) {
+  static_assert(NRB == 1 || NRB == 2, "32 or 64 rows per wavefront");
   constexpr int D = 128;
   constexpr bool F16 = KV == KVX_KV_F16;
-  constexpr int BM = W64_BM;
+  constexpr int BM = 128 * NRB;
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
+  constexpr int NO = DT * NRB;  // blocks of O: block (dt, rb) is o[dt * NRB + rb]
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1103,11 +1111,11 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   const int b = group / p.Hkv;
   const int kvh = group % p.Hkv;
 
-  const int row0w = mblk * BM + wave * 64;
-  int row[2], qi[2], g[2], qpos[2];
-  bool row_ok[2];
+  const int row0w = mblk * BM + wave * 32 * NRB;
+  int row[NRB], qi[NRB], g[NRB], qpos[NRB];
+  bool row_ok[NRB];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < NRB; ++rb) {
     row[rb] = row0w + rb * 32 + n;
     row_ok[rb] = row[rb] < p.R;
     const int rowc = row_ok[rb] ? row[rb] : p.R - 1;
@@ -1121,9 +1129,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   // accumulation registers (a load may target them) and stay there: a value the compiler first holds in a
   // vector register would be copied over in front of every matrix instruction that reads it. Rows past
   // the end load the last valid row; nothing of theirs is stored.
-  u32x4_t qf[2][KS];
+  u32x4_t qf[NRB][KS];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < NRB; ++rb) {
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)(kvh * p.G + g[rb]) * p.q_sh + (int64_t)qi[rb] * p.q_st + 8 * h;
 #pragma unroll
     for (int j = 0; j < KS; ++j) asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(qf[rb][j]) : "v"(qp + 16 * j) : "memory");
@@ -1156,7 +1164,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
     tile_end = min(tile_end, qpos_max / BN + 1);
     if (tile_end <= tile_begin) {
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+      for (int rb = 0; rb < NRB; ++rb)
         if (row_ok[rb]) {
           const int64_t prow = ((int64_t)split * p.B * p.Hkv + group) * p.R + row[rb];
           float* po = p.part_o + prow * D;
@@ -1174,45 +1182,49 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
     }
   }
 
-  f32x16_t o[DT][2];
-  zero_o<0>(o[0][0]);
-  zero_o<1>(o[0][1]);
-  zero_o<2>(o[1][0]);
-  zero_o<3>(o[1][1]);
-  zero_o<4>(o[2][0]);
-  zero_o<5>(o[2][1]);
-  zero_o<6>(o[3][0]);
-  zero_o<7>(o[3][1]);
+  f32x16_t o[NO];
+  zero_o<0>(o[0]);
+  zero_o<1>(o[1]);
+  zero_o<2>(o[2]);
+  zero_o<3>(o[3]);
+  if constexpr (NO == 8) {
+    zero_o<4>(o[4]);
+    zero_o<5>(o[5]);
+    zero_o<6>(o[6]);
+    zero_o<7>(o[7]);
+  }
   // row sums of P, in fp32 from the unrounded values (the log-sum-exp feeds the score sums, which are held to
   // 1e-3): this lane's 16 keys of every step; the other half of the wavefront holds the other 16
-  float lrow[2] = {0.0f, 0.0f};
-  float m[2] = {-INFINITY, -INFINITY};
+  float lrow[NRB], m[NRB];
+#pragma unroll
+  for (int rb = 0; rb < NRB; ++rb) {
+    lrow[rb] = 0.0f;
+    m[rb] = -INFINITY;
+  }
   const float slack = kSlackLog2 / p.c;
 
-  f32x16_t sb[2][2];     // S of a step: [buffer][row block]
-  u32x4_t pb[2][2][2];   // packed P of a step: [buffer][row block][key step of 16], the B operands of the second product
+  f32x16_t sb[2][NRB];     // S of a step: [buffer][row block]
+  u32x4_t pb[2][NRB][2];   // packed P of a step: [buffer][row block][key step of 16], the B operands of the second product
 
   TileSender ld;
   ld.init(p, sm, b, kvh, tid, tile_begin);
 
   constexpr int KBYTES = BN * CPR * 16;  // bytes of one K or V tile buffer
   // S(next) = K Q^T for 32 keys: key rows 32 MT .. of K buffer KBUF
-  auto qk_all = [&](f32x16_t (&s)[2], auto kbuf_tag, auto mt_tag) {
+  auto qk_all = [&](f32x16_t (&s)[NRB], auto kbuf_tag, auto mt_tag) {
     constexpr int OFF = decltype(kbuf_tag)::value * KBYTES + decltype(mt_tag)::value * 32 * CPR * 16;
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
       const u32x4_t kk = *(const u32x4_t __attribute__((address_space(3)))*)(ka[j] + OFF);
-      if (j == 0) {
-        mfma_s_first<F16>(s[0], kk, qf[0][0]);
-        mfma_s_first<F16>(s[1], kk, qf[1][0]);
-      } else {
-        mfma_s<F16>(s[0], kk, qf[0][j]);
-        mfma_s<F16>(s[1], kk, qf[1][j]);
+#pragma unroll
+      for (int rb = 0; rb < NRB; ++rb) {
+        if (j == 0) mfma_s_first<F16>(s[rb], kk, qf[rb][0]);
+        else mfma_s<F16>(s[rb], kk, qf[rb][j]);
       }
     }
   };
   // O += V^T P^T for the 32 keys of a step
-  auto pv_all = [&](const u32x4_t (&pp)[2][2], auto vbuf_tag, auto mt_tag) {
+  auto pv_all = [&](const u32x4_t (&pp)[NRB][2], auto vbuf_tag, auto mt_tag) {
     constexpr int OFF = decltype(vbuf_tag)::value * KBYTES + decltype(mt_tag)::value * 32 * CPR * 16;
     auto one = [&](auto dt_tag, int j) {
       constexpr int dt = decltype(dt_tag)::value;
@@ -1220,8 +1232,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
       const u32x2_t lo = lds_read_tr16(vl);
       const u32x2_t hi = lds_read_tr16(vl + 8 * CPR * 16);
       const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
-      mfma_o<F16, 2 * dt>(o[dt][0], vf, pp[0][j]);
-      mfma_o<F16, 2 * dt + 1>(o[dt][1], vf, pp[1][j]);
+      mfma_o<F16, dt * NRB>(o[dt * NRB], vf, pp[0][j]);
+      if constexpr (NRB == 2) mfma_o<F16, dt * NRB + 1>(o[dt * NRB + 1], vf, pp[NRB - 1][j]);
     };
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -1235,12 +1247,16 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   // Softmax state of the step about to run: m is the reference maximum its exponentials use, mc = m c, and alpha
   // is the factor that takes O and the row sums from the reference of the step before to this one (applied at
   // the end of the step, once the second product has added the P of the step before).
-  float mc[2] = {0.0f, 0.0f};
-  float alpha[2] = {1.0f, 1.0f};
+  float mc[NRB], alpha[NRB], mx[NRB];
+#pragma unroll
+  for (int rb = 0; rb < NRB; ++rb) {
+    mc[rb] = 0.0f;
+    alpha[rb] = 1.0f;
+    mx[rb] = -INFINITY;
+  }
   bool resc = false;
   // mask, row maxima and the rescaling decision for the S in sn: key rows 32 half .. of the tile in ring slot ts
-  float mx[2];
-  auto mask_next = [&](f32x16_t (&sn)[2], int ts, int half, int tpl) {  // tpl: sm.tp[ts][32 half + n]
+  auto mask_next = [&](f32x16_t (&sn)[NRB], int ts, int half, int tpl) {  // tpl: sm.tp[ts][32 half + n]
     const unsigned hidden = (unsigned)__ballot(tpl > qpos_min_w);  // lanes 0..31: the step's 32 keys
     if (hidden) {
 #pragma unroll
@@ -1248,7 +1264,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
         if ((hidden >> (8 * a)) & 0xffu) {
           const int4 tq = *(const int4*)&sm.tp[ts][half * 32 + 8 * a + 4 * h];
 #pragma unroll
-          for (int rb = 0; rb < 2; ++rb) {
+          for (int rb = 0; rb < NRB; ++rb) {
             if (tq.x > qpos[rb]) sn[rb][4 * a + 0] = -INFINITY;
             if (tq.y > qpos[rb]) sn[rb][4 * a + 1] = -INFINITY;
             if (tq.z > qpos[rb]) sn[rb][4 * a + 2] = -INFINITY;
@@ -1257,12 +1273,14 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
         }
     }
   };
-  auto row_max = [&](const f32x16_t& sv, float& out) { out = row_max_raw(sv); };
   auto decide = [&]() {
-    resc = __any(mx[0] > m[0] + slack || mx[1] > m[1] + slack);
+    bool need = false;
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) need |= mx[rb] > m[rb] + slack;
+    resc = __any(need);
     if (resc) {
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
+      for (int rb = 0; rb < NRB; ++rb) {
         const float m_new = fmaxf(m[rb], mx[rb]);
         const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
         alpha[rb] = fast_exp2((m[rb] - m_use) * p.c);
@@ -1270,22 +1288,26 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
         m[rb] = m_new;
       }
     }
-    mc[0] = (m[0] == -INFINITY) ? 0.0f : m[0] * p.c;
-    mc[1] = (m[1] == -INFINITY) ? 0.0f : m[1] * p.c;
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) mc[rb] = (m[rb] == -INFINITY) ? 0.0f : m[rb] * p.c;
   };
-  // The operand fragments of a step pass through a ring of four registers, each read from LDS three fragments
-  // (six matrix instructions) before its first use: fragments 0..7 are the K rows of the first product, 8..15 the
-  // V rows of the second (8 + 4 j + dt), 16..18 the first K rows of the step after.
-  u32x4_t fr[4];
+  // The operand fragments of a step pass through a ring of RING registers, each read from LDS DIST fragments
+  // before its first use (a fragment feeds NRB matrix instructions): fragments 0..7 are the K rows of the first
+  // product, 8..15 the V rows of the second (8 + 4 j + dt), 16.. the first K rows of the step after.
+  constexpr int RING = NRB == 2 ? 4 : 8;
+  constexpr int DIST = RING - 1;
+  u32x4_t fr[RING];
 
   // One step s = 2 (tile - tile_begin) + (K4 & 1), K4 = s mod 4: S(s) sits in sb[K4 & 1] with its mask, row
   // maxima and rescaling decision already taken. A wavefront issues in order, and a matrix instruction waits at
   // issue while the one before it occupies the matrix core (32 cycles), so vector work only overlaps the matrix
-  // instruction that directly precedes it: the step is 32 slots of one matrix instruction each, followed by a
-  // slot's worth of vector work. Slots 0..15 multiply S(s+1) into sb[~K4 & 1], slots 16..31 add V(s-1) P(s-1)
-  // to O; every slot also turns one element of S(s) into P(s), and three of the later ones prepare S(s+1).
-  // Tile t lives in LDS buffer (t - tile_begin) & 1; transfers start two steps before their tile is first read
-  // and are published by the barrier in the first step of every tile.
+  // instruction that directly precedes it: the step is 16 NRB slots of one matrix instruction each, followed by a
+  // slot's worth of vector work. The first half of the slots multiplies S(s+1) into sb[~K4 & 1], the second adds
+  // V(s-1) P(s-1) to O; every slot also turns one element of S(s) into P(s), and a few of the later ones prepare
+  // S(s+1). Tile t lives in LDS buffer (t - tile_begin) & 1; transfers start two steps before their tile is first
+  // read and are published by the barrier in the first step of every tile.
+  constexpr int NS = 16 * NRB;   // slots per step
+  constexpr int NQK = 8 * NRB;   // slots of the first product
   auto step = [&](auto k4_tag, int tile) {
     constexpr int K4 = decltype(k4_tag)::value;
     constexpr int PAR = K4 & 1;
@@ -1296,50 +1318,49 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
     constexpr int KOFF = KBUF_N * KBYTES + MT_N * 32 * CPR * 16;
     constexpr int KOFF_NN = KBUF_NN * KBYTES + MT_NN * 32 * CPR * 16;
     constexpr int VOFF = VBUF_P * KBYTES + MT_P * 32 * CPR * 16;
-    f32x16_t (&s)[2] = sb[PAR];
-    f32x16_t (&sn)[2] = sb[PAR ^ 1];
+    f32x16_t (&s)[NRB] = sb[PAR];
+    f32x16_t (&sn)[NRB] = sb[PAR ^ 1];
     pin_s(s);  // S(s), written by the step before, is read from here on, not earlier
     const int tsel = (tile - tile_begin) & 3;  // ring slot of this tile's token positions
     const bool has_next = K4 != 3 || tile + 1 < tile_end;  // tiles come in pairs: only the last step of a pair may be the last
     float pe = 0.0f, po = 0.0f;                // the pair of P elements to pack next
     int tpl_next = 0;                          // position of key n of the step after this one
+    float xs = fmaf(s[0][0], p.c, -mc[0]);     // scaled difference of the element whose exponential is next
     auto read_fragment = [&](auto f_tag) {
       constexpr int f = decltype(f_tag)::value;
       if constexpr (f < 8) {
-        fr[f & 3] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[f] + KOFF);
+        fr[f % RING] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[f] + KOFF);
       } else if constexpr (f < 16) {
         const lds_ptr_t vl = va[f & 3] + VOFF + 16 * ((f - 8) >> 2) * CPR * 16;
         const u32x2_t lo = lds_read_tr16(vl);
         const u32x2_t hi = lds_read_tr16(vl + 8 * CPR * 16);
-        fr[f & 3] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+        fr[f % RING] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
       } else {
-        fr[f & 3] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[f - 16] + KOFF_NN);
+        fr[f % RING] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[f - 16] + KOFF_NN);
       }
     };
     auto slot = [&](auto sl_tag) {
       constexpr int SL = decltype(sl_tag)::value;
-      constexpr int RB = SL & 1;
-      if constexpr (SL < 16) {
-        constexpr int J = SL >> 1;
+      constexpr int RB = SL % NRB;
+      if constexpr (SL < NQK) {
+        constexpr int J = SL / NRB;
         if constexpr (J == 0) mfma_s_first<F16>(sn[RB], fr[0], qf[RB][0]);
-        else mfma_s<F16>(sn[RB], fr[J & 3], qf[RB][J]);
+        else mfma_s<F16>(sn[RB], fr[J % RING], qf[RB][J]);
       } else {
-        constexpr int I = (SL - 16) >> 1, DTI = I & 3, J = I >> 2;
-        mfma_o<F16, 2 * DTI + RB>(o[DTI][RB], fr[I & 3], pb[PAR ^ 1][RB][J]);
+        constexpr int I = (SL - NQK) / NRB, DTI = I & 3, J = I >> 2;
+        mfma_o<F16, DTI * NRB + RB>(o[DTI * NRB + RB], fr[(8 + I) % RING], pb[PAR ^ 1][RB][J]);
       }
-      if constexpr (RB == 0 && SL < 26) read_fragment(std::integral_constant<int, (SL >> 1) + 3>{});
+      if constexpr (RB == 0 && SL / NRB + DIST < 16) read_fragment(std::integral_constant<int, SL / NRB + DIST>{});
       if constexpr (SL == 1 && PAR == 1) {
         // V of the next tile into the buffer the second product left in the step before, K of the tile after it
         // into the buffer the first product left there
         ld.template send<false, TBUF ^ 1>(sm, tid, 0, tile_end);                // tile + 1
         ld.template send<true, TBUF>(sm, tid, (tsel + 2) & 3, tile_end);        // tile + 2
       }
-      // P for key SL & 15 (register order) of row block SL >> 4; a pair is packed one slot after its second
-      // element (an exponential's result may not be read by the very next instruction)
-      // (each result passes through an empty volatile statement: without it the compiler sinks the whole
-      // computation below the step's last matrix instruction, where nothing overlaps it)
-      // (the row sum takes the element of the slot before: an exponential's result may not be read by the very
-      // next instruction)
+      // P for key SL % 16 (register order) of row block SL / 16. Each result passes through an empty volatile
+      // statement: without it the compiler sinks the whole computation below the step's last matrix instruction,
+      // where nothing overlaps it. An exponential's result may not be read by the very next instruction, so the
+      // row sum takes the element of the slot before, and a pair is packed one slot after its second element.
       if constexpr (SL >= 1) {
         lrow[(SL - 1) >> 4] += ((SL - 1) & 1) ? po : pe;
         asm volatile("" : "+v"(lrow[(SL - 1) >> 4]));
@@ -1350,27 +1371,33 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
         asm volatile("" : "+v"(pk));
         pb[PAR][ERB][E >> 3][(E >> 1) & 3] = pk;
       }
-      if constexpr (SL < 32) {
-        constexpr int E = SL & 15, ERB = SL >> 4;
-        float pv = fast_exp2(fmaf(s[ERB][E], p.c, -mc[ERB]));
+      {
+        // (the scaled difference of the next element is formed here, one slot before its exponential: an
+        // instruction that reads the result of the one right before it waits for it)
+        float pv = fast_exp2(xs);
         asm volatile("" : "+v"(pv));
-        if constexpr (E & 1) po = pv;
+        if constexpr (SL & 1) po = pv;
         else pe = pv;
+        if constexpr (SL + 1 < NS) {
+          constexpr int E1 = (SL + 1) & 15, ERB1 = (SL + 1) >> 4;
+          xs = fmaf(s[ERB1][E1], p.c, -mc[ERB1]);
+          asm volatile("" : "+v"(xs));
+        }
       }
-      if constexpr (SL == 8) tpl_next = sm.tp[PAR == 1 ? (tsel + 1) & 3 : tsel][(PAR ^ 1) * 32 + n];
+      if constexpr (SL == 4 * NRB) tpl_next = sm.tp[PAR == 1 ? (tsel + 1) & 3 : tsel][(PAR ^ 1) * 32 + n];
       // S(s+1) is complete two slots after the last instruction of the first product: its mask and row maxima
       // go between the instructions of the second
-      if constexpr (SL == 18) { if (has_next) mask_next(sn, PAR == 1 ? (tsel + 1) & 3 : tsel, PAR ^ 1, tpl_next); }
-      if constexpr (SL == 21) { if (has_next) row_max(sn[0], mx[0]); }
-      if constexpr (SL == 25) { if (has_next) row_max(sn[1], mx[1]); }
+      if constexpr (SL == NQK + 2) { if (has_next) mask_next(sn, PAR == 1 ? (tsel + 1) & 3 : tsel, PAR ^ 1, tpl_next); }
+      if constexpr (SL == NQK + 5) { if (has_next) mx[0] = row_max_raw(sn[0]); }
+      if constexpr (NRB == 2 && SL == NQK + 9) { if (has_next) mx[NRB - 1] = row_max_raw(sn[NRB - 1]); }
       __builtin_amdgcn_sched_barrier(0);
     };
-    unroll_seq<0, 32>(slot);
+    unroll_seq<0, NS>(slot);
     {
-      lrow[1] += po;
+      lrow[NRB - 1] += po;
       uint32_t pk = pack_pair<F16>(pe, po);
       asm volatile("" : "+v"(pk));
-      pb[PAR][1][1][3] = pk;
+      pb[PAR][NRB - 1][1][3] = pk;
     }
     pin_p(pb[PAR]);  // P(s) is complete here, a whole step before the matrix core reads it
     if constexpr (PAR == 0) {
@@ -1381,20 +1408,21 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
     }
-    read_fragment(std::integral_constant<int, 16>{});
-    read_fragment(std::integral_constant<int, 17>{});
-    read_fragment(std::integral_constant<int, 18>{});
+    auto read_ahead = [&](auto i_tag) { read_fragment(std::integral_constant<int, 16 + decltype(i_tag)::value>{}); };
+    unroll_seq<0, DIST>(read_ahead);
     __builtin_amdgcn_sched_barrier(0);
     if (resc) {  // O (now including step s - 1) moves to the reference maximum of P(s)
       settle_o(o);  // the last matrix instructions have to leave O first
-      scale_o<0>(o[0][0], alpha[0]);
-      scale_o<1>(o[0][1], alpha[1]);
-      scale_o<2>(o[1][0], alpha[0]);
-      scale_o<3>(o[1][1], alpha[1]);
-      scale_o<4>(o[2][0], alpha[0]);
-      scale_o<5>(o[2][1], alpha[1]);
-      scale_o<6>(o[3][0], alpha[0]);
-      scale_o<7>(o[3][1], alpha[1]);
+      scale_o<0>(o[0], alpha[0]);
+      scale_o<1>(o[1], alpha[1 % NRB]);
+      scale_o<2>(o[2], alpha[2 % NRB]);
+      scale_o<3>(o[3], alpha[3 % NRB]);
+      if constexpr (NO == 8) {
+        scale_o<4>(o[4], alpha[0]);
+        scale_o<5>(o[5], alpha[1 % NRB]);
+        scale_o<6>(o[6], alpha[0]);
+        scale_o<7>(o[7], alpha[1 % NRB]);
+      }
       resc = false;
     }
     if (has_next) decide();
@@ -1412,7 +1440,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
     for (int i = 0; i < BN * CPR / 256; ++i) (&sm.v[1][0][0])[tid + 256 * i] = z;
   }
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < NRB; ++rb)
 #pragma unroll
     for (int j = 0; j < 2; ++j) pb[1][rb][j] = u32x4_t{0u, 0u, 0u, 0u};
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1424,13 +1452,13 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   constexpr std::integral_constant<int, 3> I3{};
   qk_all(sb[0], I0, I0);
 #pragma unroll
-  for (int j = 0; j < 3; ++j) fr[j] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[j] + 32 * CPR * 16);  // K rows of step 1
+  for (int j = 0; j < DIST; ++j) fr[j] = *(const u32x4_t __attribute__((address_space(3)))*)(ka[j] + 32 * CPR * 16);  // K rows of step 1
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // S(0) is read right away
   pin_s(sb[0]);
   pin_p(pb[1]);
   mask_next(sb[0], 0, 0, sm.tp[0][n]);
-  row_max(sb[0][0], mx[0]);
-  row_max(sb[0][1], mx[1]);
+#pragma unroll
+  for (int rb = 0; rb < NRB; ++rb) mx[rb] = row_max_raw(sb[0][rb]);
   decide();
   // Tiles alternate between the two LDS buffers and the step templates cover a pair of them. A walk over an odd
   // number of tiles ends with a tile that is not there: nothing is transferred for it, all its positions are
@@ -1447,9 +1475,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   settle_o(o);            // O is read by the vector ALU next
   // from the fixed accumulation registers into ordinary ones (the compiler may not take parts of a fixed register)
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb) asm volatile("" : "+v"(o[dt][rb]));
+  for (int i = 0; i < NO; ++i) asm volatile("" : "+v"(o[i]));
 
   // ---- epilogue -----------------------------------------------------------------------------
   // The row coordinates are taken again from the lane number here: held across the loop they would occupy
@@ -1458,9 +1484,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
   asm volatile("" : "+v"(tid_e));
   const int h_e = (tid_e >> 5) & 1;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < NRB; ++rb) {
     const float lt = sum_halves(lrow[rb]);
-    const int row_e = mblk * BM + (tid_e >> 6) * 64 + rb * 32 + (tid_e & 31);
+    const int row_e = mblk * BM + (tid_e >> 6) * 32 * NRB + rb * 32 + (tid_e & 31);
     if (row_e >= p.R) continue;
     const int qi_e = row_e / p.G, g_e = row_e % p.G;
     if (p.num_splits == 1) {
@@ -1470,9 +1496,10 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
+          const f32x16_t& ob = o[dt * NRB + rb];
           u32x2_t w2;
-          w2[0] = pack_pair<F16>(o[dt][rb][4 * a] * inv, o[dt][rb][4 * a + 1] * inv);
-          w2[1] = pack_pair<F16>(o[dt][rb][4 * a + 2] * inv, o[dt][rb][4 * a + 3] * inv);
+          w2[0] = pack_pair<F16>(ob[4 * a] * inv, ob[4 * a + 1] * inv);
+          w2[1] = pack_pair<F16>(ob[4 * a + 2] * inv, ob[4 * a + 3] * inv);
           *(u32x2_t*)(op + dt * 32 + 8 * a + 4 * h_e) = w2;
         }
       if (p.lse && h_e == 0) p.lse[((int64_t)b * p.q_len + qi_e) * p.Hq + kvh * p.G + g_e] = m[rb] * p.c + fast_log2(lt);
@@ -1483,7 +1510,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_w64_kernel(const PrefillP
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-          f32x4_t w4 = {o[dt][rb][4 * a], o[dt][rb][4 * a + 1], o[dt][rb][4 * a + 2], o[dt][rb][4 * a + 3]};
+          const f32x16_t& ob = o[dt * NRB + rb];
+          f32x4_t w4 = {ob[4 * a], ob[4 * a + 1], ob[4 * a + 2], ob[4 * a + 3]};
           *(f32x4_t*)(po + dt * 32 + 8 * a + 4 * h_e) = w4;
         }
       if (h_e == 0) {
@@ -1528,16 +1556,22 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(const PrefillPa
   if (p.lse && dq == 0) p.lse[((int64_t)b * p.q_len + qi) * p.Hq + kvh * p.G + g] = Mu + fast_log2(L);
 }
 
-// The 64-row kernel can serve plain rows with D = 128 once a (batch, KV head) pair has a workgroup's worth of
-// rows. It halves the LDS traffic per matrix instruction but runs one wavefront per SIMD, whose instruction
-// issue then bounds it; on the measured shapes it ends a few percent behind the 32-row kernel, so it is chosen
-// only when the environment asks for it (KVX_PREFILL_ROWS64=1, looked up at every call).
-bool rows64_requested() {
-  const char* e = getenv("KVX_PREFILL_ROWS64");
-  return e && e[0] == '1';
-}
-bool use_w64(const kvx_sdpa_args& a) {
-  return rows64_requested() && a.D == 128 && kv_is_plain(a.kv_dtype) && (int64_t)a.q_len * (a.Hq / a.Hkv) >= W64_BM;
+// Three kernels serve plain rows with D = 128: the 32-row kernel above ("classic": the compiler schedules the
+// step), and the slot kernel with 32 or 64 rows per wavefront ("slots32": two workgroups per compute unit,
+// "slots64": one; 64 rows need a workgroup's worth of rows per (batch, KV head) pair). KVX_PREFILL_KERNEL in the
+// environment (looked up at every call) picks one by name; without it the default below is used.
+enum PrefillVariant { PF_CLASSIC = 0, PF_SLOTS32 = 1, PF_SLOTS64 = 2 };
+constexpr int PF_DEFAULT = PF_CLASSIC;
+int prefill_variant(const kvx_sdpa_args& a) {
+  if (a.D != 128 || !kv_is_plain(a.kv_dtype)) return PF_CLASSIC;
+  int v = PF_DEFAULT;
+  if (const char* e = getenv("KVX_PREFILL_KERNEL")) {
+    if (!strcmp(e, "classic")) v = PF_CLASSIC;
+    else if (!strcmp(e, "slots32")) v = PF_SLOTS32;
+    else if (!strcmp(e, "slots64")) v = PF_SLOTS64;
+  }
+  if (v == PF_SLOTS64 && (int64_t)a.q_len * (a.Hq / a.Hkv) < W64_BM) v = PF_SLOTS32;
+  return v;
 }
 
 int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
@@ -1545,7 +1579,7 @@ int pick_splits(const kvx_sdpa_args& a, int m_blocks, int num_tiles) {
   // Aim for one resident round of workgroups (2 per compute unit, 1 with the uint8 cache): more
   // splits only add partials to write, merge and re-read. At least 8 key tiles per split.
   const int64_t base = (int64_t)a.B * a.Hkv * m_blocks;
-  const int target = ((kv_is_plain(a.kv_dtype) && a.D <= 128 && !use_w64(a)) ? 2 : 1) * num_cus();
+  const int target = ((kv_is_plain(a.kv_dtype) && a.D <= 128 && prefill_variant(a) != PF_SLOTS64) ? 2 : 1) * num_cus();
   int s = (int)((target + base - 1) / base);
   s = max(1, min(s, num_tiles / 8));
   return max(1, min(s, 64));
@@ -1571,7 +1605,7 @@ void fill_params(PrefillParams& p, const kvx_sdpa_args& a) {
   p.R = a.q_len * p.G;
   p.input_pos = a.input_pos;
   p.num_tiles = (a.kv_len + BN - 1) / BN;
-  const int bm = use_w64(a) ? W64_BM : 32 * nwaves(a.kv_dtype);
+  const int bm = prefill_variant(a) == PF_SLOTS64 ? W64_BM : 32 * nwaves(a.kv_dtype);
   p.m_blocks = (p.R + bm - 1) / bm;
   p.num_splits = pick_splits(a, p.m_blocks, p.num_tiles);
   p.tiles_per_split = (p.num_tiles + p.num_splits - 1) / p.num_splits;
@@ -1594,10 +1628,11 @@ size_t partial_bytes(const PrefillParams& p, int D) {
 }
 
 template <int D, int KV>
-int launch_t(PrefillParams& p, hipStream_t st, bool w64 = false) {
+int launch_t(PrefillParams& p, hipStream_t st, int variant = PF_CLASSIC) {
   dim3 grid(p.B * p.Hkv, p.m_blocks, p.num_splits);
   if constexpr (D == 128 && kv_is_plain(KV)) {
-    if (w64) hipLaunchKernelGGL((sdpa_prefill_w64_kernel<KV>), grid, dim3(256), 0, st, p);
+    if (variant == PF_SLOTS64) hipLaunchKernelGGL((sdpa_prefill_slots_kernel<KV, 2>), grid, dim3(256), 0, st, p);
+    else if (variant == PF_SLOTS32) hipLaunchKernelGGL((sdpa_prefill_slots_kernel<KV, 1>), grid, dim3(256), 0, st, p);
     else hipLaunchKernelGGL((sdpa_prefill_kernel<D, KV>), grid, dim3(64 * nwaves(KV)), 0, st, p);
   } else {
     hipLaunchKernelGGL((sdpa_prefill_kernel<D, KV>), grid, dim3(64 * nwaves(KV)), 0, st, p);
@@ -1633,8 +1668,8 @@ int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {
   }
   if (a.D == 128) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st, use_w64(a));
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st, use_w64(a));
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st, prefill_variant(a));
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st, prefill_variant(a));
   }
   if (a.D == 64) {
     if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);

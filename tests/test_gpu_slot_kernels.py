@@ -1,6 +1,7 @@
 """
-The 64-row-per-wavefront prefill kernel (chosen with KVX_PREFILL_ROWS64=1 for head size 128, bf16 / fp16 rows,
-at least 256 query rows per KV head) against the oracle, and against the default kernel on the same inputs.
+The slot-structured prefill kernels (KVX_PREFILL_KERNEL=slots32 / slots64 in the environment: head size 128,
+bf16 / fp16 rows; 64 rows per wavefront need at least 256 query rows per KV head, else 32 are used) against
+the oracle, and against the default kernel on the same inputs.
 """
 import math
 import os
@@ -24,23 +25,24 @@ CASES = [
     (2, 8, 2, 128, 1024, 896, True, 2),
     (1, 8, 1, 37, 700, 1000, True, 0),
     (1, 4, 2, 300, 300, 0, False, 2),
+    (2, 4, 4, 16, 200, 300, True, 1),       # fewer rows than a workgroup holds
 ]
 
 
-@pytest.fixture
-def rows64():
-    old = os.environ.get("KVX_PREFILL_ROWS64")
-    os.environ["KVX_PREFILL_ROWS64"] = "1"
-    yield
+@pytest.fixture(params=["slots32", "slots64"])
+def variant(request):
+    old = os.environ.get("KVX_PREFILL_KERNEL")
+    os.environ["KVX_PREFILL_KERNEL"] = request.param
+    yield request.param
     if old is None:
-        del os.environ["KVX_PREFILL_ROWS64"]
+        del os.environ["KVX_PREFILL_KERNEL"]
     else:
-        os.environ["KVX_PREFILL_ROWS64"] = old
+        os.environ["KVX_PREFILL_KERNEL"] = old
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,Hq,Hkv,q_len,T,input_pos,scattered,splits", CASES)
-def test_rows64_prefill_against_oracle(gpu, rows64, B, Hq, Hkv, q_len, T, input_pos, scattered, splits, dtype):
+def test_slot_kernels_against_oracle(gpu, variant, B, Hq, Hkv, q_len, T, input_pos, scattered, splits, dtype):
     D = 128
     q, k, v, gen = make_qkv(300 + T + q_len, B, Hq, Hkv, q_len, T, D)
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
@@ -59,9 +61,9 @@ def test_rows64_prefill_against_oracle(gpu, rows64, B, Hq, Hkv, q_len, T, input_
     torch.testing.assert_close(lse.cpu(), l_ref, rtol=1e-4, atol=1e-3)
     torch.testing.assert_close(w.cpu(), w_ref, rtol=1e-3, atol=1e-6)
     # the default kernel on the same inputs: same log-sum-exp to rounding, outputs equal to bf16 rounding
-    del os.environ["KVX_PREFILL_ROWS64"]
+    os.environ["KVX_PREFILL_KERNEL"] = "classic"
     out32, w32, lse32 = ops.prefill_core(*args, **kw)
-    os.environ["KVX_PREFILL_ROWS64"] = "1"
+    os.environ["KVX_PREFILL_KERNEL"] = variant
     torch.cuda.synchronize()
     torch.testing.assert_close(lse, lse32, rtol=1e-5, atol=1e-4)
     assert rel_err(out.float(), out32.float()) < 6e-3
