@@ -1325,7 +1325,6 @@ __global__ __launch_bounds__(256, NRB == 1 ? 2 : 1) void sdpa_prefill_slots_kern
     const bool has_next = K4 != 3 || tile + 1 < tile_end;  // tiles come in pairs: only the last step of a pair may be the last
     float pe = 0.0f, po = 0.0f;                // the pair of P elements to pack next
     int tpl_next = 0;                          // position of key n of the step after this one
-    float xs = fmaf(s[0][0], p.c, -mc[0]);     // scaled difference of the element whose exponential is next
     auto read_fragment = [&](auto f_tag) {
       constexpr int f = decltype(f_tag)::value;
       if constexpr (f < 8) {
@@ -1372,17 +1371,11 @@ __global__ __launch_bounds__(256, NRB == 1 ? 2 : 1) void sdpa_prefill_slots_kern
         pb[PAR][ERB][E >> 3][(E >> 1) & 3] = pk;
       }
       {
-        // (the scaled difference of the next element is formed here, one slot before its exponential: an
-        // instruction that reads the result of the one right before it waits for it)
-        float pv = fast_exp2(xs);
+        constexpr int E = SL & 15, ERB = SL >> 4;
+        float pv = fast_exp2(fmaf(s[ERB][E], p.c, -mc[ERB]));
         asm volatile("" : "+v"(pv));
-        if constexpr (SL & 1) po = pv;
+        if constexpr (E & 1) po = pv;
         else pe = pv;
-        if constexpr (SL + 1 < NS) {
-          constexpr int E1 = (SL + 1) & 15, ERB1 = (SL + 1) >> 4;
-          xs = fmaf(s[ERB1][E1], p.c, -mc[ERB1]);
-          asm volatile("" : "+v"(xs));
-        }
       }
       if constexpr (SL == 4 * NRB) tpl_next = sm.tp[PAR == 1 ? (tsel + 1) & 3 : tsel][(PAR ^ 1) * 32 + n];
       // S(s+1) is complete two slots after the last instruction of the first product: its mask and row maxima
