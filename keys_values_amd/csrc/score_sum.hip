@@ -271,6 +271,9 @@ __global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(c
       ld.commit(st, sm, buf ^ 1, (t + 1) % 3, tid);
       if (t + 2 < num_qt) ld.fetch(st, (t + 2) * BQ, tid);
     }
+    // issue priority: lowest in the first half of a tile, highest on the way to the barrier, so that the
+    // four wavefronts of a workgroup wait less for each other (about 1 % on the kernel)
+    __builtin_amdgcn_s_setprio(0);
     const bool need_mask = tpmax > p.input_pos + (t * BQ) / p.G;
     if (need_mask) {
       mfma_block(sb, buf, 1);
@@ -281,7 +284,9 @@ __global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(c
       valu_block(std::false_type{}, sa, buf3, 0);
       interleave(std::false_type{});
     }
+    __builtin_amdgcn_s_setprio(3);
     __syncthreads();
+    __builtin_amdgcn_s_setprio(1);
     if (more) {
       if (need_mask) {
         mfma_block(sa, buf ^ 1, 0);
