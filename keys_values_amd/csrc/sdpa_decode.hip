@@ -12,13 +12,19 @@
 // the same lanes with dot2 over pairs of rows. Every row group of a wavefront keeps its own running
 // maximum, sum and fp32 accumulator (the maximum moves lazily), so the loop has no barrier and no
 // cross-lane traffic beyond the row reduction; groups and wavefronts are merged once at the end.
-// The logits (log2 units) are gathered in LDS and leave for the fp32 scratch, [key][head], in bursts
-// of 32 KB: a write stream mixed into the reads costs HBM far more than its share of the bytes.
-// A merge kernel combines the splits and produces the base-2 log-sum-exp; a last streaming kernel
-// turns the stored logits into W = (1/G) sum_g exp2(logit_g - lse_g) and, in the fused H2O form, adds
-// W to the cumulative scores and finds each row's lowest-score slot in the same pass. K and V are
-// touched once: they are loaded non-temporally. No float atomics anywhere.
+// The logits (log2 units) of a split are gathered in LDS, [key][head]. When a split's logits fit there
+// (16384 / G keys for most shapes), they never leave the chip: a workgroup publishes its partial maximum and sum, waits
+// until the other splits of its (batch, KV head) row have done the same (workgroups are dispatched in
+// index order and a row's splits are neighbours, so they run at the same time; the wait is bounded),
+// combines them into the row's base-2 log-sum-exp and turns its own logits into
+// W = (1/G) sum_g exp2(logit_g - lse_g) on the spot; in the fused H2O form it also adds W to the cumulative
+// scores and feeds the row's lowest-score slot. Longer splits, and a workgroup whose wait ran out, send the
+// logits to an fp32 scratch in bursts of 32 KB (a write stream mixed into the reads costs HBM far more than
+// its share of the bytes) and a last streaming kernel does the same work from there. A merge kernel
+// combines the splits' outputs. K and V are touched once: they are loaded non-temporally. No float atomics
+// anywhere.
 #include "kvx_common.h"
+#include <stdlib.h>
 
 namespace kvx {
 namespace {
@@ -42,6 +48,11 @@ struct DecodeParams {
   float* part_ml;  // (B, Hq, S, 2)
   float* lse_ws;   // (B, Hq)
   unsigned long long* best;  // fused H2O form: (value, slot) minimum per (b, kvh) row, else NULL
+  uint32_t* row_count;       // splits of a (b, kvh) row that have published their partial (resident form)
+  uint32_t* split_done;      // (B, Hkv, S): 1 where the split kernel itself turned its logits into weights
+  int32_t resident;          // the logits of a split stay in LDS
+  int32_t spin_limit;        // polls of row_count before a workgroup gives up and sends its logits out
+  int32_t poll_sleep;        // pause between two polls, in units of 512 cycles
   int32_t B, Hq, Hkv, kv_len, Tpad, num_splits, keys_per_split;
   int32_t Gr;  // query heads per KV head; the kernels' G is Gr rounded up to a power of two (heads Gr .. G - 1 are
                // dummies: zero queries, nothing of theirs is stored, their logits count for nothing)
@@ -72,17 +83,53 @@ __device__ __forceinline__ float row_group_sum(float x) {
   return x;
 }
 
+// Logits a workgroup holds in LDS: 64 KB where the merge buffer beside them is small enough for two workgroups
+// per compute unit (what the registers allow), else 32 KB.
+constexpr int logit_floats(int G, int D) { return G * D <= 512 ? 16384 : 8192; }
+constexpr int kCountStride = 64;  // a row's arrival counter has 256 bytes to itself: the polls of different rows go to different channels
 constexpr float kNegBig = -1.0e30f;  // running maximum before the first key (finite: no inf - inf)
 constexpr float kRescaleSlack = 8.0f;  // the running maximum moves only when a logit exceeds it by this
 
+// Monotone map float -> uint32 (a < b  <=>  key(a) < key(b)); -0.0 is folded onto +0.0.
+__device__ __forceinline__ uint32_t ordered_bits(float x) {
+  x += 0.0f;
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Base-2 log-sum-exp of a query head from its splits' (maximum, sum) pairs, by one wavefront: lane s takes
+// splits s, s + 64, ..., then butterflies; every lane returns the same bits. COHERENT: the pairs were
+// written by other workgroups of the running kernel (device-coherent loads).
+template <bool COHERENT>
+__device__ __forceinline__ float row_lse(const float* part_ml, int num_splits, int lane) {
+  const unsigned long long* ml = (const unsigned long long*)part_ml;
+  float M = -INFINITY, L = 0.0f;
+  for (int base = 0; base < num_splits; base += 64) {
+    const int sp = base + lane;
+    unsigned long long bits = 0xff800000ull;  // (maximum -inf, sum 0)
+    if (sp < num_splits) bits = COHERENT ? __hip_atomic_load(ml + sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : ml[sp];
+    const float m = __uint_as_float((uint32_t)bits), l = __uint_as_float((uint32_t)(bits >> 32));
+    const float Mn = fmaxf(M, m);
+    if (Mn > -INFINITY) L = L * fast_exp2(M - Mn) + l * fast_exp2(m - Mn);
+    M = Mn;
+  }
+  float Mw = M;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) Mw = fmaxf(Mw, __shfl_xor(Mw, off, 64));
+  L = M > -INFINITY ? L * fast_exp2(M - Mw) : 0.0f;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) L += __shfl_xor(L, off, 64);
+  return Mw + fast_log2(L);
+}
+
 template <int D, int G, int KV>
-__global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
   constexpr bool F16 = KV == KVX_KV_F16;  // element type of q, k, v, o
   constexpr int LPR = D / 8;     // lanes per row: a lane owns 8 consecutive d
   constexpr int RPI = 64 / LPR;  // rows per load instruction of a wavefront
   constexpr int U = 4;           // load instructions per step and tensor (even: rows pair up for dot2)
   constexpr int CH = U * RPI;    // keys per wavefront and step, contiguous
-  constexpr int LGK = 8192 / G;  // keys whose logits are gathered in LDS before they go out in one burst
+  constexpr int LGK = logit_floats(G, D) / G;  // keys whose logits are gathered in LDS before they go out in one burst
   __shared__ __align__(16) float lgbuf[LGK * G];  // [key][head]
   __shared__ float red[WAVES][G][D];
   __shared__ float rml[WAVES][G][2];
@@ -180,11 +227,22 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
       }
     }
     if (lgrow && dc == 0 && chunk0 < k_end) {
+      typedef float fV __attribute__((ext_vector_type(G >= 4 ? 4 : G)));  // a key's G logits leave in one or two stores
       float* dst = lgbuf + (chunk0 - lg_base + kk) * G;
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u) {
+        if constexpr (G == 1) {
+          dst[u * RPI] = s[u][0];
+        } else {
 #pragma unroll
-        for (int g = 0; g < G; ++g) dst[u * RPI * G + g] = s[u][g];
+          for (int h = 0; h < G; h += 4) {
+            fV t;
+#pragma unroll
+            for (int g = 0; g < (G >= 4 ? 4 : G); ++g) t[g] = s[u][h + g];
+            *(fV*)(dst + u * RPI * G + h) = t;
+          }
+        }
+      }
     }
     // running maximum: moved only when some logit of the wavefront exceeds it by the slack
     float smax[G];
@@ -237,6 +295,13 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     }
   };
 
+  // the gathered logits leave as one contiguous burst (keys past the end of a chunk are -inf)
+  auto flush_logits = [&]() {
+    const int nkeys = min(LGK, (k_end - lg_base + CH - 1) / CH * CH);
+    f32x4_t* dst = (f32x4_t*)(lgrow + (int64_t)lg_base * G);
+    for (int j = tid; j < nkeys * G / 4; j += NTHREADS) dst[j] = ((const f32x4_t*)lgbuf)[j];
+  };
+
   // Two steps in flight per wavefront: the loads of step i + 1 are issued before step i is consumed.
   const int nsteps = (k_end - k_begin + CH * WAVES - 1) / (CH * WAVES);
   const int stride = CH * WAVES;
@@ -255,14 +320,9 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     consume(rb, chunk + stride);
     __builtin_amdgcn_sched_barrier(0);
     chunk += 2 * stride;
-    if (lgrow && ((i + 2) % FLUSH_STEPS == 0 || i + 2 >= nsteps)) {
-      // the gathered logits leave as one contiguous burst (keys past the end of a chunk are -inf)
+    if (lgrow && !p.resident && ((i + 2) % FLUSH_STEPS == 0 || i + 2 >= nsteps)) {
       __syncthreads();
-      const int nkeys = min(LGK, (k_end - lg_base + CH - 1) / CH * CH);
-      f32x4_t* dst = (f32x4_t*)(lgrow + (int64_t)lg_base * G);
-      for (int j = tid; j < nkeys * G / 4; j += NTHREADS) {
-        dst[j] = ((const f32x4_t*)lgbuf)[j];
-      }
+      flush_logits();
       lg_base += LGK;
       __syncthreads();
     }
@@ -307,14 +367,98 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     const int64_t o = ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits + split;
     p.part_o[o * D + d] = x;
     if (d == 0) {
-      p.part_ml[o * 2] = M;
-      p.part_ml[o * 2 + 1] = l;
+      // read by the row's other workgroups while this kernel runs: a device-coherent store
+      const unsigned long long mlbits = ((unsigned long long)__float_as_uint(l) << 32) | __float_as_uint(M);
+      __hip_atomic_store((unsigned long long*)(p.part_ml + o * 2), mlbits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+  }
+  if (!lgrow || !p.resident) return;
+
+  // ---- the row's log-sum-exp, and this split's logits into weights, without leaving the chip --------
+  __shared__ float lse_sh[G];
+  __shared__ int row_ready;
+  __shared__ unsigned long long wbest[WAVES];
+  const int row = b * p.Hkv + kvh;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial above has reached device-coherent memory
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t* cnt = p.row_count + row * kCountStride;
+    __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int ok = 0;
+    for (int spin = 0; spin < p.spin_limit; ++spin) {  // bounded: a workgroup that gives up takes the scratch route
+      if (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)p.num_splits) {
+        ok = 1;
+        break;
+      }
+      for (int z = 0; z < p.poll_sleep; ++z) __builtin_amdgcn_s_sleep(8);
+    }
+    row_ready = ok;
+  }
+  __syncthreads();
+  if (!row_ready) {
+    flush_logits();
+    if (tid == 0) p.split_done[(int64_t)row * p.num_splits + split] = 0u;
+    return;
+  }
+  for (int g = wave; g < G; g += WAVES) {  // a wavefront per head: lane s takes splits s, s + 64, ...
+    float lse = INFINITY;  // dummy heads: exp2(x - inf) = 0
+    if (g < p.Gr) lse = row_lse<true>(p.part_ml + ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits * 2, p.num_splits, lane);
+    if (lane == 0) lse_sh[g] = lse;
+  }
+  __syncthreads();
+  float lse[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) lse[g] = lse_sh[g];
+  float* wr = p.w ? p.w + (int64_t)row * p.kv_len : nullptr;
+  float* sc = h2o ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
+  const int32_t* tpr = (h2o && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
+  const float inv_g = 1.0f / (float)p.Gr;
+  unsigned long long mine = ~0ull;
+  for (int k = k_begin + tid; k < k_end; k += NTHREADS) {
+    const float* lg = lgbuf + (k - k_begin) * G;
+    float acc = 0.0f;
+#pragma unroll
+    for (int g = 0; g < G; ++g) acc += fast_exp2(lg[g] - lse[g]);
+    acc *= inv_g;
+    if (wr) wr[k] = acc;
+    if (h2o) {
+      float val = sc[k] + acc;
+      sc[k] = val;
+      if (k < hh.limit) {
+        if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
+        const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
+        mine = key < mine ? key : mine;
+      }
+    }
+  }
+  if (h2o) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const unsigned long long o = __shfl_xor(mine, off, 64);
+      mine = o < mine ? o : mine;
+    }
+    if (lane == 0) wbest[wave] = mine;
+    __syncthreads();
+    if (tid == 0) {
+      unsigned long long mn = wbest[0];
+      for (int i = 1; i < WAVES; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
+      if (mn != ~0ull) atomicMin(p.best + row, mn);
+    }
+  }
+  if (tid == 0) p.split_done[(int64_t)row * p.num_splits + split] = 1u;
+}
+
+// Before the split kernel: no split of a row has arrived, no row has a lowest-score slot yet.
+__global__ void decode_init_kernel(uint32_t* row_count, unsigned long long* best, int rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) {
+    if (row_count) row_count[i * kCountStride] = 0u;
+    if (best) best[i] = ~0ull;
   }
 }
 
 // Combine the splits of one (b, query head): 4 groups of D threads each take a quarter of the
-// splits, then the groups are added through LDS. Also produces the base-2 log-sum-exp.
+// splits, then the groups are added through LDS. Its first wavefront also produces the base-2 log-sum-exp.
 template <int D, bool F16>
 __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams p) {
   __shared__ float red[4][D + 1];
@@ -329,6 +473,12 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, off, 64));
     if (threadIdx.x == 0) sM = mloc;
+    // the log-sum-exp by the routine the split kernel uses for its own weights: the same bits on either route
+    const float lse = row_lse<false>(ml, p.num_splits, threadIdx.x);
+    if (threadIdx.x == 0) {
+      p.lse_ws[bh] = lse;
+      if (p.lse_out) p.lse_out[bh] = lse;
+    }
   }
   __syncthreads();
   const float M = sM;
@@ -347,27 +497,12 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
     const float r = a4 / l4;
     const float other = __shfl_xor(r, 1, 64);
     if ((d & 1) == 0) *(uint32_t*)(p.o + b * p.o_sb + hqi * p.o_sh + d) = pack_pair<F16>(r, other);
-    if (d == 0) {
-      const float lse = M + fast_log2(l4);
-      p.lse_ws[bh] = lse;
-      if (p.lse_out) p.lse_out[bh] = lse;
-      // fused H2O form: reset the running minimum of the KV head's row for the weights kernel
-      if (p.best && hqi % (p.Hq / p.Hkv) == 0) {
-        p.best[b * p.Hkv + hqi / (p.Hq / p.Hkv)] = ~0ull;
-      }
-    }
   }
 }
 
-// Monotone map float -> uint32 (a < b  <=>  key(a) < key(b)); -0.0 is folded onto +0.0.
-__device__ __forceinline__ uint32_t ordered_bits(float x) {
-  x += 0.0f;
-  const uint32_t u = __float_as_uint(x);
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
 // W[b, kvh, k] = (1/G) sum_g exp2(logit[b, kvh, k, g] - lse[b, kvh*G+g]); one key per lane and pass,
-// 4096 keys per workgroup. With H2O set it also does the cache's score update and eviction choice
+// 4096 keys per workgroup, for the splits whose logits went to the scratch (in the resident form: those
+// whose wait ran out, normally none). With H2O set it also does the cache's score update and eviction choice
 // in the same pass (keys_values/kvcache/h2o.py:175-196, keys_values/kvcache/attn_weights.py:773-774
 // for one slot): scores += W, then the (value, slot) minimum of the row through an integer atomicMin.
 template <int G, bool H2O>
@@ -375,6 +510,13 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams 
   typedef float fG __attribute__((ext_vector_type(G >= 4 ? 4 : (G == 2 ? 2 : 1))));
   constexpr int NV = G >= 4 ? G / 4 : 1;
   const int kvh = blockIdx.y, b = blockIdx.z;
+  const uint32_t* done = p.resident ? p.split_done + ((int64_t)b * p.Hkv + kvh) * p.num_splits : nullptr;
+  if (done) {
+    const int s0 = blockIdx.x * 4096 / p.keys_per_split, s1 = min((blockIdx.x * 4096 + 4095) / p.keys_per_split, p.num_splits - 1);
+    int pending = 0;
+    for (int sp = s0 + (int)threadIdx.x; sp <= s1; sp += 256) pending |= done[sp] == 0u;
+    if (!__syncthreads_or(pending)) return;
+  }
   float lse[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) lse[g] = g < p.Gr ? p.lse_ws[(int64_t)b * p.Hq + kvh * p.Gr + g] : INFINITY;  // exp2(x - inf) = 0
@@ -395,6 +537,7 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams 
   for (int it = 0; it < PASSES; ++it) {
     const int k = blockIdx.x * 4096 + it * 256 + threadIdx.x;
     if (k >= p.kv_len) break;
+    if (done && done[k / p.keys_per_split]) continue;
     float acc = 0.0f;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -442,20 +585,34 @@ __global__ void decode_argmin_finish_kernel(const unsigned long long* best, int3
 }
 
 struct Plan {
-  int G, num_splits, keys_per_split, Tpad;
-  size_t off_logits, off_part_o, off_part_ml, off_lse, off_best, total;
+  int G, num_splits, keys_per_split, Tpad, resident;
+  size_t off_logits, off_part_o, off_part_ml, off_lse, off_best, off_count, off_done, total;
 };
+
+// KVX_DECODE_RESIDENT=0 sends every split's logits through the scratch; KVX_DECODE_SPIN_LIMIT bounds the
+// wait for a row's other splits (0: no wait, every workgroup takes the scratch route). Read at every call.
+int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e && *e ? atoi(e) : dflt;
+}
 
 Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
   const int gr = a.Hq / a.Hkv;
   pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : 8));
-  // About 16 workgroups per compute unit over the whole grid, each with at least 1024 keys.
+  // About 16 workgroups per compute unit over the whole grid, each with at least 1024 keys. When the weights
+  // are wanted, 8: a split that waits for its row holds its place on the compute unit, and the fewer,
+  // longer splits wait a smaller part of their time (measured: 4 rounds of 2 workgroups per compute unit
+  // beat 8 by 2 %, 6 are 5 % worse); and if a split's logits then do not fit in LDS, as many more splits as make them fit.
+  const bool weights = a.w || fused_h2o;
+  const int allow_resident = weights ? env_int("KVX_DECODE_RESIDENT", 1) : 0;
+  const int lgk = logit_floats(pl.G, a.D) / pl.G;
   int splits = a.num_splits;
   if (splits <= 0) {
     const int rows = a.B * a.Hkv;
-    splits = (16 * num_cus() + rows - 1) / rows;
+    splits = ((allow_resident ? 8 : 16) * num_cus() + rows - 1) / rows;
     splits = min(splits, (a.kv_len + 1023) / 1024);
+    if (allow_resident) splits = max(splits, (a.kv_len + lgk - 1) / lgk);
   }
   splits = max(1, min(splits, 512));
   int kps = (a.kv_len + splits - 1) / splits;
@@ -465,7 +622,7 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   pl.Tpad = ((a.kv_len + 63) / 64) * 64;
   size_t off = 0;
   pl.off_logits = off;
-  off += (a.w || fused_h2o) ? (size_t)a.B * a.Hkv * pl.G * pl.Tpad * 4 : 0;
+  off += weights ? (size_t)a.B * a.Hkv * pl.G * pl.Tpad * 4 : 0;
   pl.off_part_o = off;
   off += (size_t)a.B * a.Hq * pl.num_splits * a.D * 4;
   pl.off_part_ml = off;
@@ -475,6 +632,12 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   off = (off + 7) & ~(size_t)7;
   pl.off_best = off;
   off += fused_h2o ? (size_t)a.B * a.Hkv * 8 : 0;
+  pl.resident = allow_resident && kps <= lgk;
+  off = (off + 255) & ~(size_t)255;
+  pl.off_count = off;
+  off += pl.resident ? (size_t)a.B * a.Hkv * kCountStride * 4 : 0;
+  pl.off_done = off;
+  off += pl.resident ? (size_t)a.B * a.Hkv * pl.num_splits * 4 : 0;
   pl.total = (off + 255) & ~(size_t)255;
   return pl;
 }
@@ -482,12 +645,19 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
 template <int D, int G>
 int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
-  if constexpr (D <= 128) {
-    if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p);
-    else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p);
+  const int rows = p.B * p.Hkv;
+  if (p.resident || hh) {
+    hipLaunchKernelGGL(decode_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.resident ? p.row_count : nullptr, hh ? p.best : nullptr, rows);
+    KVX_HIP(hipGetLastError());
   }
-  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p);
-  else if (kv == KVX_KV_BF16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p);
+  const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
+  const int h2o = hh != nullptr;
+  if constexpr (D <= 128) {
+    if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+  }
+  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+  else if (kv == KVX_KV_BF16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
   KVX_HIP(hipGetLastError());
   if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_merge_kernel<D, true>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
   else hipLaunchKernelGGL((decode_merge_kernel<D, false>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
@@ -496,7 +666,6 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
   if (hh) {
     hipLaunchKernelGGL((decode_weights_kernel<G, true>), wgrid, dim3(256), 0, st, p, *hh);
     KVX_HIP(hipGetLastError());
-    const int rows = p.B * p.Hkv;
     hipLaunchKernelGGL(decode_argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.best, hh->next_index, rows);
     KVX_HIP(hipGetLastError());
   } else if (p.w) {
@@ -544,6 +713,11 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.part_ml = (float*)(ws + pl.off_part_ml);
   p.lse_ws = (float*)(ws + pl.off_lse);
   p.best = hh ? (unsigned long long*)(ws + pl.off_best) : nullptr;
+  p.row_count = (uint32_t*)(ws + pl.off_count);
+  p.split_done = (uint32_t*)(ws + pl.off_done);
+  p.resident = pl.resident;
+  p.spin_limit = env_int("KVX_DECODE_SPIN_LIMIT", 1 << 18);
+  p.poll_sleep = env_int("KVX_DECODE_POLL_SLEEP", 4);
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
   p.Gr = a.Hq / a.Hkv;
   KVX_REQUIRE(p.Gr <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);

@@ -29,3 +29,17 @@ def gpu(kvx):
     assert torch.cuda.is_available(), "GPU tests need a ROCm device"
     assert kvx.kvx_device_count() > 0, "libkvx sees no gfx950 device"
     return torch.device("cuda", 0)
+
+
+# How the logits become weights: inside the split kernel once the row's other splits have arrived
+# (the default), through the scratch buffer and the weights kernel (resident form switched off), and
+# the bounded wait running out in every workgroup (limit 0) or in most of them (limit 1).
+DECODE_ROUTES = {"resident": {}, "scratch": {"KVX_DECODE_RESIDENT": "0"}, "no-wait": {"KVX_DECODE_SPIN_LIMIT": "0"},
+                 "one-poll": {"KVX_DECODE_SPIN_LIMIT": "1"}}
+
+
+@pytest.fixture(params=list(DECODE_ROUTES))
+def decode_route(request, monkeypatch):
+    for name, value in DECODE_ROUTES[request.param].items():
+        monkeypatch.setenv(name, value)
+    return request.param

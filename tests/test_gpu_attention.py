@@ -150,8 +150,8 @@ DECODE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,T,D,splits", DECODE_CASES)
-def test_decode_with_weights(gpu, B, Hq, Hkv, T, D, splits):
+@pytest.mark.parametrize("B,Hq,Hkv,T,D,splits", DECODE_CASES + [(2, 8, 2, 20000, 128, 0), (1, 8, 1, 9000, 64, 0)])
+def test_decode_with_weights(gpu, decode_route, B, Hq, Hkv, T, D, splits):
     q, k, v, _ = make_qkv(900 + T, B, Hq, Hkv, 1, T, D)
     scale = 1.0 / math.sqrt(D)
     o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, T - 1, None)

@@ -418,8 +418,9 @@ def test_attention_over_uint8_cache(kvx, gpu):
     (1, 2, 1, 17, 64, 17, False, True),
     (2, 6, 2, 600, 128, 600, False, False),
     (1, 5, 1, 300, 64, 256, True, True),
+    (1, 8, 2, 12000, 128, 11000, True, False),
 ])
-def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, B, Hq, Hkv, T, D, limit, normalize, quantized):
+def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, decode_route, B, Hq, Hkv, T, D, limit, normalize, quantized):
     """kvx_sdpa_decode_h2o == kvx_sdpa_decode (with weights) followed by kvx_h2o_update_select(k=1),
     and both match the oracle."""
     q, k, v, _ = make_qkv(50 + T, B, Hq, Hkv, 1, T, D)
