@@ -142,8 +142,11 @@ int kvx_sdpa_prefill_weights(const kvx_sdpa_args* args, void* stream);
  * (keys_values/attention/flashinfer_wrapper.py:471-481, keys_values/attention/flashinfer_ops.py:250-275).
  * Stands in for sdpa_decode of the reference extension (keys_values/csrc/bindings.cpp:86-489) and
  * optimized_batched_decode_kernel (keys_values/csrc/kernels/sdpa_decode.cu:616-898). One workgroup
- * per (batch, KV head, split) serves all G query heads, so K and V are read once.
- * The workspace holds the fp32 logits (B, Hq, kv_len) and the split partials. args->lse optional. */
+ * per (batch, KV head, split) serves all G query heads, so K and V are read once. With args->w set, a
+ * split keeps its logits on the chip, waits (boundedly) until the other splits of its (batch, KV head) row
+ * have published their partial maxima and sums, and writes its part of W itself; the workspace holds
+ * the split partials, the rows' arrival counters and room for the fp32 logits (B, Hq, kv_len) of the
+ * splits that are too long for that or whose wait ran out. args->lse optional. */
 int kvx_sdpa_decode(const kvx_sdpa_args* args, void* stream);
 size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* args);
 
