@@ -54,9 +54,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (KiB per dispatch, one counter per run, on these same workloads), each scaled by what the counter
 # reads for the `calib` launch of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
 TRAFFIC_BYTES = {
-    "prefill": int((70202.9 * 2.000 + 33280.0) * 1024),    # sdpa_prefill_kernel<128, KVX_KV_BF16>
-    "decode": int((2099006.6 * 2.000 + 139780.7) * 1024),  # decode_split_kernel<128, 4, KVX_KV_BF16>
-    "quantize": int((65573.7 * 2.000 + 69632.0) * 1024),   # quantize_rows_kernel<128>
+    "prefill": int((70196.3 * 2.000 + 33283.4) * 1024),    # sdpa_prefill_kernel<128, KVX_KV_BF16>
+    "decode": int((2115128.0 * 2.000 + 37312.0) * 1024),   # decode_split_kernel<128, 4, KVX_KV_BF16>
+    "quantize": int((65573.9 * 2.000 + 69632.0) * 1024),   # quantize_rows_kernel<128>
 }
 
 
