@@ -49,6 +49,9 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
               "%s: sizes must be positive (B=%d Hq=%d Hkv=%d q_len=%d kv_len=%d)", who, a->B, a->Hq, a->Hkv, a->q_len,
               a->kv_len);
   KVX_REQUIRE(a->Hq % a->Hkv == 0, KVX_ERR_INVALID, "%s: Hq=%d must be a multiple of Hkv=%d", who, a->Hq, a->Hkv);
+  // batch and head indices are grid dimensions, and B * Hq rows are counted in 32 bits
+  KVX_REQUIRE(a->B <= 65535 && a->Hq <= 65535 && (int64_t)a->B * a->Hq < ((int64_t)1 << 24), KVX_ERR_UNSUPPORTED,
+              "%s: B=%d, Hq=%d beyond 65535 each or 2^24 together", who, a->B, a->Hq);
   KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4 || a->kv_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED,
               "%s: unknown kv_dtype %d", who, a->kv_dtype);
   KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,

@@ -716,7 +716,7 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.row_count = (uint32_t*)(ws + pl.off_count);
   p.split_done = (uint32_t*)(ws + pl.off_done);
   p.resident = pl.resident;
-  p.spin_limit = env_int("KVX_DECODE_SPIN_LIMIT", 1 << 18);
+  p.spin_limit = env_int("KVX_DECODE_SPIN_LIMIT", 1 << 15);
   p.poll_sleep = env_int("KVX_DECODE_POLL_SLEEP", 4);
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
   p.Gr = a.Hq / a.Hkv;

@@ -99,7 +99,8 @@ class H2OKVCache:
         # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
         # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
         self.dequantize_chunk_rows = dequantize_chunk_rows
-        # overlap_select: launch the score update + eviction choice of a chunk step on a second stream, so
+        # overlap_select: launch the score update + eviction choice of a chunk step (and, for a long chunk over
+        # a quantised store, the score-sum pass before them) on a second stream, so
         # that it runs beside whatever the caller enqueues next; the next forward and next_positions() wait
         # for it. The attributes scores, token_pos and _next_index are plain tensors: a caller that reads
         # them directly calls wait_for_selection() first.
@@ -212,6 +213,11 @@ class H2OKVCache:
         if self.current_length is None:
             raise IndexError("Cache is not initialized, call 'prefill' first")
         return self.token_pos[: self.batch_size, :, : self.current_length]
+
+    def _second_stream(self) -> torch.cuda.Stream:
+        if self._side_stream is None:
+            self._side_stream = torch.cuda.Stream(self.device)  # default priority
+        return self._side_stream
 
     def wait_for_selection(self):
         """Make the caller's stream wait for an eviction choice still running on the second stream."""
@@ -374,6 +380,20 @@ class H2OKVCache:
                 # once per wavefront whatever the chunk length, and reads half the bytes)
                 kd, vd = self._dequantized(b, T)
                 out, _, lse = ops.prefill_core(query, kd, vd, self.scale_factor, input_pos, tp, return_lse=True, output_transposed=True)
+                if self._overlap:
+                    # the score-sum pass too runs beside the caller's next launches: nothing needs the score-sums
+                    # before the next chunk's eviction choice
+                    main = torch.cuda.current_stream(self.device)
+                    side = self._second_stream()
+                    ready = torch.cuda.Event()
+                    ready.record(main)
+                    with torch.cuda.stream(side):
+                        side.wait_event(ready)
+                        w = ops.score_sum_core(query, kc, lse, self.scale_factor, input_pos, tp, quant=quant)
+                        self._update(w, num)
+                    query.record_stream(side)
+                    lse.record_stream(side)
+                    return out.reshape(b, num, hq * d)
                 w = ops.score_sum_core(query, kc, lse, self.scale_factor, input_pos, tp, quant=quant)
             else:
                 out, w, _ = ops.prefill_core(query, kc, vc, self.scale_factor, input_pos, tp, return_weights=True,
@@ -574,8 +594,7 @@ class H2OKVCache:
                 _lib.check(lib.kvx_h2o_update_select(ctypes.byref(a), _lib.stream_ptr(self.device)))
             else:
                 main = torch.cuda.current_stream(self.device)
-                if self._side_stream is None:
-                    self._side_stream = torch.cuda.Stream(self.device)  # default priority
+                self._second_stream()
                 ready = torch.cuda.Event()
                 ready.record(main)
                 with torch.cuda.stream(self._side_stream):

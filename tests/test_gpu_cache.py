@@ -579,3 +579,36 @@ def test_overlapped_selection_equals_in_order_selection(gpu):
         assert torch.equal(a.scores, b.scores) and torch.equal(a.token_pos, b.token_pos)
         assert torch.equal(a.k, b.k) and torch.equal(a.v, b.v)
         pos += chunk
+
+
+@pytest.mark.parametrize("bits,grace", [(8, 0), (4, 0), (8, 40)])
+def test_overlapped_score_sum_pass_equals_in_order_pass(gpu, bits, grace):
+    """Long chunks over a quantised store with overlap_select: the score-sum pass, the score update and the
+    eviction choice all run on the second stream. Outputs, scores, stores and choices equal the in-order
+    cache's bit for bit, also when the ring of recent tokens moves."""
+    B, Hq, Hkv, L, D, chunk = 2, 8, 2, 1024, 128, 64
+    gen = torch.Generator().manual_seed(123 + bits + grace)
+    total = L + 6 * chunk
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16).to(gpu)
+    params = KVCacheParams(B, Hkv, L, D, Hq)
+    kw = dict(max_chunk_size=chunk, quantized=True, num_bits=bits, device=gpu, dequantize_chunk_rows=1, grace_period=grace)
+    plain = H2OKVCache(params, **kw)
+    beside = H2OKVCache(params, overlap_select=True, **kw)
+    busy = torch.randn(1024, 1024, device=gpu)
+    for cache in (plain, beside):
+        cache.forward(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L])
+    pos = L
+    for step in range(6):
+        sl = slice(pos, pos + chunk)
+        o1 = plain.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        o2 = beside.forward(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl])
+        for _ in range(3):  # the caller's own work, enqueued while the second stream may still be running
+            busy = (busy @ busy).clamp_(-1, 1)
+        assert torch.equal(plain.next_positions(chunk), beside.next_positions(chunk))  # waits for the second stream
+        torch.cuda.synchronize()
+        assert torch.equal(o1, o2)
+        assert torch.equal(plain.scores, beside.scores) and torch.equal(plain.token_pos, beside.token_pos)
+        assert torch.equal(plain.k, beside.k) and torch.equal(plain.v, beside.v)
+        pos += chunk
