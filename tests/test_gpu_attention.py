@@ -351,3 +351,26 @@ def test_gate_mirrors_the_reference(gpu):
     assert out.shape == (B, Hq, q_len, D) and out.dtype == torch.float16
     check_o(out, o_ref)
     check_w(w, w_ref, q_len)
+
+
+def test_decode_with_weights_beside_other_work(gpu):
+    """The split kernel's wait for its row's other splits while another stream keeps the compute units busy
+    (its workgroups then start at scattered times): same bits as on an idle device."""
+    B, Hq, Hkv, T, D = 2, 8, 2, 30000, 128
+    q, k, v, _ = make_qkv(4242, B, Hq, Hkv, 1, T, D)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    scale = 1.0 / math.sqrt(D)
+    out0, w0, lse0 = ops.decode_core(qg, kg, vg, scale, return_weights=True, return_lse=True)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(gpu)
+    busy = torch.randn(4096, 4096, device=gpu, dtype=torch.bfloat16)
+    for _ in range(3):
+        with torch.cuda.stream(side):
+            for _ in range(20):
+                busy = (busy @ busy).clamp_(-1, 1)
+        out1, w1, lse1 = ops.decode_core(qg, kg, vg, scale, return_weights=True, return_lse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out0, out1) and torch.equal(w0, w1) and torch.equal(lse0, lse1)
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, T - 1, None)
+    check_o(out0.unsqueeze(2), o_ref)
+    check_w(w0, w_ref, 1)
