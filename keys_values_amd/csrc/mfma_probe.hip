@@ -7,6 +7,8 @@
 //   - nothing, with random or all-zero operands (the clock follows the power the operands draw);
 //   - K independent v_fma_f32, or 2 v_exp_f32: does vector work fit beside the matrix instruction;
 //   - the vector work of one attention slot (fma, exp, half a bf16 pack) and an LDS fragment read;
+//   - a 1 KB transfer from L2 straight into LDS (global_load_lds_dwordx4) every K rounds: what the K / V tile
+//     stream of the attention kernels (one transfer per 4 matrix instructions and wavefront) costs;
 //   and the same vector work alone, at one and two wavefronts per SIMD: the issue rate of a single wavefront.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -26,13 +28,14 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
     }                                                                        \
   } while (0)
 
-enum Mix { NONE = 0, FMA = 1, EXP = 2, SLOT = 3 };
+enum Mix { NONE = 0, FMA = 1, EXP = 2, SLOT = 3, DMA = 4 };
 constexpr int ROUNDS = 16;  // rounds per loop iteration
 
 // MF: issue the matrix instruction; MIX / K: the vector work of a round; RANDOM: operand bits
 template <bool MF, int MIX, int K>
-__global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* out, long long* cyc, int iters, int random) {
+__global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* out, long long* cyc, int iters, int random, const char* stream) {
   __shared__ u32x4 sm[1024];
+  __shared__ u32x4 landing[4][4][64];  // per wavefront: four 1 KB landing places for the transfers
   for (int i = threadIdx.x; i < 1024; i += 256) sm[i] = u32x4{0x3f003f00u, 0x3f003f00u, 0x3f003f00u, 0x3f003f00u};
   __syncthreads();
   u32x4 ar = *(const u32x4*)(rnd + ((threadIdx.x * 4 + blockIdx.x * 64) & 4092));
@@ -50,6 +53,12 @@ __global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* 
     for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
   u32x4 frag = ar;
   const u32x4 __attribute__((address_space(3)))* lp = (const u32x4 __attribute__((address_space(3)))*)sm + ((threadIdx.x & 63) ^ ((threadIdx.x >> 2) & 15));
+  // transfers walk a 256 KB window of `stream` shared by the workgroups of one XCD (workgroup i runs on XCD i % 8),
+  // as the row blocks of one KV head share its K / V tiles: L2 hits after the first pass
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(&landing[wave][0][0]));
+  const char* window = stream + (size_t)(blockIdx.x & 7) * 262144;
+  uint32_t voff = (threadIdx.x & 63) * 16 + wave * 65536;
   const long long c0 = clock64(), w0 = wall_clock64();
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -70,15 +79,21 @@ __global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* 
         if (j & 1) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pk) : "v"(pe), "v"(t));
         else pe = t;
       }
+      if (MIX == DMA && j % K == 0) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds0 + 1024u * ((j / K) & 3)), "v"(voff), "s"(window) : "memory", "m0");
+        voff = (voff & 0xffff0000u) | ((voff + 1024u) & 0xffffu);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
+    // the transfers of the iteration before have landed; those just issued stay in flight (a kernel that double-buffers its tiles waits like this)
+    if (MIX == DMA) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ROUNDS / (K > 0 ? K : 1)) : "memory");
     if (MF && (it & 63) == 63)
       for (int j = 0; j < 4; ++j)
         for (int i = 0; i < 16; ++i) acc[j][i] *= 1e-30f;  // keeps the sums finite
     if (MIX == SLOT) br[0] ^= pk & 1u;
   }
   const long long c1 = clock64(), w1 = wall_clock64();
-  float s = pe + (float)pk + __uint_as_float(frag[0]);
+  float s = pe + (float)pk + __uint_as_float(frag[0]) + (MIX == DMA ? __uint_as_float(landing[wave][1][threadIdx.x & 63][0]) : 0.0f);
   for (int i = 0; i < 8; ++i) s += v[i];
   for (int j = 0; j < 4; ++j)
     for (int i = 0; i < 16; ++i) s += acc[j][i];
@@ -92,6 +107,7 @@ __global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* 
 static uint32_t* g_rnd;
 static float* g_out;
 static long long* g_cyc;
+static char* g_stream;
 static int g_cus;
 
 template <bool MF, int MIX, int K>
@@ -100,10 +116,10 @@ int run(const char* name, int waves_per_simd, int random) {
   hipEvent_t e0, e1;
   CK(hipEventCreate(&e0));
   CK(hipEventCreate(&e1));
-  hipLaunchKernelGGL((probe_kernel<MF, MIX, K>), dim3(blocks), dim3(256), 0, 0, g_rnd, g_out, g_cyc, iters, random);
+  hipLaunchKernelGGL((probe_kernel<MF, MIX, K>), dim3(blocks), dim3(256), 0, 0, g_rnd, g_out, g_cyc, iters, random, g_stream);
   CK(hipDeviceSynchronize());
   CK(hipEventRecord(e0));
-  hipLaunchKernelGGL((probe_kernel<MF, MIX, K>), dim3(blocks), dim3(256), 0, 0, g_rnd, g_out, g_cyc, iters, random);
+  hipLaunchKernelGGL((probe_kernel<MF, MIX, K>), dim3(blocks), dim3(256), 0, 0, g_rnd, g_out, g_cyc, iters, random, g_stream);
   CK(hipEventRecord(e1));
   CK(hipEventSynchronize(e1));
   float ms;
@@ -130,6 +146,8 @@ int main() {
   CK(hipMalloc(&g_rnd, 16384));
   CK(hipMalloc(&g_out, 8192 * 256 * 4));
   CK(hipMalloc(&g_cyc, 8192 * 16));
+  CK(hipMalloc(&g_stream, (size_t)8 * 262144));
+  CK(hipMemset(g_stream, 0x3c, (size_t)8 * 262144));
   static uint32_t h[4096];
   srand(5);
   for (auto& x : h) x = ((uint32_t)rand() << 16) ^ (uint32_t)rand();
@@ -143,6 +161,9 @@ int main() {
     rc |= run<true, FMA, 8>("matrix instruction + 8 fma", wps, 1);
     rc |= run<true, EXP, 2>("matrix instruction + 2 exp", wps, 1);
     rc |= run<true, SLOT, 0>("matrix instruction + fma, exp, pack/2, LDS read/2", wps, 1);
+    rc |= run<true, DMA, 8>("matrix instruction + 1 KB L2->LDS per 8", wps, 1);
+    rc |= run<true, DMA, 4>("matrix instruction + 1 KB L2->LDS per 4", wps, 1);
+    rc |= run<true, DMA, 2>("matrix instruction + 1 KB L2->LDS per 2", wps, 1);
     rc |= run<false, FMA, 6>("6 fma", wps, 1);
     rc |= run<false, EXP, 2>("2 exp", wps, 1);
     rc |= run<false, SLOT, 0>("fma, exp, pack/2, LDS read/2", wps, 1);
