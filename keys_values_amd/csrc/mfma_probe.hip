@@ -12,6 +12,7 @@
 //   - everything the attention kernel issues per matrix instruction, as its counters give it (4.6 vector instructions:
 //     fma, exp, add, half a pack, a third of a max3, one more; 1.5 LDS reads of 8 bytes per lane; the tile stream),
 //     with no dependence of one round on another and no barrier: what that instruction mix alone allows;
+//   - the same for the score-sum kernel (two elements per matrix instruction: fma, exp, add each; a 16-byte LDS read per two);
 //   and the same vector work alone, at one and two wavefronts per SIMD: the issue rate of a single wavefront.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -32,7 +33,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
     }                                                                        \
   } while (0)
 
-enum Mix { NONE = 0, FMA = 1, EXP = 2, SLOT = 3, DMA = 4, ATT = 5 };
+enum Mix { NONE = 0, FMA = 1, EXP = 2, SLOT = 3, DMA = 4, ATT = 5, SSUM = 6 };
 constexpr int ROUNDS = 16;  // rounds per loop iteration
 
 // MF: issue the matrix instruction; MIX / K: the vector work of a round; RANDOM: operand bits
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* 
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int j = 0; j < ROUNDS; ++j) {
-      if (MF) acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, MIX == ATT ? ring[j & 3] : (MIX == SLOT ? frag : ar)), __builtin_bit_cast(bf16x8, br), acc[j & 3], 0, 0, 0);
+      if (MF) acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, MIX == ATT ? ring[j & 3] : (MIX == SSUM ? ring[(j / 2) & 3] : (MIX == SLOT ? frag : ar))), __builtin_bit_cast(bf16x8, br), acc[j & 3], 0, 0, 0);
       if (MIX == FMA) {
 #pragma unroll
         for (int i = 0; i < K; ++i) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[i % 8]) : "v"(w), "v"(v[(i + 3) % 8]));
@@ -107,6 +108,13 @@ __global__ __launch_bounds__(256) void probe_kernel(const uint32_t* rnd, float* 
         if (j & 1) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pk) : "v"(pe), "v"(t));
         else pe = t;
         if (j % 3 == 0) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mc) : "v"(t), "v"(pe));
+      }
+      if (MIX == SSUM) {  // the score-sum kernel: two elements per matrix instruction (fma, exp, add each), a 16-byte LDS read per two
+        if ((j & 1) == 0) ring[(j / 2 + 3) & 3] = lp[64 * ((j >> 1) & 7)];
+        float t0 = __builtin_amdgcn_exp2f(__builtin_fmaf(v[j & 7], w, -mc));
+        float t1 = __builtin_amdgcn_exp2f(__builtin_fmaf(v[(j + 1) & 7], w, -mc));
+        asm volatile("" : "+v"(t0), "+v"(t1));
+        pe += t0 + t1;
       }
       if ((MIX == DMA || MIX == ATT) && j % (MIX == ATT ? 4 : K) == 0) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds0 + 1024u * ((j / K) & 3)), "v"(voff), "s"(window) : "memory", "m0");
@@ -195,6 +203,7 @@ int main() {
     rc |= run<true, DMA, 4>("matrix instruction + 1 KB L2->LDS per 4", wps, 1);
     rc |= run<true, DMA, 2>("matrix instruction + 1 KB L2->LDS per 2", wps, 1);
     rc |= run<true, ATT, 0>("matrix instruction + the attention kernel's mix", wps, 1);
+    rc |= run<true, SSUM, 0>("matrix instruction + the score-sum kernel's mix", wps, 1);
     rc |= run<false, FMA, 6>("6 fma", wps, 1);
     rc |= run<false, EXP, 2>("2 exp", wps, 1);
     rc |= run<false, SLOT, 0>("fma, exp, pack/2, LDS read/2", wps, 1);
