@@ -8,7 +8,7 @@
 // Key-stationary: a wavefront keeps the K rows of its 64 keys in registers as MFMA B operands for
 // the whole kernel and owns those 64 outputs, so W needs no atomics and is bit-reproducible. The
 // G*q_len packed query rows (row r = query r / G, head r % G) stream through LDS in tiles of 64 rows,
-// double-buffered, shared by the four wavefronts of the workgroup (256 keys per workgroup).
+// double-buffered, shared by the four or eight wavefronts of the workgroup (256 or 512 keys per workgroup).
 // S = Q K^T is computed with rows along M, so a lane owns one key column: the sum over queries is a
 // per-lane running sum and the two halves of the wavefront are added once at the end.
 #include <type_traits>
@@ -20,9 +20,9 @@ namespace {
 
 constexpr int BQ = 64;    // query rows per LDS tile
 constexpr int NW = 64;    // keys per wavefront
-constexpr int WAVES = 4;
-constexpr int NTHREADS = WAVES * 64;
-constexpr int BK = NW * WAVES;  // keys per workgroup
+// Wavefronts per workgroup, a template argument W: 8 (512 keys per workgroup, one workgroup per compute unit: the
+// Q tile staged into LDS serves twice the keys, 4 % on the kernel) when that still gives every compute unit a
+// workgroup, else 4 (256 keys, two workgroups per compute unit).
 
 struct ScoreParams {
   const uint16_t* q;
@@ -45,9 +45,9 @@ struct alignas(16) Smem {
   int32_t qpos[3][BQ];
 };
 
-template <int D>
+template <int D, int W>
 struct QStage {
-  static constexpr int QCH = (BQ * D / 8) / NTHREADS;  // 4 (D=128), 2 (D=64)
+  static constexpr int QCH = (BQ * D / 8) / (64 * W);  // W = 4: 4 (D=128), 2 (D=64)
   u32x4_t qr[QCH];
   float lse;
   int32_t qpos;
@@ -56,11 +56,12 @@ struct QStage {
 // Streams the packed query rows (row r = query r / G, head r % G) of one (batch, KV head) pair.
 // The (query, head) of each row this thread loads is advanced incrementally from tile to tile,
 // so the loop has no integer division.
-template <int D>
+template <int D, int W>
 struct QLoader {
+  static constexpr int NTHREADS = 64 * W;
   static constexpr int CPR = D / 8;
   static constexpr int RPI = NTHREADS / CPR;
-  static constexpr int QCH = QStage<D>::QCH;
+  static constexpr int QCH = QStage<D, W>::QCH;
   const uint16_t* qbase;  // (b, first head of the group)
   const float* lbase;     // lse + b * q_len * Hq + kvh * G
   int64_t q_sh, q_st;
@@ -92,7 +93,7 @@ struct QLoader {
   }
 
   // fetch the tile whose first row is row0, then step the row bookkeeping to the next tile
-  __device__ __forceinline__ void fetch(QStage<D>& s, int row0, int tid) {
+  __device__ __forceinline__ void fetch(QStage<D, W>& s, int row0, int tid) {
     if (dg == 0) {
       // G divides the tile height: every row keeps its head and moves by BQ / G queries per tile.
       // Rows past the end read row 0 (finite data); their lse = +inf makes their weight zero.
@@ -130,7 +131,7 @@ struct QLoader {
     }
   }
 
-  __device__ __forceinline__ void commit(const QStage<D>& s, Smem<D>& sm, int buf, int buf3, int tid) const {
+  __device__ __forceinline__ void commit(const QStage<D, W>& s, Smem<D>& sm, int buf, int buf3, int tid) const {
 #pragma unroll
     for (int i = 0; i < QCH; ++i) sm.q[buf][row_in + i * RPI][col] = s.qr[i];
     if (tid < BQ) {
@@ -140,8 +141,9 @@ struct QLoader {
   }
 };
 
-template <int D, int KV>
-__global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
+template <int D, int KV, int W>
+__global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
+  constexpr int BK = NW * W;  // keys per workgroup
   constexpr bool F16 = KV == KVX_KV_F16;  // element type of q and k
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
@@ -195,9 +197,9 @@ __global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(c
 
   float wacc[2] = {0.0f, 0.0f};
   const int num_qt = (p.R + BQ - 1) / BQ;
-  QLoader<D> ld;
+  QLoader<D, W> ld;
   ld.init(p, b, kvh, tid);
-  QStage<D> st;
+  QStage<D, W> st;
 
   // S block = 32 query rows x 64 keys: Q rows come from LDS (A operand), K sits in registers.
   auto mfma_block = [&](f32x16_t (&s)[2], int buf, int mt) {
@@ -313,8 +315,16 @@ __global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void score_sum_kernel(c
 
 template <int D, int KV>
 int launch_t(const ScoreParams& p, hipStream_t st) {
-  dim3 grid(p.B * p.Hkv, (p.kv_len + BK - 1) / BK);
-  hipLaunchKernelGGL((score_sum_kernel<D, KV>), grid, dim3(NTHREADS), 0, st, p);
+  const int groups = p.B * p.Hkv;
+  if constexpr (D <= 128) {
+    const int wide = (p.kv_len + 8 * NW - 1) / (8 * NW);
+    if ((int64_t)groups * wide >= num_cus()) {
+      hipLaunchKernelGGL((score_sum_kernel<D, KV, 8>), dim3(groups, wide), dim3(512), 0, st, p);
+      KVX_HIP(hipGetLastError());
+      return KVX_OK;
+    }
+  }
+  hipLaunchKernelGGL((score_sum_kernel<D, KV, 4>), dim3(groups, (p.kv_len + 4 * NW - 1) / (4 * NW)), dim3(256), 0, st, p);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }

@@ -105,6 +105,28 @@ def test_score_sum_from_given_lse(gpu):
     check_w(w, w_ref, q_len)
 
 
+@pytest.mark.parametrize("store", ["bf16", "u8"])
+def test_score_sum_with_eight_wavefront_workgroups(gpu, store):
+    # enough keys for the launch to take workgroups of 512 keys (8 KV heads x 32 workgroups), the last one
+    # ragged, causal inside the chunk, scattered slots
+    B, Hq, Hkv, q_len, T, D = 1, 16, 8, 40, 16000, 64
+    q, k, v, gen = make_qkv(78, B, Hq, Hkv, q_len, T, D)
+    input_pos = T + 11
+    tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len)
+    scale = 1.0 / math.sqrt(D)
+    quant, kg = None, k.to(gpu)
+    if store == "u8":
+        kc, ks, kz = O.quantize_rows(k)
+        k = O.dequantize_rows(kc, ks, kz)
+        kg = kc.to(gpu)
+        quant = ops.QuantState(ks.to(gpu), kz.to(gpu), ks.to(gpu), kz.to(gpu))
+    _, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, tp.to(torch.int64))
+    lse = O.lse2(q, k, scale, input_pos, tp)
+    w = ops.score_sum_core(q.to(gpu), kg, lse.to(gpu), scale, input_pos, tp.to(gpu), quant=quant)
+    check_w(w, w_ref, q_len)
+    torch.testing.assert_close(w.sum(-1).cpu(), torch.full((B, Hkv), float(q_len)), rtol=1e-4, atol=1e-3)
+
+
 def test_causal_weights_decay(gpu):
     # test/attention/test_flashinfer_wrapper.py:1074-1124: early keys collect far more weight
     q, k, v, _ = make_qkv(3, 1, 8, 2, 64, 64, 64)
