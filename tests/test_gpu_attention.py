@@ -172,7 +172,7 @@ DECODE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,T,D,splits", DECODE_CASES + [(2, 8, 2, 20000, 128, 0), (1, 8, 1, 9000, 64, 0)])
+@pytest.mark.parametrize("B,Hq,Hkv,T,D,splits", DECODE_CASES + [(2, 8, 2, 20000, 128, 0), (1, 8, 1, 9000, 64, 0), (1, 4, 2, 5000, 256, 0), (1, 16, 2, 4100, 128, 0)])
 def test_decode_with_weights(gpu, decode_route, B, Hq, Hkv, T, D, splits):
     q, k, v, _ = make_qkv(900 + T, B, Hq, Hkv, 1, T, D)
     scale = 1.0 / math.sqrt(D)
