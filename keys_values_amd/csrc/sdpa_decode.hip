@@ -20,8 +20,9 @@
 // W = (1/G) sum_g exp2(logit_g - lse_g) on the spot; in the fused H2O form it also adds W to the cumulative
 // scores and feeds the row's lowest-score slot. Longer splits, and a workgroup whose wait ran out, send the
 // logits to an fp32 scratch in bursts of 32 KB (a write stream mixed into the reads costs HBM far more than
-// its share of the bytes) and a last streaming kernel does the same work from there. A merge kernel
-// combines the splits' outputs. K and V are touched once: they are loaded non-temporally. No float atomics
+// its share of the bytes). One more launch follows the split kernel: some of its workgroups combine the splits'
+// outputs, the others do the weights work of the splits that took the scratch route, and the one that finishes
+// last publishes the chosen slots. K and V are touched once: they are loaded non-temporally. No float atomics
 // anywhere.
 #include "kvx_common.h"
 #include <stdlib.h>
@@ -46,10 +47,11 @@ struct DecodeParams {
   float* logits;   // (B, Hkv, Tpad, G), G the padded group size
   float* part_o;   // (B, Hq, S, D)
   float* part_ml;  // (B, Hq, S, 2)
-  float* lse_ws;   // (B, Hq)
   unsigned long long* best;  // fused H2O form: (value, slot) minimum per (b, kvh) row, else NULL
-  uint32_t* row_count;       // splits of a (b, kvh) row that have published their partial (resident form)
+  uint32_t* row_count;       // splits of a (b, kvh) row that have published their partial (resident form), then, in
+                             // the fused H2O form, the row's workgroups of the tail kernel that have finished
   uint32_t* split_done;      // (B, Hkv, S): 1 where the split kernel itself turned its logits into weights
+  uint32_t* tail_count;      // fused H2O form: workgroups of the tail kernel's second kind that have finished
   int32_t resident;          // the logits of a split stay in LDS
   int32_t spin_limit;        // polls of row_count before a workgroup gives up and sends its logits out
   int32_t poll_sleep;        // pause between two polls, in units of 512 cycles
@@ -449,21 +451,21 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 }
 
 // Before the split kernel: no split of a row has arrived, no row has a lowest-score slot yet.
-__global__ void decode_init_kernel(uint32_t* row_count, unsigned long long* best, int rows) {
+__global__ void decode_init_kernel(uint32_t* row_count, unsigned long long* best, uint32_t* tail_count, int rows) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < rows) {
     if (row_count) row_count[i * kCountStride] = 0u;
     if (best) best[i] = ~0ull;
   }
+  if (i == 0 && tail_count) *tail_count = 0u;
 }
 
 // Combine the splits of one (b, query head): 4 groups of D threads each take a quarter of the
 // splits, then the groups are added through LDS. Its first wavefront also produces the base-2 log-sum-exp.
 template <int D, bool F16>
-__global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams p) {
+__device__ __forceinline__ void merge_job(const DecodeParams& p, const int bh) {
   __shared__ float red[4][D + 1];
   __shared__ float sM;
-  const int bh = blockIdx.x;
   const int b = bh / p.Hq, hqi = bh % p.Hq;
   const int d = threadIdx.x % D, grp = threadIdx.x / D;
   const float* ml = p.part_ml + (int64_t)bh * p.num_splits * 2;
@@ -475,10 +477,7 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
     if (threadIdx.x == 0) sM = mloc;
     // the log-sum-exp by the routine the split kernel uses for its own weights: the same bits on either route
     const float lse = row_lse<false>(ml, p.num_splits, threadIdx.x);
-    if (threadIdx.x == 0) {
-      p.lse_ws[bh] = lse;
-      if (p.lse_out) p.lse_out[bh] = lse;
-    }
+    if (threadIdx.x == 0 && p.lse_out) p.lse_out[bh] = lse;
   }
   __syncthreads();
   const float M = sM;
@@ -501,92 +500,132 @@ __global__ __launch_bounds__(4 * D) void decode_merge_kernel(const DecodeParams 
 }
 
 // W[b, kvh, k] = (1/G) sum_g exp2(logit[b, kvh, k, g] - lse[b, kvh*G+g]); one key per lane and pass,
-// 4096 keys per workgroup, for the splits whose logits went to the scratch (in the resident form: those
-// whose wait ran out, normally none). With H2O set it also does the cache's score update and eviction choice
+// 4096 keys per workgroup of NT threads, for the splits whose logits went to the scratch (in the resident form:
+// those whose wait ran out, normally none). With H2O set it also does the cache's score update and eviction choice
 // in the same pass (keys_values/kvcache/h2o.py:175-196, keys_values/kvcache/attn_weights.py:773-774
-// for one slot): scores += W, then the (value, slot) minimum of the row through an integer atomicMin.
-template <int G, bool H2O>
-__global__ __launch_bounds__(256) void decode_weights_kernel(const DecodeParams p, const kvx_h2o_args hh) {
+// for one slot): scores += W, then the (value, slot) minimum of the row through an integer atomicMin; the workgroup
+// that finishes last publishes the slot of every row's minimum. (That needs no fence: the minima and the count of
+// finished workgroups are device-scope atomics, each waited for before the next; a release fence per workgroup
+// would write the whole L2 back on this multi-die part.)
+template <int G, bool H2O, int NT>
+__device__ __forceinline__ void weights_job(const DecodeParams& p, const kvx_h2o_args& hh, const int bx, const int kvh, const int b, const int jobs) {
   typedef float fG __attribute__((ext_vector_type(G >= 4 ? 4 : (G == 2 ? 2 : 1))));
   constexpr int NV = G >= 4 ? G / 4 : 1;
-  const int kvh = blockIdx.y, b = blockIdx.z;
+  constexpr int PASSES = 4096 / NT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ float lse_sh[G];
+  __shared__ unsigned long long wbest[NT / 64];
+  __shared__ int last_job;
   const uint32_t* done = p.resident ? p.split_done + ((int64_t)b * p.Hkv + kvh) * p.num_splits : nullptr;
+  int pending = 1;
   if (done) {
-    const int s0 = blockIdx.x * 4096 / p.keys_per_split, s1 = min((blockIdx.x * 4096 + 4095) / p.keys_per_split, p.num_splits - 1);
-    int pending = 0;
-    for (int sp = s0 + (int)threadIdx.x; sp <= s1; sp += 256) pending |= done[sp] == 0u;
-    if (!__syncthreads_or(pending)) return;
+    const int s0 = bx * 4096 / p.keys_per_split, s1 = min((bx * 4096 + 4095) / p.keys_per_split, p.num_splits - 1);
+    pending = 0;
+    for (int sp = s0 + tid; sp <= s1; sp += NT) pending |= done[sp] == 0u;
+    pending = __syncthreads_or(pending);
   }
-  float lse[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) lse[g] = g < p.Gr ? p.lse_ws[(int64_t)b * p.Hq + kvh * p.Gr + g] : INFINITY;  // exp2(x - inf) = 0
-  const float* lgrow = p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G;
-  float* wr = p.w ? p.w + ((int64_t)b * p.Hkv + kvh) * p.kv_len : nullptr;
-  float* sc = H2O ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
-  const int32_t* tpr = (H2O && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
   unsigned long long mine = ~0ull;
-  constexpr int PASSES = 16;
-  fG t[PASSES][NV];
-#pragma unroll
-  for (int it = 0; it < PASSES; ++it) {
-    const int k = min(blockIdx.x * 4096 + it * 256 + (int)threadIdx.x, p.Tpad - 1);
-#pragma unroll
-    for (int j = 0; j < NV; ++j) t[it][j] = *((const fG*)(lgrow + (int64_t)k * G) + j);
-  }
-#pragma unroll
-  for (int it = 0; it < PASSES; ++it) {
-    const int k = blockIdx.x * 4096 + it * 256 + threadIdx.x;
-    if (k >= p.kv_len) break;
-    if (done && done[k / p.keys_per_split]) continue;
-    float acc = 0.0f;
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float x;
-      if constexpr (G >= 4) x = t[it][g / 4][g % 4];
-      else if constexpr (G == 2) x = t[it][0][g];
-      else x = t[it][0][0];
-      acc += fast_exp2(x - lse[g]);
+  if (pending) {
+    // the row's log-sum-exps from the splits' partials, by the routine the split kernel and the merge use
+    for (int g = wave; g < G; g += NT / 64) {
+      float l = INFINITY;  // dummy heads: exp2(x - inf) = 0
+      if (g < p.Gr) l = row_lse<false>(p.part_ml + ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits * 2, p.num_splits, lane);
+      if (lane == 0) lse_sh[g] = l;
     }
-    acc *= 1.0f / (float)p.Gr;
-    if (wr) wr[k] = acc;
-    if constexpr (H2O) {
-      float val = sc[k] + acc;
-      sc[k] = val;
-      if (k < hh.limit) {
-        if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
-        const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
-        mine = key < mine ? key : mine;
+    __syncthreads();
+    float lse[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) lse[g] = lse_sh[g];
+    const float* lgrow = p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G;
+    float* wr = p.w ? p.w + ((int64_t)b * p.Hkv + kvh) * p.kv_len : nullptr;
+    float* sc = H2O ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
+    const int32_t* tpr = (H2O && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
+    fG t[PASSES][NV];
+#pragma unroll
+    for (int it = 0; it < PASSES; ++it) {
+      const int k = min(bx * 4096 + it * NT + tid, p.Tpad - 1);
+#pragma unroll
+      for (int j = 0; j < NV; ++j) t[it][j] = *((const fG*)(lgrow + (int64_t)k * G) + j);
+    }
+#pragma unroll
+    for (int it = 0; it < PASSES; ++it) {
+      const int k = bx * 4096 + it * NT + tid;
+      if (k >= p.kv_len) break;
+      if (done && done[k / p.keys_per_split]) continue;
+      float acc = 0.0f;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float x;
+        if constexpr (G >= 4) x = t[it][g / 4][g % 4];
+        else if constexpr (G == 2) x = t[it][0][g];
+        else x = t[it][0][0];
+        acc += fast_exp2(x - lse[g]);
+      }
+      acc *= 1.0f / (float)p.Gr;
+      if (wr) wr[k] = acc;
+      if constexpr (H2O) {
+        float val = sc[k] + acc;
+        sc[k] = val;
+        if (k < hh.limit) {
+          if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
+          const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
+          mine = key < mine ? key : mine;
+        }
       }
     }
   }
   if constexpr (H2O) {
+    if (pending) {
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const unsigned long long o = __shfl_xor(mine, off, 64);
-      mine = o < mine ? o : mine;
+      for (int off = 32; off >= 1; off >>= 1) {
+        const unsigned long long o = __shfl_xor(mine, off, 64);
+        mine = o < mine ? o : mine;
+      }
+      if (lane == 0) wbest[wave] = mine;
+      __syncthreads();
     }
-    __shared__ unsigned long long wbest[4];
-    if ((threadIdx.x & 63) == 0) wbest[threadIdx.x >> 6] = mine;
+    if (tid == 0) {
+      if (pending) {
+        unsigned long long mn = wbest[0];
+        for (int i = 1; i < NT / 64; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
+        if (mn != ~0ull) {
+          const unsigned long long old = __hip_atomic_fetch_min(p.best + b * p.Hkv + kvh, mn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          asm volatile("s_waitcnt vmcnt(0)" : : "v"(old) : "memory");  // performed before this workgroup counts itself
+        }
+      }
+      // counted per row first (the row's counter goes on from where the split kernel's arrivals left it), rows second:
+      // no counter sees more than a few dozen increments
+      const int wx = jobs / (p.B * p.Hkv);
+      const uint32_t row_full = (p.resident ? (uint32_t)p.num_splits : 0u) + (uint32_t)wx - 1u;
+      const bool row_last = __hip_atomic_fetch_add(p.row_count + (b * p.Hkv + kvh) * kCountStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == row_full;
+      last_job = row_last && __hip_atomic_fetch_add(p.tail_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(p.B * p.Hkv - 1);
+    }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      unsigned long long mn = wbest[0];
-      for (int i = 1; i < 4; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
-      if (mn != ~0ull) atomicMin(p.best + b * p.Hkv + kvh, mn);
+    if (last_job) {
+      for (int i = tid; i < p.B * p.Hkv; i += NT)
+        hh.next_index[i] = (int32_t)(__hip_atomic_load(p.best + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffffffffull);
     }
   }
 }
 
-// Publishes the slot of each row's minimum. A separate launch: doing it in the last workgroup of the
-// weights kernel needs a device-scope fence per workgroup, which on this multi-die part writes back L2
-// and more than doubles that kernel's time.
-__global__ void decode_argmin_finish_kernel(const unsigned long long* best, int32_t* next_index, int rows) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < rows) next_index[i] = (int32_t)(best[i] & 0xffffffffull);
+// What follows the split kernel, in one launch: the first merge_jobs workgroups combine the splits of one (batch,
+// query head) each; the others (MODE 1: weights wanted, MODE 2: fused H2O step) take 4096 keys of a (batch, KV head)
+// row each. The two kinds do not depend on each other: both read what the split kernel left.
+template <int D, bool F16, int G, int MODE>
+__global__ __launch_bounds__(4 * D) void decode_tail_kernel(const DecodeParams p, const kvx_h2o_args hh, const int merge_jobs, const int wx) {
+  if ((int)blockIdx.x < merge_jobs) {
+    merge_job<D, F16>(p, blockIdx.x);
+    return;
+  }
+  if constexpr (MODE > 0) {
+    const int j = blockIdx.x - merge_jobs;
+    weights_job<G, MODE == 2, 4 * D>(p, hh, j % wx, (j / wx) % p.Hkv, j / (wx * p.Hkv), (int)gridDim.x - merge_jobs);
+  }
 }
 
 struct Plan {
   int G, num_splits, keys_per_split, Tpad, resident;
-  size_t off_logits, off_part_o, off_part_ml, off_lse, off_best, off_count, off_done, total;
+  size_t off_logits, off_part_o, off_part_ml, off_best, off_tail, off_count, off_done, total;
 };
 
 // KVX_DECODE_RESIDENT=0 sends every split's logits through the scratch; KVX_DECODE_SPIN_LIMIT bounds the
@@ -627,27 +666,42 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   off += (size_t)a.B * a.Hq * pl.num_splits * a.D * 4;
   pl.off_part_ml = off;
   off += (size_t)a.B * a.Hq * pl.num_splits * 2 * 4;
-  pl.off_lse = off;
-  off += (size_t)a.B * a.Hq * 4;
   off = (off + 7) & ~(size_t)7;
   pl.off_best = off;
   off += fused_h2o ? (size_t)a.B * a.Hkv * 8 : 0;
+  pl.off_tail = off;
+  off += fused_h2o ? 8 : 0;
   pl.resident = allow_resident && kps <= lgk;
   off = (off + 255) & ~(size_t)255;
   pl.off_count = off;
-  off += pl.resident ? (size_t)a.B * a.Hkv * kCountStride * 4 : 0;
+  off += (pl.resident || fused_h2o) ? (size_t)a.B * a.Hkv * kCountStride * 4 : 0;
   pl.off_done = off;
   off += pl.resident ? (size_t)a.B * a.Hkv * pl.num_splits * 4 : 0;
   pl.total = (off + 255) & ~(size_t)255;
   return pl;
 }
 
+template <int D, bool F16, int G>
+int launch_tail(const DecodeParams& p, const kvx_h2o_args* hh, hipStream_t st) {
+  const int merge_jobs = p.B * p.Hq, wx = (p.kv_len + 4095) / 4096;
+  const int weight_jobs = (hh || p.w) ? wx * p.Hkv * p.B : 0;
+  const dim3 grid(merge_jobs + weight_jobs), block(4 * D);
+  const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
+  if (hh) hipLaunchKernelGGL((decode_tail_kernel<D, F16, G, 2>), grid, block, 0, st, p, h2, merge_jobs, wx);
+  else if (p.w) hipLaunchKernelGGL((decode_tail_kernel<D, F16, G, 1>), grid, block, 0, st, p, h2, merge_jobs, wx);
+  else hipLaunchKernelGGL((decode_tail_kernel<D, F16, 1, 0>), grid, block, 0, st, p, h2, merge_jobs, wx);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+// Three launches: the counters' reset (only when something counts), the split kernel, the tail.
 template <int D, int G>
 int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
   const int rows = p.B * p.Hkv;
   if (p.resident || hh) {
-    hipLaunchKernelGGL(decode_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.resident ? p.row_count : nullptr, hh ? p.best : nullptr, rows);
+    hipLaunchKernelGGL(decode_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.row_count, hh ? p.best : nullptr,
+                       hh ? p.tail_count : nullptr, rows);
     KVX_HIP(hipGetLastError());
   }
   const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
@@ -659,21 +713,7 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
   if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
   else if (kv == KVX_KV_BF16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
   KVX_HIP(hipGetLastError());
-  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_merge_kernel<D, true>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
-  else hipLaunchKernelGGL((decode_merge_kernel<D, false>), dim3(p.B * p.Hq), dim3(4 * D), 0, st, p);
-  KVX_HIP(hipGetLastError());
-  const dim3 wgrid((p.kv_len + 4095) / 4096, p.Hkv, p.B);
-  if (hh) {
-    hipLaunchKernelGGL((decode_weights_kernel<G, true>), wgrid, dim3(256), 0, st, p, *hh);
-    KVX_HIP(hipGetLastError());
-    hipLaunchKernelGGL(decode_argmin_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.best, hh->next_index, rows);
-    KVX_HIP(hipGetLastError());
-  } else if (p.w) {
-    kvx_h2o_args none = {};
-    hipLaunchKernelGGL((decode_weights_kernel<G, false>), wgrid, dim3(256), 0, st, p, none);
-    KVX_HIP(hipGetLastError());
-  }
-  return KVX_OK;
+  return kv == KVX_KV_F16 ? launch_tail<D, true, G>(p, hh, st) : launch_tail<D, false, G>(p, hh, st);
 }
 
 template <int D>
@@ -711,8 +751,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.logits = (a.w || hh) ? (float*)(ws + pl.off_logits) : nullptr;
   p.part_o = (float*)(ws + pl.off_part_o);
   p.part_ml = (float*)(ws + pl.off_part_ml);
-  p.lse_ws = (float*)(ws + pl.off_lse);
   p.best = hh ? (unsigned long long*)(ws + pl.off_best) : nullptr;
+  p.tail_count = hh ? (uint32_t*)(ws + pl.off_tail) : nullptr;
   p.row_count = (uint32_t*)(ws + pl.off_count);
   p.split_done = (uint32_t*)(ws + pl.off_done);
   p.resident = pl.resident;
