@@ -390,7 +390,7 @@ def bench_decode(args, torch, dev):
     bytes_alg = 2 * B * Hkv * L * ((D // 2 if u4 else D) + 8 if u8 else 2 * D) + 2 * B * Hkv * L * 4
     gbs = bytes_alg / (ms_step * 1e-3) / 1e9
     # the dominant launch alone: the fused attention + score update + argmin call (split attention,
-    # merge, weights kernels), events on the launch stream around each call
+    # tail kernel), events on the launch stream around each call
     launch, _ = cache._decode_h2o_prepare(qs[0], cache.k, cache.v, cache._quant_state(L))
     launch()
     torch.cuda.synchronize()
@@ -425,7 +425,7 @@ def bench_decode(args, torch, dev):
         "config": {"workload": "BASELINE.json configs[3]: decode + H2O eviction, B8 Hq32 Hkv8 D128 T131072, seed 3" + (f", {args.kv} cache" if u8 else ""),
                    "bytes_algorithmic_per_step": bytes_alg, "ms_per_step_gpu_events": round(ms_gpu, 4),
                    "decode_tokens_per_s": round(B / (ms_step * 1e-3), 1)},
-        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + merge + weights/score update/argmin" % {"bf16": "KVX_KV_BF16", "uint8": "KVX_KV_U8", "uint4": "KVX_KV_U4"}[args.kv],
+        "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + tail (merge, scratch-route weights, slot publishing)" % {"bf16": "KVX_KV_BF16", "uint8": "KVX_KV_U8", "uint4": "KVX_KV_U4"}[args.kv],
                      "achieved": round(bytes_alg / (ms_call * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(bytes_alg / (ms_call * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "ms_per_launch": round(ms_call, 4),
                      "traffic": None if u8 else TRAFFIC_BYTES["decode"]},
