@@ -639,19 +639,27 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
   const int gr = a.Hq / a.Hkv;
   pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : 8));
-  // About 16 workgroups per compute unit over the whole grid, each with at least 1024 keys. When the weights
-  // are wanted, 8: a split that waits for its row holds its place on the compute unit, and the fewer,
-  // longer splits wait a smaller part of their time (measured: 4 rounds of 2 workgroups per compute unit
-  // beat 8 by 2 %, 6 are 5 % worse); and if a split's logits then do not fit in LDS, as many more splits as make them fit.
+  // Without weights: about 16 workgroups per compute unit over the whole grid, each with at least 1024 keys.
+  // With weights a split that waits for its row holds its place on the compute unit, so the splits are as long as
+  // the LDS holds their logits and the device still gets one full round of workgroups (two per compute unit, what
+  // the registers allow): rows * kv_len / (2 CUs) keys, between 512 and the LDS limit. (Measured at 8 x 8 x 131072:
+  // 4 rounds of 4096 keys beat 8 rounds of 2048 by 2 %; at 8 rows x 262144 one round of 4096 keys takes 178 us,
+  // four rounds of 1024 keys 265; short caches with few rows want the 512.)
   const bool weights = a.w || fused_h2o;
   const int allow_resident = weights ? env_int("KVX_DECODE_RESIDENT", 1) : 0;
   const int lgk = logit_floats(pl.G, a.D) / pl.G;
   int splits = a.num_splits;
   if (splits <= 0) {
-    const int rows = a.B * a.Hkv;
-    splits = ((allow_resident ? 8 : 16) * num_cus() + rows - 1) / rows;
-    splits = min(splits, (a.kv_len + 1023) / 1024);
-    if (allow_resident) splits = max(splits, (a.kv_len + lgk - 1) / lgk);
+    const int64_t rows = (int64_t)a.B * a.Hkv;
+    if (allow_resident) {
+      int64_t keys = rows * a.kv_len / (2 * num_cus());
+      keys = keys > lgk ? lgk : keys;
+      keys = keys < 512 ? 512 : keys;
+      splits = (int)((a.kv_len + keys - 1) / keys);
+    } else {
+      const int64_t by_cus = (16 * num_cus() + rows - 1) / rows, by_keys = (a.kv_len + 1023) / 1024;
+      splits = (int)(by_cus < by_keys ? by_cus : by_keys);
+    }
   }
   splits = max(1, min(splits, 512));
   int kps = (a.kv_len + splits - 1) / splits;
