@@ -639,27 +639,25 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
   const int gr = a.Hq / a.Hkv;
   pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : 8));
-  // Without weights: about 16 workgroups per compute unit over the whole grid, each with at least 1024 keys.
-  // With weights a split that waits for its row holds its place on the compute unit, so the splits are as long as
-  // the LDS holds their logits and the device still gets one full round of workgroups (two per compute unit, what
-  // the registers allow): rows * kv_len / (2 CUs) keys, between 512 and the LDS limit. (Measured at 8 x 8 x 131072:
-  // 4 rounds of 4096 keys beat 8 rounds of 2048 by 2 %; at 8 rows x 262144 one round of 4096 keys takes 178 us,
-  // four rounds of 1024 keys 265; short caches with few rows want the 512.)
+  // One full round of workgroups (two per compute unit, what the registers allow) over the whole grid:
+  // rows * kv_len / (2 CUs) keys per split, at least 256; with weights at most what the LDS holds of a split's
+  // logits (a split that waits for its row holds its place, so the device then runs several rounds) and, LDS
+  // permitting, at least kv_len / 128 (2 rows of 65536 keys: 45 us with 128 splits waiting for each other, 56 with 256).
+  // Measured, with weights: 8 x 8 rows of 131072 keys, 4 rounds of 4096 keys beat 8 rounds of 2048 by 2 %; 8 rows of
+  // 262144 keys take 182 us in one round of 4096 keys and 265 in four of 1024. Without weights: 32 rows of 262144
+  // keys 631 us in 16 splits, 658 in 128; 8 rows of 16384 keys 22 us in 32 splits, 26 in 16 of 1024.
   const bool weights = a.w || fused_h2o;
   const int allow_resident = weights ? env_int("KVX_DECODE_RESIDENT", 1) : 0;
   const int lgk = logit_floats(pl.G, a.D) / pl.G;
   int splits = a.num_splits;
   if (splits <= 0) {
-    const int64_t rows = (int64_t)a.B * a.Hkv;
-    if (allow_resident) {
-      int64_t keys = rows * a.kv_len / (2 * num_cus());
-      keys = keys > lgk ? lgk : keys;
-      keys = keys < 512 ? 512 : keys;
-      splits = (int)((a.kv_len + keys - 1) / keys);
-    } else {
-      const int64_t by_cus = (16 * num_cus() + rows - 1) / rows, by_keys = (a.kv_len + 1023) / 1024;
-      splits = (int)(by_cus < by_keys ? by_cus : by_keys);
+    int64_t keys = (int64_t)a.B * a.Hkv * a.kv_len / (2 * num_cus());
+    if (keys < 256) keys = 256;
+    if (allow_resident) {  // at most 128 splits wait for each other, unless the LDS limit asks for more
+      if (keys < (a.kv_len + 127) / 128) keys = (a.kv_len + 127) / 128;
+      if (keys > lgk) keys = lgk;
     }
+    splits = (int)((a.kv_len + keys - 1) / keys);
   }
   splits = max(1, min(splits, 512));
   int kps = (a.kv_len + splits - 1) / splits;
