@@ -128,7 +128,9 @@ size_t kvx_sdpa_prefill_workspace_bytes(const kvx_sdpa_args* args);
  * W[b,h,k] = (1/G) * sum_{i,g} exp2(s*log2(e)*q_{i,g}.k - lse[b,i,h*G+g]) * [tp[b,h,k] <= input_pos+i].
  * Stands in for triton_score_sum / _score_sum_kernel
  * (keys_values/attention/flashinfer_wrapper.py:51-273). Deterministic: every W element is owned by
- * one wavefront, no atomics. Reads args->lse, writes args->w; o and v are ignored. */
+ * one wavefront, no atomics. Reads args->lse, writes args->w; o and v are ignored. args->workspace is optional:
+ * given kvx_sdpa_prefill_workspace_bytes(args) bytes, a short cache (too few keys to give every compute unit a
+ * workgroup) has its query rows split over more workgroups, whose partial sums are added in a fixed order. */
 int kvx_score_sum(const kvx_sdpa_args* args, void* stream);
 
 /* kvx_sdpa_prefill followed by kvx_score_sum on the same stream: the whole

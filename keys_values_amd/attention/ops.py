@@ -217,7 +217,12 @@ def score_sum_core(query, key, lse, scale, input_pos, token_positions=None, quan
         _fill_common(a, query, key, None, scale, input_pos, token_positions, quant, 0)
         a.lse = lse.data_ptr()
         a.w = w.data_ptr()
-        _lib.check(_lib.load().kvx_score_sum(ctypes.byref(a), _lib.stream_ptr(dev)))
+        lib = _lib.load()
+        # short caches split the query rows over more workgroups; the partial sums need a workspace
+        ws = _lib.workspace(dev, lib.kvx_sdpa_prefill_workspace_bytes(ctypes.byref(a)))
+        a.workspace = _lib.ptr(ws)
+        a.workspace_bytes = 0 if ws is None else ws.numel()
+        _lib.check(lib.kvx_score_sum(ctypes.byref(a), _lib.stream_ptr(dev)))
     return w
 
 

@@ -40,6 +40,7 @@ int hip_error(hipError_t e, const char* what);
 int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st);
 size_t sdpa_prefill_workspace(const kvx_sdpa_args& a);
 int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st);
+size_t score_sum_workspace(const kvx_sdpa_args& a);
 int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* fused_h2o, hipStream_t st);
 size_t sdpa_decode_workspace(const kvx_sdpa_args& a, bool fused_h2o);
 int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,

@@ -32,6 +32,8 @@ struct ScoreParams {
   const int32_t* tp;
   const float* lse;
   float* w;
+  float* part;           // query rows split over several workgroups: (splits, B, Hkv, kv_len) partial sums, else NULL
+  int32_t tiles_per_z;   // query tiles per split
   int32_t B, Hq, Hkv, G, q_len, kv_len, R, input_pos;
   float c, inv_g;
   int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, qs_sb, qs_sh, tp_sb, tp_sh;
@@ -72,7 +74,7 @@ struct QLoader {
   const uint16_t* src[QCH];  // dg == 0: address of chunk i in the current tile
   int64_t step;              // dg == 0: elements between consecutive tiles
 
-  __device__ __forceinline__ void init(const ScoreParams& p, int b, int kvh, int tid) {
+  __device__ __forceinline__ void init(const ScoreParams& p, int b, int kvh, int tid, int row_start) {
     col = tid % CPR;
     row_in = tid / CPR;
     G = p.G; R = p.R; Hq = p.Hq; input_pos = p.input_pos;
@@ -82,14 +84,14 @@ struct QLoader {
     dq = BQ / G; dg = BQ % G;
 #pragma unroll
     for (int i = 0; i < QCH; ++i) {
-      const int r = row_in + i * RPI;
+      const int r = row_start + row_in + i * RPI;
       qi[i] = r / G;
       g[i] = r % G;
       src[i] = qbase + (int64_t)g[i] * q_sh + (int64_t)qi[i] * q_st + col * 8;
     }
     step = (int64_t)dq * q_st;
-    lqi = tid / G;
-    lg = tid % G;
+    lqi = (row_start + tid) / G;
+    lg = (row_start + tid) % G;
   }
 
   // fetch the tile whose first row is row0, then step the row bookkeeping to the next tile
@@ -141,7 +143,9 @@ struct QLoader {
   }
 };
 
-template <int D, int KV, int W>
+// QSPLIT: the query rows are split over blockIdx.z (short caches that would otherwise leave compute units
+// idle); every split writes its sums to p.part and a second kernel adds them in a fixed order.
+template <int D, int KV, int W, bool QSPLIT>
 __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
   constexpr int BK = NW * W;  // keys per workgroup
   constexpr bool F16 = KV == KVX_KV_F16;  // element type of q and k
@@ -196,9 +200,10 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
   tpmax = __builtin_amdgcn_readfirstlane(tpmax);
 
   float wacc[2] = {0.0f, 0.0f};
-  const int num_qt = (p.R + BQ - 1) / BQ;
+  const int tbase = QSPLIT ? (int)blockIdx.z * p.tiles_per_z : 0;  // first query tile of this workgroup
+  const int num_qt = QSPLIT ? min(p.tiles_per_z, (p.R + BQ - 1) / BQ - tbase) : (p.R + BQ - 1) / BQ;
   QLoader<D, W> ld;
-  ld.init(p, b, kvh, tid);
+  ld.init(p, b, kvh, tid, tbase * BQ);
   QStage<D, W> st;
 
   // S block = 32 query rows x 64 keys: Q rows come from LDS (A operand), K sits in registers.
@@ -257,9 +262,9 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
     }
   };
 
-  ld.fetch(st, 0, tid);
+  ld.fetch(st, tbase * BQ, tid);
   ld.commit(st, sm, 0, 0, tid);
-  if (num_qt > 1) ld.fetch(st, BQ, tid);
+  if (num_qt > 1) ld.fetch(st, (tbase + 1) * BQ, tid);
   __syncthreads();
   f32x16_t sa[2], sb[2];  // blocks 0 and 1 of the current tile
   mfma_block(sa, 0, 0);
@@ -271,12 +276,12 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
     const bool more = t + 1 < num_qt;
     if (more) {
       ld.commit(st, sm, buf ^ 1, (t + 1) % 3, tid);
-      if (t + 2 < num_qt) ld.fetch(st, (t + 2) * BQ, tid);
+      if (t + 2 < num_qt) ld.fetch(st, (tbase + t + 2) * BQ, tid);
     }
     // issue priority: lowest in the first half of a tile, highest on the way to the barrier, so that the
     // four wavefronts of a workgroup wait less for each other (about 1 % on the kernel)
     __builtin_amdgcn_s_setprio(0);
-    const bool need_mask = tpmax > p.input_pos + (t * BQ) / p.G;
+    const bool need_mask = tpmax > p.input_pos + ((tbase + t) * BQ) / p.G;
     if (need_mask) {
       mfma_block(sb, buf, 1);
       valu_block(std::true_type{}, sa, buf3, 0);
@@ -309,30 +314,80 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
   for (int nt = 0; nt < 2; ++nt) {
     const float tot = sum_halves(wacc[nt]);
     const int key = key0 + nt * 32 + n;
-    if (h == 0 && key < p.kv_len) p.w[((int64_t)b * p.Hkv + kvh) * p.kv_len + key] = tot * p.inv_g;
+    if (h == 0 && key < p.kv_len) {
+      if constexpr (QSPLIT) p.part[(((int64_t)blockIdx.z * p.B + b) * p.Hkv + kvh) * p.kv_len + key] = tot;
+      else p.w[((int64_t)b * p.Hkv + kvh) * p.kv_len + key] = tot * p.inv_g;
+    }
   }
 }
 
+// W = (1/G) * (part[0] + part[1] + ...), in that order.
+__global__ void score_sum_reduce_kernel(const float* part, float* w, int64_t n, int splits, float inv_g) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float acc = part[i];
+  for (int z = 1; z < splits; ++z) acc += part[(int64_t)z * n + i];
+  w[i] = acc * inv_g;
+}
+
+// Splits of the query rows: none when the keys alone give every compute unit two workgroups of 256 keys; else as
+// many as that takes, each at least 8 tiles of 64 rows (the second launch costs a short chunk more than it
+// gains), at most 16.
+struct ScorePlan {
+  int splits, tiles_per_z;
+};
+ScorePlan score_plan(const kvx_sdpa_args& a) {
+  const int G = a.Hq / a.Hkv;
+  const int num_qt = (int)(((int64_t)a.q_len * G + BQ - 1) / BQ);
+  const int64_t wgs = (int64_t)a.B * a.Hkv * ((a.kv_len + 4 * NW - 1) / (4 * NW));
+  int64_t splits = (2 * num_cus() + wgs - 1) / wgs;
+  if (splits > num_qt / 8) splits = num_qt / 8;
+  if (splits > 16) splits = 16;
+  if (splits < 1) splits = 1;
+  ScorePlan pl;
+  pl.tiles_per_z = (num_qt + (int)splits - 1) / (int)splits;
+  pl.splits = (num_qt + pl.tiles_per_z - 1) / pl.tiles_per_z;
+  return pl;
+}
+
 template <int D, int KV>
-int launch_t(const ScoreParams& p, hipStream_t st) {
+int launch_t(const ScoreParams& p, int splits, hipStream_t st) {
   const int groups = p.B * p.Hkv;
+  if (splits > 1) {
+    hipLaunchKernelGGL((score_sum_kernel<D, KV, 4, true>), dim3(groups, (p.kv_len + 4 * NW - 1) / (4 * NW), splits), dim3(256), 0, st, p);
+    KVX_HIP(hipGetLastError());
+    const int64_t n = (int64_t)groups * p.kv_len;
+    hipLaunchKernelGGL(score_sum_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p.part, p.w, n, splits, p.inv_g);
+    KVX_HIP(hipGetLastError());
+    return KVX_OK;
+  }
   if constexpr (D <= 128) {
     const int wide = (p.kv_len + 8 * NW - 1) / (8 * NW);
     if ((int64_t)groups * wide >= num_cus()) {
-      hipLaunchKernelGGL((score_sum_kernel<D, KV, 8>), dim3(groups, wide), dim3(512), 0, st, p);
+      hipLaunchKernelGGL((score_sum_kernel<D, KV, 8, false>), dim3(groups, wide), dim3(512), 0, st, p);
       KVX_HIP(hipGetLastError());
       return KVX_OK;
     }
   }
-  hipLaunchKernelGGL((score_sum_kernel<D, KV, 4>), dim3(groups, (p.kv_len + 4 * NW - 1) / (4 * NW)), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((score_sum_kernel<D, KV, 4, false>), dim3(groups, (p.kv_len + 4 * NW - 1) / (4 * NW)), dim3(256), 0, st, p);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
 
 }  // namespace
 
+size_t score_sum_workspace(const kvx_sdpa_args& a) {
+  const ScorePlan pl = score_plan(a);
+  return pl.splits > 1 ? (size_t)pl.splits * a.B * a.Hkv * a.kv_len * sizeof(float) : 0;
+}
+
 int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
+  // the query rows are split only if the caller's workspace holds the partial sums
+  ScorePlan pl = score_plan(a);
+  if (pl.splits > 1 && !(a.workspace && a.workspace_bytes >= score_sum_workspace(a) && ((uintptr_t)a.workspace & 15) == 0)) pl.splits = 1;
   ScoreParams p;
+  p.part = pl.splits > 1 ? (float*)a.workspace : nullptr;
+  p.tiles_per_z = pl.tiles_per_z;
   p.q = (const uint16_t*)a.q;
   p.k = a.k;
   p.k_scale = a.k_scale;
@@ -349,17 +404,17 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
   if (a.D == 128) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, pl.splits, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, pl.splits, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, pl.splits, st) : launch_t<128, KVX_KV_BF16>(p, pl.splits, st);
   }
   if (a.D == 64) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
+    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, pl.splits, st);
+    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, pl.splits, st);
+    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, pl.splits, st) : launch_t<64, KVX_KV_BF16>(p, pl.splits, st);
   }
   if (a.D == 256 && kv_is_plain(a.kv_dtype))
-    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, st) : launch_t<256, KVX_KV_BF16>(p, st);
+    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, pl.splits, st) : launch_t<256, KVX_KV_BF16>(p, pl.splits, st);
   return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
 }
 

@@ -1659,7 +1659,9 @@ int launch_t(PrefillParams& p, hipStream_t st, int variant = PF_CLASSIC) {
 size_t sdpa_prefill_workspace(const kvx_sdpa_args& a) {
   PrefillParams p;
   fill_params(p, a);
-  return partial_bytes(p, a.D);
+  // the score-sum pass that may follow on the same stream reuses the workspace for its partial sums
+  const size_t own = partial_bytes(p, a.D), after = score_sum_workspace(a);
+  return own > after ? own : after;
 }
 
 int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {

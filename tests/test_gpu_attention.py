@@ -1,10 +1,12 @@
 """GPU parity of the attention kernels against the CPU oracle, through the C ABI (ctypes)."""
+import ctypes
 import math
 
 import pytest
 import torch
 
 from helpers import make_qkv, rel_err, scattered_positions
+from keys_values_amd import _lib
 from keys_values_amd.attention import ops
 from keys_values_amd.attention.sdpa import HipSDPA
 from oracle import kvx_oracle as O
@@ -125,6 +127,31 @@ def test_score_sum_with_eight_wavefront_workgroups(gpu, store):
     w = ops.score_sum_core(q.to(gpu), kg, lse.to(gpu), scale, input_pos, tp.to(gpu), quant=quant)
     check_w(w, w_ref, q_len)
     torch.testing.assert_close(w.sum(-1).cpu(), torch.full((B, Hkv), float(q_len)), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,q_len,T,D", [(1, 8, 2, 700, 900, 128), (2, 4, 1, 1100, 1100, 64), (1, 16, 2, 300, 2048, 128)])
+def test_score_sum_over_split_query_rows(kvx, gpu, B, Hq, Hkv, q_len, T, D):
+    # a short cache: with a workspace the query rows are split over several workgroups and the partial sums
+    # added by a second launch; without one the kernel walks all rows. Both against the oracle, and each other.
+    q, k, v, gen = make_qkv(79 + T, B, Hq, Hkv, q_len, T, D)
+    input_pos = T - q_len + 3
+    tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len)
+    scale = 1.0 / math.sqrt(D)
+    _, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, tp.to(torch.int64))
+    lse = O.lse2(q, k, scale, input_pos, tp).to(gpu)
+    qg, kg, tpg = q.to(gpu), k.to(gpu), tp.to(gpu)
+    w_split = ops.score_sum_core(qg, kg, lse, scale, input_pos, tpg)
+    check_w(w_split, w_ref, q_len)
+    a = _lib.SdpaArgs()
+    ops._fill_common(a, qg, kg, None, scale, input_pos, tpg, None, 0)
+    assert kvx.kvx_sdpa_prefill_workspace_bytes(ctypes.byref(a)) > 0  # the shape does split
+    w_whole = torch.empty_like(w_split)
+    a.lse, a.w = lse.data_ptr(), w_whole.data_ptr()
+    _lib.check(kvx.kvx_score_sum(ctypes.byref(a), _lib.stream_ptr(gpu)))  # no workspace: no split
+    torch.cuda.synchronize()
+    check_w(w_whole, w_ref, q_len)
+    torch.testing.assert_close(w_split, w_whole, rtol=1e-5, atol=1e-7)
+    assert torch.equal(w_split, ops.score_sum_core(qg, kg, lse, scale, input_pos, tpg))  # the same bits every time
 
 
 def test_causal_weights_decay(gpu):
