@@ -19,14 +19,11 @@ Inputs are resident in HBM before the timed region.
 `--workload policy`  : the same 1024-token chunk through the cache object (write with the ring move, attention,
                        score-sum, score update, choice of the next 1024 slots) for each eviction-policy variant
                        (grace period, normalised scores, V-norm weighting, Q-Hitter); ms per chunk step.
-`--workload ceiling` : runs the stand-alone probe built next to the library (keys_values_amd/mfma_probe): what the
-                       matrix cores sustain (clock, TFLOP/s) alone and with vector work beside them, and how fast
-                       a single wavefront issues; prints the probe's table on stderr and the sustained pure-matrix
-                       figure as the JSON line.
 `--workload calib`   : a plain elementwise kernel that reads 1 GiB and writes 1 GiB, the known-size
                        launch against which the FETCH_SIZE / WRITE_SIZE counters are scaled.
 
-The default run also times, after the headline workload, the decode + H2O step, the quantiser and the
+The default run also times, after the headline workload, the decode + H2O step, the quantiser, attention +
+score-sum over the uint8 store (BASELINE.json configs[2]: fused dequantisation and the dequantised-copy path) and the
 long-context prefill on their own configurations and reports them under `config.secondary`
 (`--no-secondary` skips them).
 
@@ -50,9 +47,13 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch, one counter per run, on these same workloads), each scaled by what the counter
-# reads for the `calib` launch of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+# HBM bytes per launch of each workload's dominant kernel. NOT measured by this run: the figures of the
+# committed counter runs (profiles/hbm_traffic_fetch_write_size.txt: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
+# KiB per dispatch, one counter per run, on these same workloads), each scaled by what the counter reads for
+# the `calib` launch of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000). Reported as `roofline.traffic`
+# with `roofline.traffic_source` saying so. (The quantiser's 2 x 205 MB working set is close to the 256 MB
+# last-level cache; its FETCH_SIZE still reads the full 134 MB per launch, so the rows do come from HBM.)
+TRAFFIC_SOURCE = "committed counter run (profiles/hbm_traffic_fetch_write_size.txt), not measured in this run"
 TRAFFIC_BYTES = {
     "prefill": int((70196.3 * 2.000 + 33283.4) * 1024),    # sdpa_prefill_kernel<128, KVX_KV_BF16>
     "decode": int((2115128.0 * 2.000 + 37312.0) * 1024),   # decode_split_kernel<128, 4, KVX_KV_BF16>
@@ -60,18 +61,46 @@ TRAFFIC_BYTES = {
 }
 
 
+def cpu_threads(torch):
+    """Threads for the CPU baseline: the GPU box's share of host cores is 16 per GPU whatever os.cpu_count() shows
+    there, so more threads than that would only time-slice."""
+    n = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(n)
+    return n
+
+
+def cpu_time(fn):
+    """Seconds of one pass of `fn`: the median of 5 passes when a pass takes at most 2 s (after the first pass, which
+    then counts as the warm-up), else that single pass. Returns (seconds, result of the last pass, note)."""
+    t0 = time.perf_counter()
+    res = fn()
+    first = time.perf_counter() - t0
+    if first > 2.0:
+        return first, res, "one pass"
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        res = fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2], res, "median of 5 passes after 1 warm-up"
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib", "ceiling"])
+    ap.add_argument("--workload", default="prefill", choices=["prefill", "decode", "quantize", "longctx", "policy", "calib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
                     help="default workload only: skip the decode, quantiser and long-context legs that are reported under config.secondary")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--layers", type=int, default=36, help="longctx: number of layers")
     ap.add_argument("--tokens", type=int, default=131072, help="longctx: prompt length")
+    ap.add_argument("--no-gemm-table", action="store_true",
+                    help="longctx: leave the choice of the library GEMM kernels to the library instead of reading the committed per-shape "
+                         "table (keys_values_amd/longctx/gemm_table_gfx950.csv; switches PyTorch's TunableOp on for the process)")
     ap.add_argument("--tune-gemms", action="store_true",
                     help="longctx: let PyTorch's TunableOp pick the library GEMM kernels during the warm-up pass (adds about a minute)")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8", "uint4"],
@@ -227,18 +256,18 @@ def bench_prefill(args, torch, dev):
     if not args.no_cpu_baseline:
         # bounded sample: the first KV heads with their query heads, same op sequence as the
         # reference's eager path (fp32 upcast, <= 3 GB score slices, mask, softmax, mean/sum)
-        torch.set_num_threads(min(16, os.cpu_count() or 1))
-        hs = Hkv  # the whole workload: a second or two on the host's cores
+        nthreads = cpu_threads(torch)
+        hs = 1 if u8 else Hkv  # bf16: the whole workload, a second or two on the host's cores; quantised store: one KV head
         qs, ks, vs = q_c[:, : 4 * hs], k_c[:, :hs], v_c[:, :hs]
-        t_c0 = time.perf_counter()
-        o_ref, w_ref = O.sdpa_in_blocks(qs, ks, vs, scale, input_pos, None)
-        t_c = time.perf_counter() - t_c0
+        t_c, (o_ref, w_ref), how = cpu_time(lambda: O.sdpa_in_blocks(qs, ks, vs, scale, input_pos, None))
         cpu = {
             "value": round(flops_alg * hs / Hkv / t_c / 1e12, 4),
             "unit": "TFLOP/s",
-            "cores": torch.get_num_threads(),
+            "cores": nthreads,
+            "host_cpus": os.cpu_count(),
             "kind": "port",
-            "sample": f"KV heads 0-{hs - 1} of {Hkv} ({4 * hs} query heads x 1024 queries x {T} keys), one pass, {t_c:.1f} s",
+            "sample": f"KV heads 0-{hs - 1} of {Hkv} ({4 * hs} query heads x 1024 queries x {T} keys"
+                      + (", over the dequantised rows" if u8 else "") + f"), {how}, {t_c:.2f} s a pass",
         }
         # the sample doubles as an end-to-end check of the timed outputs
         err = ((out.permute(0, 2, 1, 3)[:, : 4 * hs].float().cpu() - o_ref.float()).norm() / o_ref.float().norm()).item()
@@ -281,6 +310,7 @@ def bench_prefill(args, torch, dev):
             "unit": "TFLOP/s",
             "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
             "traffic": None if u8 else TRAFFIC_BYTES["prefill"],
+            "traffic_source": None if u8 else TRAFFIC_SOURCE,
         },
         "cpu_baseline": cpu,
     }
@@ -323,12 +353,10 @@ def bench_quantize(args, torch, dev):
     kgbs = bytes_alg / (ms_kernel * 1e-3) / 1e9
     cpu = None
     if not args.no_cpu_baseline:
-        torch.set_num_threads(min(16, os.cpu_count() or 1))
-        t_c0 = time.perf_counter()
-        c_ref, s_ref, z_ref = O.quantize_rows(kx)
-        t_c = time.perf_counter() - t_c0
-        cpu = {"value": round(bytes_alg / t_c / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": f"K tensor only (half the workload), one pass, {t_c:.1f} s"}
+        nthreads = cpu_threads(torch)
+        t_c, (c_ref, s_ref, z_ref), how = cpu_time(lambda: O.quantize_rows(kx))
+        cpu = {"value": round(bytes_alg / t_c / 1e9, 3), "unit": "GB/s", "cores": nthreads, "host_cpus": os.cpu_count(), "kind": "port",
+               "sample": f"K tensor only (half the workload), {how}, {t_c:.2f} s a pass"}
         assert torch.equal(outs[0][0].cpu(), c_ref) and torch.equal(outs[0][1].cpu(), s_ref) and torch.equal(outs[0][2].cpu(), z_ref)
     return {
         "metric": "uint8 row quantiser GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
@@ -337,7 +365,7 @@ def bench_quantize(args, torch, dev):
         "config": {"workload": "BASELINE.json configs[2] quantiser: K and V (1, 8, 65536, 128) bf16 -> uint8 + fp32 scale + int32 zero point, seed 2",
                    "bytes_algorithmic_per_tensor": bytes_alg},
         "roofline": {"bound": "hbm", "kernel": "quantize_rows_kernel<128>", "achieved": round(kgbs, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(kgbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["quantize"]},
+                     "unit": "GB/s", "frac": round(kgbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["quantize"], "traffic_source": TRAFFIC_SOURCE},
         "cpu_baseline": cpu,
     }
 
@@ -403,7 +431,7 @@ def bench_decode(args, torch, dev):
     ms_call = sum(a0.elapsed_time(a1) for a0, a1 in evs) / args.steps
     cpu = None
     if not args.no_cpu_baseline:
-        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        nthreads = cpu_threads(torch)
         nb = B  # the attention of one whole step
         if u8:
             unpack = O.uncompress4 if u4 else (lambda c: c)
@@ -412,12 +440,10 @@ def bench_decode(args, torch, dev):
         else:
             kc, vc = cache.k[:nb].cpu(), cache.v[:nb].cpu()
         qc = qs[0, :nb].cpu()
-        t_c0 = time.perf_counter()
-        O.sdpa_in_blocks(qc, kc, vc, D ** -0.5, L, None)
-        t_c = time.perf_counter() - t_c0
+        t_c, _, how = cpu_time(lambda: O.sdpa_in_blocks(qc, kc, vc, D ** -0.5, L, None))
         frac = nb / B
-        cpu = {"value": round(bytes_alg * frac / t_c / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": f"attention + score-sums of one step for batch rows 0-{nb - 1} of {B} ({frac:.2f} of a step), {t_c:.1f} s"}
+        cpu = {"value": round(bytes_alg * frac / t_c / 1e9, 3), "unit": "GB/s", "cores": nthreads, "host_cpus": os.cpu_count(), "kind": "port",
+               "sample": f"attention + score-sums of one step for batch rows 0-{nb - 1} of {B} ({frac:.2f} of a step), {how}, {t_c:.2f} s a pass"}
     return {
         "metric": "decode + H2O step GB/s (% HBM peak)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
@@ -428,7 +454,7 @@ def bench_decode(args, torch, dev):
         "roofline": {"bound": "hbm", "kernel": "kvx_sdpa_decode_h2o: decode_split_kernel<128,4,%s> + tail (merge, scratch-route weights, slot publishing)" % {"bf16": "KVX_KV_BF16", "uint8": "KVX_KV_U8", "uint4": "KVX_KV_U4"}[args.kv],
                      "achieved": round(bytes_alg / (ms_call * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(bytes_alg / (ms_call * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "ms_per_launch": round(ms_call, 4),
-                     "traffic": None if u8 else TRAFFIC_BYTES["decode"]},
+                     "traffic": None if u8 else TRAFFIC_BYTES["decode"], "traffic_source": None if u8 else TRAFFIC_SOURCE},
         "cpu_baseline": cpu,
     }
 
@@ -441,7 +467,7 @@ def bench_longctx(args, torch, dev):
     cfg = dataclasses.replace(QWEN3_4B, n_layer=args.layers)
     L, chunk, seq = 16384, 1024, args.tokens
     model = LongContextPrefillModel(cfg, cache_length=L, chunk_size=chunk, max_batch_size=1, quantized=True, max_context=max(seq, L), seed=4,
-                                    device=dev)
+                                    device=dev, gemm_table=not args.no_gemm_table)
     ids = torch.randint(0, cfg.vocab_size, (1, seq), generator=torch.Generator().manual_seed(4))
     sizes = model.chunk_sizes(seq)
     steps = max(1, min(args.steps, 3))
@@ -483,7 +509,7 @@ def bench_longctx(args, torch, dev):
         # 2048-slot cache, through the CPU oracle of the same stack (same op sequence as the reference's eager path)
         from oracle import longctx_oracle as LO
 
-        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        nthreads = cpu_threads(torch)
         c1 = dataclasses.replace(cfg, n_layer=1)
         layer = model.layers[0]
         weights = [{k: getattr(layer, k).cpu() for k in ("qkv", "proj", "fc_1", "fc_2", "mlp_proj", "norm_1", "norm_2", "norm_q", "norm_k")}]
@@ -493,7 +519,7 @@ def bench_longctx(args, torch, dev):
         ref.forward_chunk(ids[:, 2048:3072])
         ref.forward_chunk(ids[:, 3072:4096])
         t_c = time.perf_counter() - t_c0
-        cpu = {"value": round(4096 / t_c / cfg.n_layer, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        cpu = {"value": round(4096 / t_c / cfg.n_layer, 2), "unit": "tokens/s", "cores": nthreads, "host_cpus": os.cpu_count(), "kind": "port",
                "sample": f"one layer over 4096 tokens (2048-token first chunk, two 1024-token chunks, 2048-slot cache) in {t_c:.1f} s, "
                          f"scaled to {cfg.n_layer} layers"}
     tps = seq / (ms_step * 1e-3)
@@ -617,32 +643,6 @@ def bench_calib(args, torch, dev):
             "config": {"workload": "elementwise negate, 1 GiB read + 1 GiB written per launch", "bytes_read": 2 * n, "bytes_written": 2 * n}}
 
 
-def bench_ceiling(args, torch, dev):
-    import subprocess
-
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keys_values_amd", "mfma_probe")
-    if not os.path.exists(exe):
-        raise RuntimeError("keys_values_amd/mfma_probe is not built: run `python -m keys_values_amd.build`")
-    t0 = time.perf_counter()
-    out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300).stdout
-    print(out, file=sys.stderr, flush=True)
-    rows = []
-    for line in out.splitlines():
-        if "TFLOP/s" not in line:
-            continue
-        f = line.split()
-        i = f.index("wave/SIMD")
-        rows.append({"what": " ".join(f[: i - 1]), "waves_per_simd": int(f[i - 1]), "operands": f[i + 1], "ms": float(f[i + 2]),
-                     "ghz": float(f[i + 4]), "cycles_per_round": float(f[i + 6]), "tflops": float(f[i + 8])})
-    pure = [r for r in rows if r["what"] == "matrix instruction only" and r["operands"] == "random"]
-    best = max(pure, key=lambda r: r["tflops"])
-    return {"metric": "sustained bf16 MFMA TFLOP/s, matrix instructions only, random operands", "value": best["tflops"], "unit": "TFLOP/s",
-            "n_gpus": 1, "steps": 1, "warmup": 1, "ms_per_step": best["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": "keys_values_amd/mfma_probe: v_mfma_f32_32x32x16_bf16 loops over the whole device", "shader_clock_ghz": best["ghz"],
-                       "frac_of_nominal_peak": round(best["tflops"] / 2500.0, 3), "rows": rows, "wall_s": round(time.perf_counter() - t0, 1)}}
-
-
 def main():
     args = parse()
     if args.gpus != 1:
@@ -656,8 +656,7 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    fns = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib,
-           "ceiling": bench_ceiling}
+    fns = {"prefill": bench_prefill, "quantize": bench_quantize, "decode": bench_decode, "longctx": bench_longctx, "policy": bench_policy, "calib": bench_calib}
     res = fns[args.workload](args, torch, dev)
     if args.workload == "prefill" and args.kv == "bf16" and not args.no_secondary:
         # The other kernels with a target of their own, each on its own configuration, in the same run: the
@@ -666,14 +665,16 @@ def main():
         import gc
 
         secondary = {}
-        for name, steps, warmup in (("decode", 20, 5), ("quantize", 20, 5), ("longctx", 1, 1)):
+        legs = (("decode", "decode", "bf16", 20, 5), ("quantize", "quantize", "bf16", 20, 5),
+                ("prefill_uint8", "prefill", "uint8", 10, 3), ("longctx", "longctx", "bf16", 1, 1))
+        for name, workload, kv, steps, warmup in legs:
             sub = copy.copy(args)
-            sub.workload, sub.steps, sub.warmup = name, steps, warmup
+            sub.workload, sub.kv, sub.steps, sub.warmup = workload, kv, steps, warmup
             gc.collect()
             torch.cuda.empty_cache()
             t0 = time.perf_counter()
             try:
-                r = fns[name](sub, torch, dev)
+                r = fns[workload](sub, torch, dev)
                 secondary[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
                                    "steps": r["steps"], "warmup": r["warmup"], "dtype": r["dtype"], "workload": r["config"]["workload"],
                                    "detail": {k: v for k, v in r["config"].items() if k != "workload"},

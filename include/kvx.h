@@ -92,6 +92,12 @@ typedef struct kvx_sdpa_args {
 
   void* workspace;     /* scratch, kvx_sdpa_*_workspace_bytes(); may be NULL when that returns 0 */
   size_t workspace_bytes;
+
+  /* kvx_sdpa_decode / kvx_sdpa_decode_h2o with score-sums only, optional (NULL: not wanted): one device uint32 that the
+   * call sets to the number of (batch, KV head, split) workgroups whose logits went through the fp32 scratch in HBM
+   * instead of staying on the chip -- all of them when the splits are too long for the LDS or that form is switched
+   * off, else those whose bounded wait for their row ran out (normally 0; such a call is about 15 % slower). */
+  uint32_t* decode_scratch_splits;
 } kvx_sdpa_args;
 
 /* ---- library ------------------------------------------------------------------------------- */
@@ -164,6 +170,15 @@ size_t kvx_sdpa_decode_workspace_bytes(const kvx_sdpa_args* args);
 struct kvx_h2o_args;
 int kvx_sdpa_decode_h2o(const kvx_sdpa_args* args, const struct kvx_h2o_args* h, void* stream);
 size_t kvx_sdpa_decode_h2o_workspace_bytes(const kvx_sdpa_args* args);
+
+/* Process-wide switches of the decode kernels' weights route, for tests and measurement; no counterpart in the
+ * reference. resident: 0 sends every split's logits through the workspace and the tail kernel, 1 keeps them on the
+ * chip where they fit. spin_limit: polls a split spends waiting for the other splits of its row before it gives up
+ * and takes the workspace route (0 = never wait; clamped to 2^20). poll_sleep: pause between two polls in units of
+ * 512 cycles (clamped to 64). A negative value restores that switch to its default: the environment variables
+ * KVX_DECODE_RESIDENT / KVX_DECODE_SPIN_LIMIT / KVX_DECODE_POLL_SLEEP as read once at the first decode call
+ * (else 1, 32768, 4). A workspace size query and the call it is for must see the same setting of `resident`. */
+void kvx_decode_tuning(int resident, int spin_limit, int poll_sleep);
 
 /* ---- cache: quantiser ---------------------------------------------------------------------- */
 

@@ -27,6 +27,7 @@ class SdpaArgs(ctypes.Structure):
         ("o", c_void_p), ("o_stride_b", c_int64), ("o_stride_h", c_int64), ("o_stride_t", c_int64),
         ("lse", c_void_p), ("w", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("decode_scratch_splits", c_void_p),
     ]
 
 
@@ -92,6 +93,7 @@ SYMBOLS = {
     "kvx_sdpa_decode_workspace_bytes": (c_size_t, [POINTER(SdpaArgs)]),
     "kvx_sdpa_decode_h2o": (ctypes.c_int, [POINTER(SdpaArgs), POINTER(H2OArgs), c_void_p]),
     "kvx_sdpa_decode_h2o_workspace_bytes": (c_size_t, [POINTER(SdpaArgs)]),
+    "kvx_decode_tuning": (None, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "kvx_quantize_rows": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "kvx_dequantize_rows": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
     "kvx_quantize_rows4": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),

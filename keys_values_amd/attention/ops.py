@@ -235,9 +235,12 @@ def decode_core(
     return_lse: bool = False,
     quant: Optional[QuantState] = None,
     num_splits: int = 0,
+    scratch_splits: Optional[torch.Tensor] = None,
 ):
     """Single-token decode on strided views: query (B, Hq, 1, D), key/value (B, Hkv, T, D).
-    Returns ``(out (B, Hq, D), weights (B, Hkv, T) or None, lse (B, 1, Hq) or None)``."""
+    Returns ``(out (B, Hq, D), weights (B, Hkv, T) or None, lse (B, 1, Hq) or None)``.
+    ``scratch_splits``: optional one-element int32 device tensor that receives the number of KV splits whose logits
+    went through the HBM scratch instead of staying on the chip (0 in the normal case)."""
     _lib.require_gpu(query, key, value)
     for n, t in (("query", query), ("key", key), ("value", value)):
         _check_bhtd(n, t)
@@ -265,6 +268,10 @@ def decode_core(
         a.o_stride_b, a.o_stride_h, a.o_stride_t = o_view.stride(0), o_view.stride(1), o_view.stride(2)
         a.w = _lib.ptr(w)
         a.lse = _lib.ptr(lse)
+        if scratch_splits is not None:
+            if scratch_splits.dtype != torch.int32 or scratch_splits.numel() != 1 or scratch_splits.device != dev:
+                raise ValueError("scratch_splits must be a one-element int32 tensor on the query's device")
+            a.decode_scratch_splits = scratch_splits.data_ptr()
         nbytes = lib.kvx_sdpa_decode_workspace_bytes(ctypes.byref(a))
         ws = _lib.workspace(dev, nbytes)
         a.workspace = _lib.ptr(ws)

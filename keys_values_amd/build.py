@@ -50,22 +50,7 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{res.stdout}")
     if verbose:
         print(f"built {LIB}")
-    build_probe(verbose)
     return LIB
-
-
-PROBE = os.path.join(HERE, "mfma_probe")
-
-
-def build_probe(verbose: bool = True) -> str:
-    """The stand-alone ceiling probe (csrc/mfma_probe.hip), an executable next to the library."""
-    cmd = [HIPCC] + [f for f in FLAGS if f != "-fPIC"] + [os.path.join(CSRC, "mfma_probe.hip"), "-o", PROBE]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed on mfma_probe.hip:\n{res.stdout}")
-    if verbose:
-        print(f"built {PROBE}")
-    return PROBE
 
 
 if __name__ == "__main__":

@@ -162,6 +162,8 @@ size_t kvx_sdpa_decode_h2o_workspace_bytes(const kvx_sdpa_args* a) {
   return sdpa_decode_workspace(*a, true);
 }
 
+void kvx_decode_tuning(int resident, int spin_limit, int poll_sleep) { set_decode_tuning(resident, spin_limit, poll_sleep); }
+
 int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
   int rc = check_sdpa_common(a, "kvx_sdpa_decode", true);
   if (rc != KVX_OK) return rc;

@@ -7,6 +7,14 @@
 
 #include "../../include/kvx.h"
 
+// The kernels are written for gfx950 alone: its matrix instructions and transposing LDS reads, the direct
+// global -> LDS transfers, and (decode) cross-workgroup hand-offs through device-scope relaxed atomics that rely on
+// what this hardware does -- such stores write through to memory shared by all its dies and are counted by vmcnt,
+// such loads do not hit in the per-CU cache. Another target has to revisit all of that.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "libkvx: device code must be compiled with --offload-arch=gfx950 only"
+#endif
+
 namespace kvx {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -43,6 +51,7 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st);
 size_t score_sum_workspace(const kvx_sdpa_args& a);
 int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* fused_h2o, hipStream_t st);
 size_t sdpa_decode_workspace(const kvx_sdpa_args& a, bool fused_h2o);
+void set_decode_tuning(int resident, int spin_limit, int poll_sleep);
 int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,
                          int32_t* zp, hipStream_t st);
 int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,

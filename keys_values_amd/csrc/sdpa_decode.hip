@@ -27,6 +27,9 @@
 #include "kvx_common.h"
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
+
 namespace kvx {
 namespace {
 
@@ -52,6 +55,7 @@ struct DecodeParams {
                              // the fused H2O form, the row's workgroups of the tail kernel that have finished
   uint32_t* split_done;      // (B, Hkv, S): 1 where the split kernel itself turned its logits into weights
   uint32_t* tail_count;      // fused H2O form: workgroups of the tail kernel's second kind that have finished
+  uint32_t* scratch_splits;  // caller's counter of the splits whose logits went through the scratch, or NULL
   int32_t resident;          // the logits of a split stay in LDS
   int32_t spin_limit;        // polls of row_count before a workgroup gives up and sends its logits out
   int32_t poll_sleep;        // pause between two polls, in units of 512 cycles
@@ -399,7 +403,10 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
   __syncthreads();
   if (!row_ready) {
     flush_logits();
-    if (tid == 0) p.split_done[(int64_t)row * p.num_splits + split] = 0u;
+    if (tid == 0) {
+      p.split_done[(int64_t)row * p.num_splits + split] = 0u;
+      if (p.scratch_splits) atomicAdd(p.scratch_splits, 1u);
+    }
     return;
   }
   for (int g = wave; g < G; g += WAVES) {  // a wavefront per head: lane s takes splits s, s + 64, ...
@@ -451,13 +458,15 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 }
 
 // Before the split kernel: no split of a row has arrived, no row has a lowest-score slot yet.
-__global__ void decode_init_kernel(uint32_t* row_count, unsigned long long* best, uint32_t* tail_count, int rows) {
+__global__ void decode_init_kernel(uint32_t* row_count, unsigned long long* best, uint32_t* tail_count, int rows,
+                                   uint32_t* scratch_splits, uint32_t scratch_splits_init) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < rows) {
     if (row_count) row_count[i * kCountStride] = 0u;
     if (best) best[i] = ~0ull;
   }
   if (i == 0 && tail_count) *tail_count = 0u;
+  if (i == 0 && scratch_splits) *scratch_splits = scratch_splits_init;
 }
 
 // Combine the splits of one (b, query head): 4 groups of D threads each take a quarter of the
@@ -628,11 +637,37 @@ struct Plan {
   size_t off_logits, off_part_o, off_part_ml, off_best, off_tail, off_count, off_done, total;
 };
 
-// KVX_DECODE_RESIDENT=0 sends every split's logits through the scratch; KVX_DECODE_SPIN_LIMIT bounds the
-// wait for a row's other splits (0: no wait, every workgroup takes the scratch route). Read at every call.
+// Switches of the route the logits take, process-wide. Defaults come from the environment, read ONCE (first use):
+// KVX_DECODE_RESIDENT=0 sends every split's logits through the scratch; KVX_DECODE_SPIN_LIMIT bounds the wait for a
+// row's other splits in polls (0: no wait, every workgroup takes the scratch route); KVX_DECODE_POLL_SLEEP is the
+// pause between two polls in units of 512 cycles. kvx_decode_tuning() replaces them at run time. Values are clamped:
+// the longest wait a workgroup can spend is spin_limit x (poll_sleep x 512 + a load's latency) cycles, i.e.
+// 2^20 x 64 x 512 cycles = 16 s at the clamps and about 30 ms at the defaults (2^15 polls, 4 x 512 cycles).
+constexpr int kSpinDefault = 1 << 15, kSpinMax = 1 << 20, kSleepDefault = 4, kSleepMax = 64;
+struct Tuning {
+  std::atomic<int> resident{1}, spin_limit{kSpinDefault}, poll_sleep{kSleepDefault};
+  int env_resident = 1, env_spin = kSpinDefault, env_sleep = kSleepDefault;
+};
+int clampi(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
 int env_int(const char* name, int dflt) {
   const char* e = getenv(name);
-  return e && *e ? atoi(e) : dflt;
+  if (!e || !*e) return dflt;
+  char* end = nullptr;
+  const long v = strtol(e, &end, 10);
+  return (end == e || *end) ? dflt : (int)(v < -1 ? -1 : (v > (1l << 30) ? (1l << 30) : v));  // not a number: the default
+}
+Tuning& tuning() {
+  static Tuning t;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    t.env_resident = env_int("KVX_DECODE_RESIDENT", 1) != 0;
+    t.env_spin = clampi(env_int("KVX_DECODE_SPIN_LIMIT", kSpinDefault), 0, kSpinMax);
+    t.env_sleep = clampi(env_int("KVX_DECODE_POLL_SLEEP", kSleepDefault), 0, kSleepMax);
+    t.resident = t.env_resident;
+    t.spin_limit = t.env_spin;
+    t.poll_sleep = t.env_sleep;
+  });
+  return t;
 }
 
 Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
@@ -647,7 +682,7 @@ Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   // 262144 keys take 182 us in one round of 4096 keys and 265 in four of 1024. Without weights: 32 rows of 262144
   // keys 631 us in 16 splits, 658 in 128; 8 rows of 16384 keys 22 us in 32 splits, 26 in 16 of 1024.
   const bool weights = a.w || fused_h2o;
-  const int allow_resident = weights ? env_int("KVX_DECODE_RESIDENT", 1) : 0;
+  const int allow_resident = weights ? tuning().resident.load() : 0;
   const int lgk = logit_floats(pl.G, a.D) / pl.G;
   int splits = a.num_splits;
   if (splits <= 0) {
@@ -705,9 +740,11 @@ template <int D, int G>
 int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t st) {
   dim3 grid(p.num_splits, p.Hkv, p.B);
   const int rows = p.B * p.Hkv;
-  if (p.resident || hh) {
-    hipLaunchKernelGGL(decode_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, p.row_count, hh ? p.best : nullptr,
-                       hh ? p.tail_count : nullptr, rows);
+  if (p.resident || hh || p.scratch_splits) {
+    // splits that take the scratch route by plan (the resident form switched off or too long for the LDS) count from the start
+    const uint32_t by_plan = (p.logits && !p.resident) ? (uint32_t)(rows * p.num_splits) : 0u;
+    hipLaunchKernelGGL(decode_init_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, (p.resident || hh) ? p.row_count : nullptr,
+                       hh ? p.best : nullptr, hh ? p.tail_count : nullptr, rows, p.scratch_splits, by_plan);
     KVX_HIP(hipGetLastError());
   }
   const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
@@ -737,6 +774,13 @@ int launch_d(const DecodeParams& p, int G, int kv, const kvx_h2o_args* hh, hipSt
 
 size_t sdpa_decode_workspace(const kvx_sdpa_args& a, bool fused_h2o) { return make_plan(a, fused_h2o).total; }
 
+void set_decode_tuning(int resident, int spin_limit, int poll_sleep) {
+  Tuning& t = tuning();
+  t.resident = resident < 0 ? t.env_resident : (resident != 0);
+  t.spin_limit = spin_limit < 0 ? t.env_spin : clampi(spin_limit, 0, kSpinMax);
+  t.poll_sleep = poll_sleep < 0 ? t.env_sleep : clampi(poll_sleep, 0, kSleepMax);
+}
+
 int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream_t st) {
   const Plan pl = make_plan(a, hh != nullptr);
   KVX_REQUIRE(a.workspace && a.workspace_bytes >= pl.total, KVX_ERR_WORKSPACE,
@@ -761,9 +805,10 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.tail_count = hh ? (uint32_t*)(ws + pl.off_tail) : nullptr;
   p.row_count = (uint32_t*)(ws + pl.off_count);
   p.split_done = (uint32_t*)(ws + pl.off_done);
+  p.scratch_splits = a.decode_scratch_splits;
   p.resident = pl.resident;
-  p.spin_limit = env_int("KVX_DECODE_SPIN_LIMIT", 1 << 15);
-  p.poll_sleep = env_int("KVX_DECODE_POLL_SLEEP", 4);
+  p.spin_limit = tuning().spin_limit.load();
+  p.poll_sleep = tuning().poll_sleep.load();
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
   p.Gr = a.Hq / a.Hkv;
   KVX_REQUIRE(p.Gr <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);

@@ -130,6 +130,8 @@ class KVCacheBuffers:
     def forward(self, positions: PositionsType, key: torch.Tensor, value: torch.Tensor) -> KeysAndValues:
         """Write ``key`` / ``value`` to the slots ``positions``, return the buffers up to the current length
         (keys_values/kvcache/buffers.py:231-262)."""
+        if self.batch_size is None or self.current_length is None:
+            raise IndexError("Buffers are not initialised, call 'prefill' first")
         num = key.shape[2]
         self.current_length = min(self.cache_length, self.current_length + num)
         return self._forward(positions, key, value)
@@ -241,6 +243,8 @@ class HipKVCacheBuffers(KVCacheBuffers):
     def _require_buffers(self):
         if not self.buffers_are_allocated:
             raise IndexError("Buffers are not allocated. Call 'prefill' first")
+        if self.batch_size is None or self.current_length is None:
+            raise IndexError("Buffers are not initialised, call 'prefill' first")
 
     # -- slots (keys_values/kvcache/buffers.py:482-551) ----------------------------------------------------
 

@@ -10,7 +10,6 @@ keys_values/model.py:294-301); the linear layers are plain library GEMMs through
 else runs on the HIP kernels of this package. There is no CPU path.
 """
 import os
-import tempfile
 from dataclasses import dataclass
 from typing import List, Optional
 
@@ -63,29 +62,44 @@ GEMM_TABLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_tabl
 
 
 def use_gemm_table(path: str = GEMM_TABLE) -> bool:
-    """The linear layers are plain library GEMMs, and which kernel serves a shape is the library's choice; its
+    """Opt-in, process-wide: fix which library kernel serves each GEMM shape of this stack.
+
+    The linear layers are plain library GEMMs, and which kernel serves a shape is the library's choice; its
     default is a poor one for some of the shapes of this stack. The table next to this file records, per shape
     (Qwen3-4B widths, chunks of 1024 and 16384 tokens), the kernel PyTorch's TunableOp measured as fastest on
     gfx950; it is read with tuning switched off, so nothing is measured at run time and the choice is the same in
-    every run. The file names the library versions it was made with: PyTorch refuses it under other versions,
-    and the library's default choice stays in place (returns False). Process-wide, like TunableOp itself."""
+    every run. This switches TunableOp on for EVERY GEMM of the process (shapes outside the table keep the
+    library default, but the table's shapes change kernel, and with it summation order, wherever they occur),
+    which is why nothing calls it implicitly. The file names the library versions it was made with: PyTorch
+    refuses it under other versions; then, or on any other failure, the switches of TunableOp are put back as
+    they were found and False is returned. TunableOp's own results file name is left alone."""
     import torch.cuda.tunable as tunable
 
     if not os.path.exists(path):
         return False
     try:
+        before = (tunable.is_enabled(), tunable.tuning_is_enabled(), tunable.record_untuned_is_enabled())
+    except Exception:  # a PyTorch without TunableOp
+        return False
+    ok = False
+    try:
         tunable.enable(True)
         tunable.tuning_enable(False)
         tunable.record_untuned_enable(False)
-        tunable.set_filename(os.path.join(tempfile.gettempdir(), "kvx_tunableop_results.csv"))  # never into the caller's directory
-        return bool(tunable.read_file(path))
-    except Exception:  # a PyTorch without TunableOp, or a table it cannot parse: the default choice stays
-        return False
+        ok = bool(tunable.read_file(path))
+    except Exception:  # a table it cannot parse
+        ok = False
+    if not ok:
+        tunable.enable(before[0])
+        tunable.tuning_enable(before[1])
+        tunable.record_untuned_enable(before[2])
+    return ok
 
 
 class LongContextPrefillModel:
     def __init__(self, cfg: PrefillConfig, cache_length: int, chunk_size: int, max_batch_size: int = 1, quantized: bool = True,
-                 max_context: int = 131072, seed: int = 4, device: Optional[torch.device] = None, gemm_table: bool = True):
+                 max_context: int = 131072, seed: int = 4, device: Optional[torch.device] = None, gemm_table: bool = False):
+        """``gemm_table=True`` calls :func:`use_gemm_table` (process-wide, see there); off by default."""
         self.cfg = cfg
         self.gemm_table = use_gemm_table() if gemm_table else False
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())

@@ -34,12 +34,12 @@ def gpu(kvx):
 # How the logits become weights: inside the split kernel once the row's other splits have arrived
 # (the default), through the scratch buffer and the weights kernel (resident form switched off), and
 # the bounded wait running out in every workgroup (limit 0) or in most of them (limit 1).
-DECODE_ROUTES = {"resident": {}, "scratch": {"KVX_DECODE_RESIDENT": "0"}, "no-wait": {"KVX_DECODE_SPIN_LIMIT": "0"},
-                 "one-poll": {"KVX_DECODE_SPIN_LIMIT": "1"}}
+# (resident, spin_limit, poll_sleep) for kvx_decode_tuning; -1 = the default
+DECODE_ROUTES = {"resident": (-1, -1, -1), "scratch": (0, -1, -1), "no-wait": (-1, 0, -1), "one-poll": (-1, 1, -1)}
 
 
 @pytest.fixture(params=list(DECODE_ROUTES))
-def decode_route(request, monkeypatch):
-    for name, value in DECODE_ROUTES[request.param].items():
-        monkeypatch.setenv(name, value)
-    return request.param
+def decode_route(request, kvx):
+    kvx.kvx_decode_tuning(*DECODE_ROUTES[request.param])
+    yield request.param
+    kvx.kvx_decode_tuning(-1, -1, -1)

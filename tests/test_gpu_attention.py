@@ -219,6 +219,30 @@ def test_decode_with_weights(gpu, decode_route, B, Hq, Hkv, T, D, splits):
     check_o(out3.unsqueeze(2), o_ref)
 
 
+def test_decode_reports_the_splits_that_took_the_scratch_route(kvx, gpu):
+    """The optional counter of a decode call: 0 when every split turned its own logits into weights, every split
+    when that form is switched off or no split waits, and nothing written without score-sums."""
+    B, Hq, Hkv, T, D = 2, 8, 2, 20000, 128
+    q, k, v, _ = make_qkv(77, B, Hq, Hkv, 1, T, D)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    scale = 1.0 / math.sqrt(D)
+    counts, ws = {}, {}
+    try:
+        for name, setting in (("resident", (-1, -1, -1)), ("scratch", (0, -1, -1)), ("no-wait", (-1, 0, -1))):
+            kvx.kvx_decode_tuning(*setting)
+            n = torch.full((1,), -5, dtype=torch.int32, device=gpu)
+            _, ws[name], _ = ops.decode_core(qg, kg, vg, scale, return_weights=True, scratch_splits=n)
+            counts[name] = int(n.item())
+    finally:
+        kvx.kvx_decode_tuning(-1, -1, -1)
+    assert counts["resident"] == 0
+    assert counts["scratch"] == counts["no-wait"] and counts["scratch"] >= B * Hkv and counts["scratch"] % (B * Hkv) == 0
+    assert torch.equal(ws["resident"], ws["scratch"]) and torch.equal(ws["resident"], ws["no-wait"])
+    n = torch.full((1,), -5, dtype=torch.int32, device=gpu)
+    ops.decode_core(qg, kg, vg, scale, return_weights=False, scratch_splits=n)
+    assert int(n.item()) == 0  # no logits, nothing through the scratch
+
+
 def test_full_size_prefill_properties(gpu):
     """Configuration 2 at its real shape (B1, 32/8 heads, D128, 32768 slots, 1024 queries, RoPE):
     one KV head against the oracle, row sums, and layout independence (scattered slots give the
@@ -413,6 +437,7 @@ def test_decode_with_weights_beside_other_work(gpu):
     torch.cuda.synchronize()
     side = torch.cuda.Stream(gpu)
     busy = torch.randn(4096, 4096, device=gpu, dtype=torch.bfloat16)
+    side.wait_stream(torch.cuda.current_stream(gpu))  # `busy` was made on the current stream
     for _ in range(3):
         with torch.cuda.stream(side):
             for _ in range(20):

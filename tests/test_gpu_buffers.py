@@ -81,3 +81,15 @@ def test_buffers_reject_the_cpu(gpu):
         bufs.prefill(torch.zeros(1, 2, 4, 64, dtype=torch.bfloat16), torch.zeros(1, 2, 4, 64, dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
         create_kv_cache_buffers("bnb-quantized4", KVCacheBuffersParams(1, 2, 64, None, torch.bfloat16), 16)
+
+
+def test_buffers_before_prefill_raise_a_clear_error(gpu):
+    """forward / set_slots / get_slots on buffers that have not seen a prefill: IndexError, not a TypeError from None."""
+    bufs = create_kv_cache_buffers("default", KVCacheBuffersParams(1, 2, 64, None, torch.bfloat16), 16)
+    x = torch.zeros(1, 2, 4, 64, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(IndexError):
+        bufs.forward((0, 4), x, x)
+    with pytest.raises(IndexError):
+        bufs.set_slots((0, 4), x, x)
+    with pytest.raises(IndexError):
+        bufs.get_slots((0, 4))

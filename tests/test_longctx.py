@@ -393,3 +393,26 @@ def test_prefill_model_vs_oracle(gpu, quantized):
         for li, cache in enumerate(model.caches):
             assert torch.equal(cache.token_pos.cpu(), ref.caches[li].token_pos)
         start += n
+
+
+@pytest.mark.gpu
+def test_gemm_table_is_opt_in_and_restores_state(gpu, tmp_path):
+    """Building the model does not touch TunableOp; a table PyTorch refuses (other library versions) leaves its
+    switches as they were found."""
+    import torch.cuda.tunable as tunable
+
+    from keys_values_amd.longctx.model import LongContextPrefillModel, PrefillConfig, use_gemm_table
+
+    def state():
+        return tunable.is_enabled(), tunable.tuning_is_enabled(), tunable.record_untuned_is_enabled()
+
+    before = state()
+    cfg = PrefillConfig(n_layer=1, n_embd=128, n_head=4, n_query_groups=2, head_size=64, intermediate_size=256, vocab_size=100)
+    model = LongContextPrefillModel(cfg, cache_length=128, chunk_size=64, max_batch_size=1, quantized=False, max_context=512, seed=4, device=gpu)
+    assert model.gemm_table is False and state() == before
+    bad = tmp_path / "mismatch.csv"
+    bad.write_text("Validator,PT_VERSION,0.0.1\nValidator,HIP_VERSION,1\nGemmTunableOp_BFloat16_TN,tn_8_8_8_ld_8_8_8,Gemm_Rocblas_1,0.01\n")
+    assert use_gemm_table(str(bad)) is False
+    assert state() == before
+    assert use_gemm_table(str(tmp_path / "absent.csv")) is False
+    assert state() == before
