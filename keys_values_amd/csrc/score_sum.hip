@@ -39,112 +39,141 @@ struct ScoreParams {
   int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, qs_sb, qs_sh, tp_sb, tp_sh;
 };
 
+// Q tile in LDS: [row][16-byte chunk], rows unpadded (what the global -> LDS transfer writes: a wavefront
+// instruction fills 1024 contiguous bytes), chunk c of row r stored at position c ^ swz(r). The operand reads
+// (ds_read_b128, 16 consecutive rows and the same chunk per phase) then touch every bank once.
+template <int CPR>
+__device__ __forceinline__ int swz(int r) { return CPR >= 16 ? (r & 15) : ((r >> 1) & 7); }
+
 template <int D>
 struct alignas(16) Smem {
-  static constexpr int QCH16 = D / 8 + 1;  // 16-byte chunks per row incl. pad (conflict-free ds_read_b128)
-  u32x4_t q[2][BQ][QCH16];
-  float lse[3][BQ];   // read one phase later than q, hence one more buffer
-  int32_t qpos[3][BQ];
+  static constexpr int CPR = D / 8;  // 16-byte chunks per row
+  u32x4_t q[2][BQ][CPR];
+  float lse[2][BQ];     // a tile's log-sum-exps are in registers before the barrier that frees its Q buffer
+  int32_t qpos[4][BQ];  // read through the whole step (only by tiles that need the mask): a ring of four
 };
 
-template <int D, int W>
-struct QStage {
-  static constexpr int QCH = (BQ * D / 8) / (64 * W);  // W = 4: 4 (D=128), 2 (D=64)
-  u32x4_t qr[QCH];
-  float lse;
-  int32_t qpos;
-};
-
-// Streams the packed query rows (row r = query r / G, head r % G) of one (batch, KV head) pair.
-// The (query, head) of each row this thread loads is advanced incrementally from tile to tile,
-// so the loop has no integer division.
+// Streams the packed query rows (row r = query r / G, head r % G) of one (batch, KV head) pair into LDS, tile by
+// tile, with global -> LDS transfers: no registers hold the rows on their way. Wavefront w issues instructions
+// w, w + W, ... of the CPR that make a tile (RPW = 64 / CPR rows each); lane l of instruction i fills LDS position
+// l % CPR of row i RPW + l / CPR, so it fetches the chunk that belongs there under the swizzle. Addresses are a
+// uniform base plus a 32-bit byte offset per lane (the host checks the range). Wavefront 0 also fetches the rows'
+// log-sum-exps (4 bytes per lane) and writes their positions.
+//   issue_steady: G divides the tile height and the tile is full. Every row keeps its head and moves by BQ / G
+//     queries from tile to tile: the base advances by scalar adds and the lane offsets stay.
+//   issue: any tile. The offsets are formed per lane from the row's (query, head); rows past the end re-read the
+//     last valid row, and land() overwrites their log-sum-exp with +inf, so their weight is exactly zero.
 template <int D, int W>
 struct QLoader {
-  static constexpr int NTHREADS = 64 * W;
   static constexpr int CPR = D / 8;
-  static constexpr int RPI = NTHREADS / CPR;
-  static constexpr int QCH = QStage<D, W>::QCH;
-  const uint16_t* qbase;  // (b, first head of the group)
-  const float* lbase;     // lse + b * q_len * Hq + kvh * G
-  int64_t q_sh, q_st;
-  int G, R, Hq, input_pos, row_in, col;
-  int qi[QCH], g[QCH];    // row of chunk i in the current tile
-  int lqi, lg;            // row of the lse / position this thread stages (tid < BQ)
-  int dq, dg;             // BQ / G, BQ % G
-  const uint16_t* src[QCH];  // dg == 0: address of chunk i in the current tile
-  int64_t step;              // dg == 0: elements between consecutive tiles
+  static constexpr int RPW = 64 / CPR;
+  static constexpr int NI = CPR / W;      // transfers per wavefront and tile
+  static constexpr int TILE_BYTES = BQ * CPR * 16;
+  const char* qbase;   // (b, first head of the group)
+  const char* lbase;   // lse + b * q_len * Hq + kvh * G
+  const char* qtile;   // issue_steady: qbase advanced to the tile it fetches next
+  const char* ltile;   // likewise for the log-sum-exps
+  uint32_t voff0[NI];  // issue_steady: byte offset of this lane's chunk of instruction i relative to qtile
+  uint32_t loff0;      // likewise for the log-sum-exp of row `lane`
+  int qpv;             // likewise the position of row `lane`
+  uint32_t cb[NI];     // byte offset of the chunk inside a row
+  int rin[NI];         // row inside the tile
+  uint32_t q_shb, q_stb, qstep, lstep;
+  float inv_g;         // 1 / G: (int)((r + 0.5f) * inv_g) == r / G for the small r of a tile
+  int G, R, Hq, input_pos, dq, dg, wave, lane;
+  int q0, g0;          // (query, head) of the first row of the next tile to fetch
+  uint32_t lds_qw, lds_lse, lds_qpos;
+  int next_row0;       // first row of the next tile to fetch
 
-  __device__ __forceinline__ void init(const ScoreParams& p, int b, int kvh, int tid, int row_start) {
-    col = tid % CPR;
-    row_in = tid / CPR;
+  // steady_first: index (counted from row_start) of the first tile issue_steady will be asked for
+  __device__ __forceinline__ void init(const ScoreParams& p, Smem<D>& sm, int b, int kvh, int tid, int row_start, int steady_first) {
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    lane = tid & 63;
     G = p.G; R = p.R; Hq = p.Hq; input_pos = p.input_pos;
-    q_sh = p.q_sh; q_st = p.q_st;
-    qbase = p.q + b * p.q_sb + (int64_t)(kvh * p.G) * p.q_sh;
-    lbase = p.lse + (int64_t)b * p.q_len * p.Hq + kvh * p.G;
+    q_shb = (uint32_t)p.q_sh * 2u; q_stb = (uint32_t)p.q_st * 2u;
+    qbase = (const char*)(p.q + b * p.q_sb + (int64_t)(kvh * p.G) * p.q_sh);
+    lbase = (const char*)(p.lse + (int64_t)b * p.q_len * p.Hq + kvh * p.G);
     dq = BQ / G; dg = BQ % G;
+    inv_g = 1.0f / (float)G;
+    qstep = (uint32_t)dq * q_stb;
+    lstep = (uint32_t)(dq * Hq) * 4u;
+    q0 = row_start / G;
+    g0 = row_start % G;
+    const int qs = q0 + steady_first * dq;        // dg == 0: row_start is a multiple of BQ, hence of G
+    qtile = qbase + (uint64_t)qs * q_stb;
+    ltile = lbase + (uint64_t)(qs * Hq) * 4u;
+    qpv = input_pos + qs + lane / G;
+    lds_qw = __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.q[0][0][0]) + (uint32_t)(wave * 1024));
+    lds_lse = __builtin_amdgcn_readfirstlane(lds_addr_of(&sm.lse[0][0]));
+    lds_qpos = lds_addr_of(&sm.qpos[0][0]) + (uint32_t)(lane * 4);
 #pragma unroll
-    for (int i = 0; i < QCH; ++i) {
-      const int r = row_start + row_in + i * RPI;
-      qi[i] = r / G;
-      g[i] = r % G;
-      src[i] = qbase + (int64_t)g[i] * q_sh + (int64_t)qi[i] * q_st + col * 8;
+    for (int i = 0; i < NI; ++i) {
+      rin[i] = (wave + W * i) * RPW + lane / CPR;
+      cb[i] = (uint32_t)(((lane % CPR) ^ swz<CPR>(rin[i])) * 16);
+      voff0[i] = (uint32_t)(rin[i] % G) * q_shb + (uint32_t)(rin[i] / G) * q_stb + cb[i];
     }
-    step = (int64_t)dq * q_st;
-    lqi = (row_start + tid) / G;
-    lg = (row_start + tid) % G;
+    loff0 = (uint32_t)((lane / G) * Hq + lane % G) * 4u;
+    next_row0 = row_start;
   }
 
-  // fetch the tile whose first row is row0, then step the row bookkeeping to the next tile
-  __device__ __forceinline__ void fetch(QStage<D, W>& s, int row0, int tid) {
-    if (dg == 0) {
-      // G divides the tile height: every row keeps its head and moves by BQ / G queries per tile.
-      // Rows past the end read row 0 (finite data); their lse = +inf makes their weight zero.
-#pragma unroll
-      for (int i = 0; i < QCH; ++i) {
-        const bool ok = row0 + row_in + i * RPI < R;
-        s.qr[i] = *(const u32x4_t*)(ok ? src[i] : qbase);
-        src[i] += step;
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < QCH; ++i) {
-        const bool ok = row0 + row_in + i * RPI < R;
-        const uint16_t* ptr = qbase + (int64_t)g[i] * q_sh + (int64_t)(ok ? qi[i] : 0) * q_st + col * 8;
-        s.qr[i] = *(const u32x4_t*)(ok ? ptr : qbase);
-        qi[i] += dq;
-        g[i] += dg;
-        if (g[i] >= G) {
-          g[i] -= G;
-          qi[i] += 1;
-        }
-      }
+  template <int BUF, int I = 0>
+  __device__ __forceinline__ void dma_q_steady() {
+    dma16_at<(uint32_t)(BUF * TILE_BYTES + W * I * 1024)>(qtile, voff0[I], lds_qw);
+    if constexpr (I + 1 < NI) dma_q_steady<BUF, I + 1>();
+  }
+  template <int BUF>
+  __device__ __forceinline__ void issue_steady(Smem<D>& sm, int ring) {
+    dma_q_steady<BUF>();
+    if (wave == 0) {
+      dma4_at<(uint32_t)(BUF * BQ * 4)>(ltile, loff0, lds_lse);
+      sm.qpos[ring][lane] = qpv;
+      qpv += dq;
     }
-    if (tid < BQ) {
-      const bool ok = row0 + tid < R;
-      // rows past the end get lse = +inf so that exp2(... - lse) = 0
-      s.lse = ok ? lbase[(int64_t)lqi * Hq + lg] : INFINITY;
-      s.qpos = ok ? input_pos + lqi : INT_MAX;
-      lqi += dq;
-      lg += dg;
-      if (lg >= G) {
-        lg -= G;
-        lqi += 1;
-      }
-    }
+    qtile += qstep;
+    ltile += lstep;
+    q0 += dq;
+    next_row0 += BQ;
   }
 
-  __device__ __forceinline__ void commit(const QStage<D, W>& s, Smem<D>& sm, int buf, int buf3, int tid) const {
+  // start the transfers of the next tile into Q / lse buffer `buf` and position buffer `ring`
+  __device__ __forceinline__ void issue(Smem<D>& sm, int buf, int ring) {
+    const int row0 = next_row0;
+    const int rl = R - 1;
 #pragma unroll
-    for (int i = 0; i < QCH; ++i) sm.q[buf][row_in + i * RPI][col] = s.qr[i];
-    if (tid < BQ) {
-      sm.lse[buf3][tid] = s.lse;
-      sm.qpos[buf3][tid] = s.qpos;
+    for (int i = 0; i < NI; ++i) {
+      const int r = min(g0 + rin[i] + q0 * G, rl) - q0 * G;  // row relative to (q0, head 0), clamped to the last valid row
+      const int dqi = (int)(((float)r + 0.5f) * inv_g);         // r / G, r < G + BQ
+      dma16(qbase, (uint32_t)(r - dqi * G) * q_shb + (uint32_t)(q0 + dqi) * q_stb + cb[i], lds_qw + (uint32_t)(buf * TILE_BYTES + W * i * 1024));
     }
+    if (wave == 0) {
+      const bool ok = row0 + lane < R;
+      const int r = min(g0 + lane + q0 * G, rl) - q0 * G;
+      const int dqi = (int)(((float)r + 0.5f) * inv_g);
+      dma4(lbase, (uint32_t)((q0 + dqi) * Hq + (r - dqi * G)) * 4u, lds_lse + (uint32_t)(buf * BQ * 4));
+      sm.qpos[ring][lane] = ok ? input_pos + q0 + dqi : INT_MAX;
+    }
+    q0 += dq;
+    g0 += dg;
+    if (g0 >= G) {
+      g0 -= G;
+      q0 += 1;
+    }
+    next_row0 = row0 + BQ;
+  }
+
+  // after s_waitcnt vmcnt(0), before the barrier that publishes the tile whose first row is row0
+  __device__ __forceinline__ void land(Smem<D>& sm, int row0, int buf) const {
+    if (row0 + BQ > R && wave == 0 && row0 + lane >= R) sm.lse[buf][lane] = INFINITY;  // exp2(... - inf) = 0
   }
 };
 
 // QSPLIT: the query rows are split over blockIdx.z (short caches that would otherwise leave compute units
 // idle); every split writes its sums to p.part and a second kernel adds them in a fixed order.
+//
+// The kernel is bound by the number of instructions a wavefront issues per tile (two wavefronts per SIMD issue
+// about one instruction per ten cycles each, whatever its kind), so the tile loop comes in three forms: tiles that
+// need the position mask and tiles that do not, each unrolled by two with every LDS address an immediate and the
+// transfers of the tile after next sent without bounds checks ("steady"), and a general form for the last tiles.
 template <int D, int KV, int W, bool QSPLIT>
 __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
   constexpr int BK = NW * W;  // keys per workgroup
@@ -202,40 +231,69 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
   float wacc[2] = {0.0f, 0.0f};
   const int tbase = QSPLIT ? (int)blockIdx.z * p.tiles_per_z : 0;  // first query tile of this workgroup
   const int num_qt = QSPLIT ? min(p.tiles_per_z, (p.R + BQ - 1) / BQ - tbase) : (p.R + BQ - 1) / BQ;
+  // Steps [0, t_steady) are steady: G divides the tile height and tiles t + 1 and t + 2 exist and are full.
+  // Steps [0, t_masked) need the mask: the first query position of tile t, input_pos + (tbase + t) BQ / G, is below
+  // the largest key position of this wavefront. Both are even, so the buffer index stays a compile-time constant.
+  const int nfull = min(num_qt, p.R / BQ - tbase);
+  const int t_steady = (BQ % p.G == 0) ? (max(nfull - 2, 0) & ~1) : 0;
+  int t_masked;
+  {
+    const int64_t need = (int64_t)max(min(tpmax, p.input_pos + p.q_len) - p.input_pos, 0) * p.G;  // rows whose position is below tpmax
+    const int64_t tiles = (need + BQ - 1) / BQ - tbase;
+    t_masked = (int)max((int64_t)0, min(tiles, (int64_t)num_qt));
+    t_masked = min((t_masked + 1) & ~1, t_steady);
+  }
   QLoader<D, W> ld;
-  ld.init(p, b, kvh, tid, tbase * BQ);
-  QStage<D, W> st;
+  ld.init(p, sm, b, kvh, tid, tbase * BQ, 2);
+  // LDS byte offsets of this lane's Q fragments (A operand): row mt 32 + n, chunk 2 j + h at position chunk ^ swz(row)
+  constexpr int CPR = D / 8;
+  uint32_t qa[D / 16];
+#pragma unroll
+  for (int j = 0; j < D / 16; ++j) qa[j] = (uint32_t)((n * CPR + ((2 * j + h) ^ swz<CPR>(n))) * 16);
 
-  // S block = 32 query rows x 64 keys: Q rows come from LDS (A operand), K sits in registers.
-  auto mfma_block = [&](f32x16_t (&s)[2], int buf, int mt) {
+  // The Q fragments of a block (32 query rows, A operand) and the rows' log-sum-exps are requested together, ahead
+  // of the block's first matrix instruction: the reads then have the previous block's tail to arrive in. BUF is a
+  // compile-time constant, so every read is one address register plus an immediate offset.
+  auto load_q = [&](u32x4_t (&qq)[D / 16], auto buf_tag, auto mt_tag) {
+    constexpr int BUF = decltype(buf_tag)::value, MT = decltype(mt_tag)::value;
+    const char* qb = (const char*)&sm.q[BUF][MT * 32][0];
+#pragma unroll
+    for (int j = 0; j < D / 16; ++j) qq[j] = *(const u32x4_t*)(qb + qa[j]);
+  };
+  // accumulator rows of a lane are 8 a + 4 h + (0..3)
+  auto load_lse = [&](f32x4_t (&ls)[4], auto buf_tag, auto mt_tag) {
+    constexpr int BUF = decltype(buf_tag)::value, MT = decltype(mt_tag)::value;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) ls[a] = *(const f32x4_t*)&sm.lse[BUF][MT * 32 + 8 * a + 4 * h];
+  };
+  // S block = 32 query rows x 64 keys, K in registers
+  auto mfma_block = [&](f32x16_t (&s)[2], const u32x4_t (&qq)[D / 16]) {
 #pragma unroll
     for (int j = 0; j < D / 16; ++j) {
-      const u32x4_t qq = sm.q[buf][mt * 32 + n][2 * j + h];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
         if (j == 0) {
           const f32x16_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          s[nt] = mfma_32x32x16<F16>(qq, kf[nt][j], zero);
+          s[nt] = mfma_32x32x16<F16>(qq[j], kf[nt][j], zero);
         } else {
-          s[nt] = mfma_32x32x16<F16>(qq, kf[nt][j], s[nt]);
+          s[nt] = mfma_32x32x16<F16>(qq[j], kf[nt][j], s[nt]);
         }
       }
     }
   };
-  // p = exp2(c S - lse) summed over the block's rows; accumulator rows are 8 a + 4 h + (0..3)
-  auto valu_block = [&](auto mask_tag, const f32x16_t (&s)[2], int buf3, int mt) {
+  // p = exp2(c S - lse) summed over the block's rows
+  auto valu_block = [&](auto mask_tag, const f32x16_t (&s)[2], const f32x4_t (&ls)[4], int ring, int mt) {
     constexpr bool MASK = decltype(mask_tag)::value;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const f32x4_t ls = *(const f32x4_t*)&sm.lse[buf3][mt * 32 + 8 * a + 4 * h];
       int4 qp = {0, 0, 0, 0};
-      if constexpr (MASK) qp = *(const int4*)&sm.qpos[buf3][mt * 32 + 8 * a + 4 * h];
+      if constexpr (MASK) qp = *(const int4*)&sm.qpos[ring][mt * 32 + 8 * a + 4 * h];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[0]));
-        float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[1]));
-        float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[2]));
-        float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[3]));
+        float e0 = fast_exp2(fmaf(s[nt][4 * a + 0], p.c, -ls[a][0]));
+        float e1 = fast_exp2(fmaf(s[nt][4 * a + 1], p.c, -ls[a][1]));
+        float e2 = fast_exp2(fmaf(s[nt][4 * a + 2], p.c, -ls[a][2]));
+        float e3 = fast_exp2(fmaf(s[nt][4 * a + 3], p.c, -ls[a][3]));
         if constexpr (MASK) {
           e0 = tpk[nt] > qp.x ? 0.0f : e0;
           e1 = tpk[nt] > qp.y ? 0.0f : e1;
@@ -246,69 +304,100 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
       }
     }
   };
-  // one matrix instruction, its share of the LDS reads, then its share of the other block's
-  // vector work (6 or 10 instructions per matrix instruction, 2 of them transcendental)
+  // one matrix instruction, then its share of the other block's vector work (6 or 10 instructions per matrix
+  // instruction, 2 of them transcendental)
   auto interleave = [&](auto mask_tag) {
     constexpr bool MASK = decltype(mask_tag)::value;
-    // the first LDS reads go out ahead of the first matrix instruction, so that every operand has
-    // been on its way for several steps when its (in-order) consumer is reached
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
-    for (int i = 0; i < 2 * (D / 16); ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, MASK ? 8 * 16 / (2 * (D / 16)) : 4 * 16 / (2 * (D / 16)), 0);
-      __builtin_amdgcn_sched_group_barrier(0x400, 2 * 16 / (2 * (D / 16)), 0);
+    for (int a = 0; a < 4; ++a) {
+      if constexpr (MASK) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the positions of rows 8 a .. 8 a + 7
+#pragma unroll
+      for (int i = 0; i < (D / 16) / 2; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, MASK ? 8 * 16 / (2 * (D / 16)) : 4 * 16 / (2 * (D / 16)), 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 2 * 16 / (2 * (D / 16)), 0);
+      }
     }
   };
 
-  ld.fetch(st, tbase * BQ, tid);
-  ld.commit(st, sm, 0, 0, tid);
-  if (num_qt > 1) ld.fetch(st, (tbase + 1) * BQ, tid);
+  // Keeps a half step's work in that half: without a use here the optimiser moves the exponentials of several
+  // half steps below the matrix instructions of the next ones (out of their shadow, and every block's scores then
+  // need registers of their own).
+  auto pin = [&](f32x16_t (&s)[2]) {
+    asm volatile("" : "+v"(s[0]), "+v"(s[1]), "+v"(wacc[0]), "+v"(wacc[1]));
+  };
+  constexpr std::integral_constant<int, 0> I0{};
+  constexpr std::integral_constant<int, 1> I1{};
+  ld.issue(sm, 0, 0);
+  if (num_qt > 1) ld.issue(sm, 1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K fragments and the first tiles have arrived
+  ld.land(sm, tbase * BQ, 0);
+  if (num_qt > 1) ld.land(sm, (tbase + 1) * BQ, 1);
   __syncthreads();
   f32x16_t sa[2], sb[2];  // blocks 0 and 1 of the current tile
-  mfma_block(sa, 0, 0);
+  u32x4_t qq[D / 16];
+  load_q(qq, I0, I0);
+  mfma_block(sa, qq);
 
   // Software pipeline: the matrix work of one block runs under the vector work of the block before.
-  // Tile t + 1 is committed at the start of iteration t and first read after the barrier inside it.
-  for (int t = 0; t < num_qt; ++t) {
-    const int buf = t & 1, buf3 = t % 3;
-    const bool more = t + 1 < num_qt;
-    if (more) {
-      ld.commit(st, sm, buf ^ 1, (t + 1) % 3, tid);
-      if (t + 2 < num_qt) ld.fetch(st, (tbase + t + 2) * BQ, tid);
+  // Tile t + 2 is requested right behind the barrier of step t (the buffers of tile t are free from there on: its
+  // Q rows have been multiplied and its log-sum-exps are in registers), has the rest of that step and the first
+  // half of the next to arrive, and is published by the barrier of step t + 1.
+  auto step = [&](auto mask_tag, auto steady_tag, auto buf_tag, int t) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    constexpr int BUF = decltype(buf_tag)::value;
+    constexpr std::integral_constant<int, BUF ^ 1> NEXT{};
+    const int ring = t & 3;
+    const bool more = STEADY || t + 1 < num_qt;
+    f32x4_t ls[4];
+    load_q(qq, buf_tag, I1);
+    load_lse(ls, buf_tag, I0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_block(sb, qq);
+    valu_block(mask_tag, sa, ls, ring, 0);
+    interleave(mask_tag);
+    pin(sb);
+    __builtin_amdgcn_sched_barrier(0);
+    load_lse(ls, buf_tag, I1);  // into registers before the barrier that hands the buffer to tile t + 2
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile t + 1 has landed
+    if constexpr (!STEADY) {
+      if (more) ld.land(sm, (tbase + t + 1) * BQ, BUF ^ 1);
     }
-    // issue priority: lowest in the first half of a tile, highest on the way to the barrier, so that the
-    // four wavefronts of a workgroup wait less for each other (about 1 % on the kernel)
-    __builtin_amdgcn_s_setprio(0);
-    const bool need_mask = tpmax > p.input_pos + ((tbase + t) * BQ) / p.G;
-    if (need_mask) {
-      mfma_block(sb, buf, 1);
-      valu_block(std::true_type{}, sa, buf3, 0);
-      interleave(std::true_type{});
-    } else {
-      mfma_block(sb, buf, 1);
-      valu_block(std::false_type{}, sa, buf3, 0);
-      interleave(std::false_type{});
-    }
-    __builtin_amdgcn_s_setprio(3);
     __syncthreads();
-    __builtin_amdgcn_s_setprio(1);
-    if (more) {
-      if (need_mask) {
-        mfma_block(sa, buf ^ 1, 0);
-        valu_block(std::true_type{}, sb, buf3, 1);
-        interleave(std::true_type{});
-      } else {
-        mfma_block(sa, buf ^ 1, 0);
-        valu_block(std::false_type{}, sb, buf3, 1);
-        interleave(std::false_type{});
-      }
+    if constexpr (STEADY) {
+      ld.template issue_steady<BUF>(sm, (t + 2) & 3);
     } else {
-      if (need_mask) valu_block(std::true_type{}, sb, buf3, 1);
-      else valu_block(std::false_type{}, sb, buf3, 1);
+      if (t + 2 < num_qt) ld.issue(sm, BUF, (t + 2) & 3);
     }
+    if (more) {
+      load_q(qq, NEXT, I0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(sa, qq);
+      valu_block(mask_tag, sb, ls, ring, 1);
+      interleave(mask_tag);
+      pin(sa);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      valu_block(mask_tag, sb, ls, ring, 1);
+    }
+  };
+  constexpr std::true_type YES{};
+  constexpr std::false_type NO{};
+  int t = 0;
+  for (; t < t_masked; t += 2) {
+    step(YES, YES, I0, t);
+    step(YES, YES, I1, t + 1);
   }
+  for (; t < t_steady; t += 2) {
+    step(NO, YES, I0, t);
+    step(NO, YES, I1, t + 1);
+  }
+  // the last tiles (and all of them when G does not divide the tile height): masked whether they need it or not
+  for (; t + 1 < num_qt; t += 2) {
+    step(YES, NO, I0, t);
+    step(YES, NO, I1, t + 1);
+  }
+  if (t < num_qt) step(YES, NO, I0, t);
 
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
@@ -385,6 +474,13 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   // the query rows are split only if the caller's workspace holds the partial sums
   ScorePlan pl = score_plan(a);
   if (pl.splits > 1 && !(a.workspace && a.workspace_bytes >= score_sum_workspace(a) && ((uintptr_t)a.workspace & 15) == 0)) pl.splits = 1;
+  // the query rows are fetched at a uniform base plus a 32-bit byte offset per lane
+  {
+    const int64_t G = a.Hq / a.Hkv;
+    KVX_REQUIRE(a.q_stride_h >= 0 && a.q_stride_t >= 0 && ((G - 1) * a.q_stride_h + (int64_t)(a.q_len - 1) * a.q_stride_t + a.D) * 2 < (1ll << 32),
+                KVX_ERR_UNSUPPORTED, "kvx_score_sum: the query rows of one (batch, KV head) pair must span less than 4 GiB (strides %lld / %lld)",
+                (long long)a.q_stride_h, (long long)a.q_stride_t);
+  }
   ScoreParams p;
   p.part = pl.splits > 1 ? (float*)a.workspace : nullptr;
   p.tiles_per_z = pl.tiles_per_z;

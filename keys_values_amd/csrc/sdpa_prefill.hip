@@ -87,36 +87,6 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(lds_ptr_t p) {
   return __builtin_bit_cast(u32x2_t, t);
 }
 
-// 16 bytes per lane straight from global memory into LDS (global_load_lds_dwordx4): lane l lands at
-// lds_addr + 16 l, lds_addr uniform over the wavefront. Written as inline assembly so that the
-// compiler does not serialise later LDS reads of OTHER buffers behind the transfer; the kernel
-// waits for its transfers itself (s_waitcnt vmcnt(0)) before the barrier that publishes a tile.
-__device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(base)
-               : "memory", "m0");
-}
-// the same with the LDS address formed as lds_base + IMM in M0 by the one scalar instruction the
-// transfer needs anyway
-template <uint32_t IMM>
-__device__ __forceinline__ void dma16_at(const char* base, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_base), "v"(voff), "s"(base), "n"(IMM)
-               : "memory", "m0", "scc");
-}
-// same for 4 bytes per lane (global_load_lds_dword): lane l lands at lds_addr + 4 l
-__device__ __forceinline__ void dma4(const char* base, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(base)
-               : "memory", "m0");
-}
-__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
-  return (uint32_t)(uintptr_t)((const __attribute__((address_space(3))) char*)p);
-}
-
 // 8 codes (two dwords) -> 8 bf16 (four dwords)
 __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp, float scale) { return dequant_words(c0, c1, zp, scale); }
 
