@@ -103,15 +103,21 @@ def parse():
                          "table (keys_values_amd/longctx/gemm_table_gfx950.csv; switches PyTorch's TunableOp on for the process)")
     ap.add_argument("--tune-gemms", action="store_true",
                     help="longctx: let PyTorch's TunableOp pick the library GEMM kernels during the warm-up pass (adds about a minute)")
+    ap.add_argument("--operands", default="random", choices=["random", "zeros"],
+                    help="prefill: `zeros` runs the same launches on all-zero q, k, v (not the benchmark: a probe of how much of the "
+                         "duration is the clock following the operands; the line says so in `data`)")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "uint8", "uint4"],
                     help="cache storage for the prefill / decode workloads; uint8 = BASELINE.json configs[2]: codes + per-row "
                          "scale and zero point, dequantised inside the attention kernels; uint4 = the 4-bit store of the same quantiser")
     return ap.parse_args()
 
 
-def rope_inputs(torch, O, dev, T=32768, seed=1):
+def rope_inputs(torch, O, dev, T=32768, seed=1, zeros=False):
     B, Hq, Hkv, q_len, D = 1, 32, 8, 1024, 128
     input_pos = T - q_len
+    if zeros:  # the same launches on operands that toggle nothing: what the clock does without the data's share of the power
+        z = lambda *shape: torch.zeros(shape, dtype=torch.bfloat16)
+        return (B, Hq, Hkv, q_len, T, D, input_pos), z(B, Hq, q_len, D), z(B, Hkv, T, D), z(B, Hkv, T, D)
     gen = torch.Generator().manual_seed(seed)
     q = torch.randn(B, Hq, q_len, D, generator=gen)
     k = torch.randn(B, Hkv, T, D, generator=gen)
@@ -129,7 +135,7 @@ def bench_prefill(args, torch, dev):
     lib = _lib.load()
     u8 = args.kv != "bf16"   # a quantised store: codes + row state
     u4 = args.kv == "uint4"
-    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev, 65536 if u8 else 32768, 2 if u8 else 1)
+    (B, Hq, Hkv, q_len, T, D, input_pos), q_c, k_c, v_c = rope_inputs(torch, O, dev, 65536 if u8 else 32768, 2 if u8 else 1, args.operands == "zeros")
     scale = D ** -0.5
     q, k, v = q_c.to(dev), k_c.to(dev), v_c.to(dev)
     quant = None
@@ -286,7 +292,7 @@ def bench_prefill(args, torch, dev):
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic" if args.operands == "random" else "synthetic, ALL-ZERO operands (clock probe, not the benchmark)",
         "config": {
             "workload": (f"BASELINE.json configs[2]: attention + score-sum over the {args.kv} cache (dequantised in the kernels), B1 Hq32 Hkv8 D128 T65536 q1024, seed 2"
                          if u8 else

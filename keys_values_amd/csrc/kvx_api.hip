@@ -169,7 +169,7 @@ int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
   if (rc != KVX_OK) return rc;
   KVX_REQUIRE(a->q_len == 1, KVX_ERR_INVALID, "kvx_sdpa_decode: q_len must be 1, got %d", a->q_len);
   const int G = a->Hq / a->Hkv;
-  KVX_REQUIRE(G >= 1 && G <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in 1 .. 8", G);
+  KVX_REQUIRE(G >= 1 && G <= 16 && (G <= 8 || a->D <= 128), KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: group size %d not in 1 .. 16 (1 .. 8 with head size 256)", G);
   KVX_REQUIRE(aligned16(a->workspace), KVX_ERR_WORKSPACE, "kvx_sdpa_decode: workspace must be 16-byte aligned");
   return launch_sdpa_decode(*a, nullptr, (hipStream_t)stream);
 }
@@ -316,7 +316,7 @@ int kvx_sdpa_decode_h2o(const kvx_sdpa_args* a, const kvx_h2o_args* h, void* str
   if (rc != KVX_OK) return rc;
   KVX_REQUIRE(a->q_len == 1, KVX_ERR_INVALID, "kvx_sdpa_decode_h2o: q_len must be 1, got %d", a->q_len);
   const int G = a->Hq / a->Hkv;
-  KVX_REQUIRE(G >= 1 && G <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode_h2o: group size %d not in 1 .. 8", G);
+  KVX_REQUIRE(G >= 1 && G <= 16 && (G <= 8 || a->D <= 128), KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode_h2o: group size %d not in 1 .. 16 (1 .. 8 with head size 256)", G);
   KVX_REQUIRE(!h->v_norm && !h->q_errors, KVX_ERR_UNSUPPORTED,
               "kvx_sdpa_decode_h2o: v_norm / q_errors policies take kvx_sdpa_decode + kvx_h2o_update_select");
   KVX_REQUIRE(h->k == 1 && h->kv_len == a->kv_len && h->B == a->B && h->Hkv == a->Hkv, KVX_ERR_INVALID,

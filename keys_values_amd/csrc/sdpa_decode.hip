@@ -24,6 +24,9 @@
 // outputs, the others do the weights work of the splits that took the scratch route, and the one that finishes
 // last publishes the chosen slots. K and V are touched once: they are loaded non-temporally. No float atomics
 // anywhere.
+// Quantised stores, and plain rows with 8 to 16 query heads per KV head, take a second form of the split kernel
+// (decode_mfma_kernel, below) that does both products on the matrix cores: with codes to dequantise, or with that
+// many dot products per loaded value, the form above is bound by its vector arithmetic, not by HBM.
 #include "kvx_common.h"
 #include <stdlib.h>
 
@@ -56,6 +59,7 @@ struct DecodeParams {
   uint32_t* split_done;      // (B, Hkv, S): 1 where the split kernel itself turned its logits into weights
   uint32_t* tail_count;      // fused H2O form: workgroups of the tail kernel's second kind that have finished
   uint32_t* scratch_splits;  // caller's counter of the splits whose logits went through the scratch, or NULL
+  int32_t qs_vec;            // quantiser state arrays are 16-byte aligned with strides that keep them so (vector loads of 4 keys)
   int32_t resident;          // the logits of a split stay in LDS
   int32_t spin_limit;        // polls of row_count before a workgroup gives up and sends its logits out
   int32_t poll_sleep;        // pause between two polls, in units of 512 cycles
@@ -91,7 +95,9 @@ __device__ __forceinline__ float row_group_sum(float x) {
 
 // Logits a workgroup holds in LDS: 64 KB where the merge buffer beside them is small enough for two workgroups
 // per compute unit (what the registers allow), else 32 KB.
-constexpr int logit_floats(int G, int D) { return G * D <= 512 ? 16384 : 8192; }
+// Two workgroups per compute unit share 160 KB of LDS: the logits take what the merge buffer (4 G D floats) leaves of
+// 80 KB, in whole pairs of steps of the widest kernel (256 keys).
+constexpr int logit_floats(int G, int D) { return G * D <= 512 ? 16384 : (G * D <= 1024 ? (G == 16 ? 12288 : 14336) : 8192); }
 constexpr int kCountStride = 64;  // a row's arrival counter has 256 bytes to itself: the polls of different rows go to different channels
 constexpr float kNegBig = -1.0e30f;  // running maximum before the first key (finite: no inf - inf)
 constexpr float kRescaleSlack = 8.0f;  // the running maximum moves only when a logit exceeds it by this
@@ -126,6 +132,124 @@ __device__ __forceinline__ float row_lse(const float* part_ml, int num_splits, i
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) L += __shfl_xor(L, off, 64);
   return Mw + fast_log2(L);
+}
+
+// The logits gathered in LDS leave as one contiguous burst (keys past the end of a chunk of CHUNK keys are -inf).
+template <int G, int LGK, int CHUNK>
+__device__ __forceinline__ void flush_logits(const float* lgbuf, float* lgrow, int lg_base, int k_end, int tid) {
+  const int nkeys = min(LGK, (k_end - lg_base + CHUNK - 1) / CHUNK * CHUNK);
+  f32x4_t* dst = (f32x4_t*)(lgrow + (int64_t)lg_base * G);
+  for (int j = tid; j < nkeys * G / 4; j += NTHREADS) dst[j] = ((const f32x4_t*)lgbuf)[j];
+}
+
+// What a split does once its wavefronts have left their partial results in LDS (red: unnormalised outputs, rml:
+// maximum and sum, per wavefront and head): combine them into the split's partial, and, in the resident form, wait
+// for the row's other splits and turn this split's logits (lgbuf, [key][head]) into weights.
+template <int D, int G, int LGK, int CHUNK>
+__device__ __forceinline__ void finish_split(const DecodeParams& p, const kvx_h2o_args& hh, const int h2o, const float* lgbuf,
+                                             const float (&red)[WAVES][G][D], const float (&rml)[WAVES][G][2], float* lgrow,
+                                             const int lg_base, const int k_begin, const int k_end) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  __syncthreads();
+  for (int i = tid; i < G * D; i += NTHREADS) {
+    const int g = i / D, d = i % D;
+    if (g >= p.Gr) continue;
+    float M = rml[0][g][0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, rml[w][g][0]);
+    float x = 0.0f, l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float sc = fast_exp2(rml[w][g][0] - M);
+      x += red[w][g][d] * sc;
+      l += rml[w][g][1] * sc;
+    }
+    const int64_t o = ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits + split;
+    p.part_o[o * D + d] = x;
+    if (d == 0) {
+      // read by the row's other workgroups while this kernel runs: a device-coherent store
+      const unsigned long long mlbits = ((unsigned long long)__float_as_uint(l) << 32) | __float_as_uint(M);
+      __hip_atomic_store((unsigned long long*)(p.part_ml + o * 2), mlbits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (!lgrow || !p.resident) return;
+
+  // ---- the row's log-sum-exp, and this split's logits into weights, without leaving the chip --------
+  __shared__ float lse_sh[G];
+  __shared__ int row_ready;
+  __shared__ unsigned long long wbest[WAVES];
+  const int row = b * p.Hkv + kvh;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial above has reached device-coherent memory
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t* cnt = p.row_count + row * kCountStride;
+    __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int ok = 0;
+    for (int spin = 0; spin < p.spin_limit; ++spin) {  // bounded: a workgroup that gives up takes the scratch route
+      if (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)p.num_splits) {
+        ok = 1;
+        break;
+      }
+      for (int z = 0; z < p.poll_sleep; ++z) __builtin_amdgcn_s_sleep(8);
+    }
+    row_ready = ok;
+  }
+  __syncthreads();
+  if (!row_ready) {
+    flush_logits<G, LGK, CHUNK>(lgbuf, lgrow, lg_base, k_end, tid);
+    if (tid == 0) {
+      p.split_done[(int64_t)row * p.num_splits + split] = 0u;
+      if (p.scratch_splits) atomicAdd(p.scratch_splits, 1u);
+    }
+    return;
+  }
+  for (int g = wave; g < G; g += WAVES) {  // a wavefront per head: lane s takes splits s, s + 64, ...
+    float lse = INFINITY;  // dummy heads: exp2(x - inf) = 0
+    if (g < p.Gr) lse = row_lse<true>(p.part_ml + ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits * 2, p.num_splits, lane);
+    if (lane == 0) lse_sh[g] = lse;
+  }
+  __syncthreads();
+  float lse[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) lse[g] = lse_sh[g];
+  float* wr = p.w ? p.w + (int64_t)row * p.kv_len : nullptr;
+  float* sc = h2o ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
+  const int32_t* tpr = (h2o && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
+  const float inv_g = 1.0f / (float)p.Gr;
+  unsigned long long mine = ~0ull;
+  for (int k = k_begin + tid; k < k_end; k += NTHREADS) {
+    const float* lg = lgbuf + (k - k_begin) * G;
+    float acc = 0.0f;
+#pragma unroll
+    for (int g = 0; g < G; ++g) acc += fast_exp2(lg[g] - lse[g]);
+    acc *= inv_g;
+    if (wr) wr[k] = acc;
+    if (h2o) {
+      float val = sc[k] + acc;
+      sc[k] = val;
+      if (k < hh.limit) {
+        if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
+        const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
+        mine = key < mine ? key : mine;
+      }
+    }
+  }
+  if (h2o) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const unsigned long long o = __shfl_xor(mine, off, 64);
+      mine = o < mine ? o : mine;
+    }
+    if (lane == 0) wbest[wave] = mine;
+    __syncthreads();
+    if (tid == 0) {
+      unsigned long long mn = wbest[0];
+      for (int i = 1; i < WAVES; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
+      if (mn != ~0ull) atomicMin(p.best + row, mn);
+    }
+  }
+  if (tid == 0) p.split_done[(int64_t)row * p.num_splits + split] = 1u;
 }
 
 template <int D, int G, int KV>
@@ -301,13 +425,6 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     }
   };
 
-  // the gathered logits leave as one contiguous burst (keys past the end of a chunk are -inf)
-  auto flush_logits = [&]() {
-    const int nkeys = min(LGK, (k_end - lg_base + CH - 1) / CH * CH);
-    f32x4_t* dst = (f32x4_t*)(lgrow + (int64_t)lg_base * G);
-    for (int j = tid; j < nkeys * G / 4; j += NTHREADS) dst[j] = ((const f32x4_t*)lgbuf)[j];
-  };
-
   // Two steps in flight per wavefront: the loads of step i + 1 are issued before step i is consumed.
   const int nsteps = (k_end - k_begin + CH * WAVES - 1) / (CH * WAVES);
   const int stride = CH * WAVES;
@@ -328,7 +445,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     chunk += 2 * stride;
     if (lgrow && !p.resident && ((i + 2) % FLUSH_STEPS == 0 || i + 2 >= nsteps)) {
       __syncthreads();
-      flush_logits();
+      flush_logits<G, LGK, CH>(lgbuf, lgrow, lg_base, k_end, tid);
       lg_base += LGK;
       __syncthreads();
     }
@@ -356,105 +473,327 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
       rml[wave][g][1] = l;
     }
   }
-  __syncthreads();
-  for (int i = tid; i < G * D; i += NTHREADS) {
-    const int g = i / D, d = i % D;
-    if (g >= p.Gr) continue;
-    float M = rml[0][g][0];
-#pragma unroll
-    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, rml[w][g][0]);
-    float x = 0.0f, l = 0.0f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      const float sc = fast_exp2(rml[w][g][0] - M);
-      x += red[w][g][d] * sc;
-      l += rml[w][g][1] * sc;
-    }
-    const int64_t o = ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits + split;
-    p.part_o[o * D + d] = x;
-    if (d == 0) {
-      // read by the row's other workgroups while this kernel runs: a device-coherent store
-      const unsigned long long mlbits = ((unsigned long long)__float_as_uint(l) << 32) | __float_as_uint(M);
-      __hip_atomic_store((unsigned long long*)(p.part_ml + o * 2), mlbits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  if (!lgrow || !p.resident) return;
+  finish_split<D, G, LGK, CH>(p, hh, h2o, lgbuf, red, rml, lgrow, lg_base, k_begin, k_end);
+}
 
-  // ---- the row's log-sum-exp, and this split's logits into weights, without leaving the chip --------
-  __shared__ float lse_sh[G];
-  __shared__ int row_ready;
-  __shared__ unsigned long long wbest[WAVES];
-  const int row = b * p.Hkv + kvh;
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial above has reached device-coherent memory
-  __syncthreads();
-  if (tid == 0) {
-    uint32_t* cnt = p.row_count + row * kCountStride;
-    __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    int ok = 0;
-    for (int spin = 0; spin < p.spin_limit; ++spin) {  // bounded: a workgroup that gives up takes the scratch route
-      if (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)p.num_splits) {
-        ok = 1;
-        break;
+// ---- the same split with both products on the matrix cores --------------------------------------------------------
+//
+// For quantised stores and for more than four query heads per KV head the kernel above is bound by its vector
+// arithmetic (G dot products per loaded pair of values on top of the dequantisation), not by HBM. Here the G heads are
+// padded to the 16 columns of v_mfma_f32_16x16x32: S^T = K Q^T per 16 keys (the lane that holds key m of the tile
+// loads 8 consecutive d of that row per matrix instruction: the row as it lies in memory is the A operand), then
+// O^T += V^T P^T per 32 keys. The accumulator layout of S^T (lane = (head, keys 4 kg .. 4 kg + 3)) becomes the B
+// operand of the second product without any exchange once the 32 keys of a block are taken in the order (tile 0:
+// 4 kg .. 4 kg + 3, tile 1: 4 kg .. 4 kg + 3) per lane group kg; V^T is gathered to match: a lane loads, from each of
+// its 8 keys, the D / 16 values of its d rows and regroups them (one byte permute per pair of bf16 values; for codes
+// the regrouping is part of the dequantisation). What is left for the vector ALU is the dequantisation (3.5
+// instructions per element, as the reference rounds) or half an instruction per V element, and the softmax of 16
+// head columns per key. The running maximum is one per head (the four lane groups of a head column agree on it), it
+// moves lazily as above. Everything after the key loop is shared with the kernel above.
+template <bool F16>
+__device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c) {
+  if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// bf16( (float)((int)code - zp) * scale ) for two codes with their own row state (two keys)
+__device__ __forceinline__ uint32_t dequant_pair2(uint32_t c0, int32_t zp0, float sc0, uint32_t c1, int32_t zp1, float sc1) {
+  return pack_bf16((float)((int32_t)c0 - zp0) * sc0, (float)((int32_t)c1 - zp1) * sc1);
+}
+
+template <int D, int G, int KV>
+__global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
+  constexpr bool F16 = KV == KVX_KV_F16;
+  constexpr bool U8 = !kv_is_plain(KV);  // codes + row state (8-bit or 4-bit store)
+  constexpr bool U4 = KV == KVX_KV_U4;
+  constexpr int KJ = D / 32;   // matrix instructions of the first product per 16-key tile
+  constexpr int DPL = D / 16;  // d rows per lane = matrix instructions of the second product per 32-key block
+  constexpr int CH = 32;       // keys per wavefront and step
+  constexpr int KR = U4 ? 1 : (U8 ? D / 64 : KJ);                          // 16-byte loads per key of K
+  constexpr int VW = U4 ? 1 : (U8 ? (DPL + 3) / 4 : DPL / 2);              // dwords per key of V
+  constexpr int LGK = logit_floats(G, D) / G;
+  __shared__ __align__(16) float lgbuf[LGK * G];  // [key][head]
+  __shared__ float red[WAVES][G][D];
+  __shared__ float rml[WAVES][G][2];
+  static_assert(D == 64 || D == 128, "head sizes 64 and 128");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int m = lane & 15, kg = lane >> 4;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int k_begin = split * p.keys_per_split;
+  const int k_end = min(k_begin + p.keys_per_split, p.kv_len);
+
+  // first d of the 8 this lane group supplies to matrix instruction e of the first product
+  auto kslice = [&](int e) -> int {
+    if constexpr (!U8) return 8 * (kg + 4 * e);
+    else if constexpr (U4 && D == 64) return 8 * kg + 32 * e;
+    else return 16 * kg + 8 * (e & 1) + 64 * (e >> 1);
+  };
+  // d of row `mrow` of matrix instruction t of the second product
+  auto dmap = [&](int t, int mrow) -> int {
+    if constexpr (U4) return t < DPL / 2 ? (DPL / 2) * mrow + t : D / 2 + (DPL / 2) * mrow + (t - DPL / 2);
+    else return DPL * mrow + t;
+  };
+
+  u32x4_t qb[KJ];  // B operands of the first product: head m (zero beyond the group), d slice of lane group kg
+#pragma unroll
+  for (int e = 0; e < KJ; ++e) {
+    qb[e] = u32x4_t{0u, 0u, 0u, 0u};
+    if (m < p.Gr) qb[e] = *(const u32x4_t*)(p.q + b * p.q_sb + (int64_t)(kvh * p.Gr + m) * p.q_sh + kslice(e));
+  }
+  constexpr int ES = U8 ? 1 : 2;
+  const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
+  const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * ES;
+  const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES;
+  const uint32_t k_lane = U4 ? (D == 128 ? 16 * kg : 8 * kg) : 16 * kg;    // + 64 r for the r-th load of the row
+  const uint32_t v_lane = (uint32_t)m * (U4 ? DPL / 2 : (U8 ? DPL : 2 * DPL));
+  const int64_t qs_off = b * p.qs_sb + kvh * p.qs_sh;
+  const char* ksb = (const char*)(p.k_scale + qs_off);
+  const char* kzb = (const char*)(p.k_zp + qs_off);
+  const char* vsb = (const char*)(p.v_scale + qs_off);
+  const char* vzb = (const char*)(p.v_zp + qs_off);
+  float* lgrow = p.logits ? p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G : nullptr;
+  int lg_base = k_begin;
+
+  f32x4_t acc[DPL];
+#pragma unroll
+  for (int t = 0; t < DPL; ++t) acc[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  float m_run = kNegBig, l_run = 0.0f;
+
+  struct Rows {
+    u32x4_t k[2][KR];
+    float ks[2];
+    int32_t kz[2];
+    uint32_t v[8][VW];
+    float vs[8];
+    int32_t vz[8];
+  };
+  // Byte offsets of this lane's rows in the block at `chunk0`: K rows chunk0 + m and chunk0 + 16 + m, V rows
+  // chunk0 + 4 kg (+ 0..3, + 16..19). A full block addresses them from two per-lane offsets that advance with the
+  // block and multiples of the row stride; a block that reaches past the end clamps every key to the last valid row
+  // (its logits become -inf below).
+  const uint32_t k16 = 16u * k_rowb, v16 = 16u * v_rowb;
+  auto load_k = [&](Rows& r, int gi, uint32_t off, int key) {
+    const uint8_t* row = kbase + off;
+#pragma unroll
+    for (int x = 0; x < KR; ++x) {
+      if constexpr (U4 && D == 64) {
+        const u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)row);
+        r.k[gi][x] = u32x4_t{c[0], c[1], 0u, 0u};
+      } else {
+        r.k[gi][x] = __builtin_nontemporal_load((const u32x4_t*)(row + 64 * x));
       }
-      for (int z = 0; z < p.poll_sleep; ++z) __builtin_amdgcn_s_sleep(8);
     }
-    row_ready = ok;
-  }
-  __syncthreads();
-  if (!row_ready) {
-    flush_logits();
-    if (tid == 0) {
-      p.split_done[(int64_t)row * p.num_splits + split] = 0u;
-      if (p.scratch_splits) atomicAdd(p.scratch_splits, 1u);
+    if constexpr (U8) {  // uniform base + 32-bit offset
+      r.ks[gi] = *(const float*)(ksb + (uint32_t)key * 4u);
+      r.kz[gi] = *(const int32_t*)(kzb + (uint32_t)key * 4u);
     }
-    return;
-  }
-  for (int g = wave; g < G; g += WAVES) {  // a wavefront per head: lane s takes splits s, s + 64, ...
-    float lse = INFINITY;  // dummy heads: exp2(x - inf) = 0
-    if (g < p.Gr) lse = row_lse<true>(p.part_ml + ((int64_t)b * p.Hq + kvh * p.Gr + g) * p.num_splits * 2, p.num_splits, lane);
-    if (lane == 0) lse_sh[g] = lse;
-  }
-  __syncthreads();
-  float lse[G];
+  };
+  auto load_v = [&](Rows& r, int j, uint32_t off) {
+    const uint8_t* row = vbase + off;
+    if constexpr (!U8) {
+      if constexpr (D == 128) {
+        const u32x4_t x = __builtin_nontemporal_load((const u32x4_t*)row);
+        r.v[j][0] = x[0]; r.v[j][1] = x[1]; r.v[j][2] = x[2]; r.v[j][3] = x[3];
+      } else {
+        const u32x2_t x = __builtin_nontemporal_load((const u32x2_t*)row);
+        r.v[j][0] = x[0]; r.v[j][1] = x[1];
+      }
+    } else if constexpr (!U4) {
+      if constexpr (D == 128) {
+        const u32x2_t x = __builtin_nontemporal_load((const u32x2_t*)row);
+        r.v[j][0] = x[0]; r.v[j][1] = x[1];
+      } else {
+        r.v[j][0] = __builtin_nontemporal_load((const uint32_t*)row);
+      }
+    } else {
+      if constexpr (D == 128) r.v[j][0] = __builtin_nontemporal_load((const uint32_t*)row);
+      else r.v[j][0] = (uint32_t)__builtin_nontemporal_load((const uint16_t*)row);
+    }
+  };
+  auto issue = [&](Rows& r, int chunk0) {
+    if (chunk0 + CH <= k_end) {
+      const uint32_t ko = (uint32_t)(chunk0 + m) * k_rowb + k_lane;
+      load_k(r, 0, ko, chunk0 + m);
+      load_k(r, 1, ko + k16, chunk0 + 16 + m);
+      const int q0 = chunk0 + 4 * kg;
+      if constexpr (U8) {
+        if (p.qs_vec) {  // the four keys of a tile this lane group owns are neighbours: one 16-byte load each
 #pragma unroll
-  for (int g = 0; g < G; ++g) lse[g] = lse_sh[g];
-  float* wr = p.w ? p.w + (int64_t)row * p.kv_len : nullptr;
-  float* sc = h2o ? hh.scores + b * hh.sc_stride_b + kvh * hh.sc_stride_h : nullptr;
-  const int32_t* tpr = (h2o && hh.token_pos) ? hh.token_pos + b * hh.tp_stride_b + kvh * hh.tp_stride_h : nullptr;
-  const float inv_g = 1.0f / (float)p.Gr;
-  unsigned long long mine = ~0ull;
-  for (int k = k_begin + tid; k < k_end; k += NTHREADS) {
-    const float* lg = lgbuf + (k - k_begin) * G;
-    float acc = 0.0f;
+          for (int gi = 0; gi < 2; ++gi) {
+            const f32x4_t sc = *(const f32x4_t*)(vsb + (uint32_t)(q0 + 16 * gi) * 4u);
+            const int4 zp = *(const int4*)(vzb + (uint32_t)(q0 + 16 * gi) * 4u);
+            r.vs[4 * gi] = sc[0]; r.vs[4 * gi + 1] = sc[1]; r.vs[4 * gi + 2] = sc[2]; r.vs[4 * gi + 3] = sc[3];
+            r.vz[4 * gi] = zp.x; r.vz[4 * gi + 1] = zp.y; r.vz[4 * gi + 2] = zp.z; r.vz[4 * gi + 3] = zp.w;
+          }
+        } else {
 #pragma unroll
-    for (int g = 0; g < G; ++g) acc += fast_exp2(lg[g] - lse[g]);
-    acc *= inv_g;
-    if (wr) wr[k] = acc;
-    if (h2o) {
-      float val = sc[k] + acc;
-      sc[k] = val;
-      if (k < hh.limit) {
-        if (hh.normalize) val = val / (float)(hh.input_pos - max(tpr[k], hh.prefill_len - 1));
-        const unsigned long long key = ((unsigned long long)ordered_bits(val) << 32) | (unsigned)k;
-        mine = key < mine ? key : mine;
+          for (int j = 0; j < 8; ++j) {
+            r.vs[j] = *(const float*)(vsb + (uint32_t)(q0 + 16 * (j >> 2) + (j & 3)) * 4u);
+            r.vz[j] = *(const int32_t*)(vzb + (uint32_t)(q0 + 16 * (j >> 2) + (j & 3)) * 4u);
+          }
+        }
+      }
+      const uint32_t vo = (uint32_t)q0 * v_rowb + v_lane;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) load_v(r, j, vo + (uint32_t)(j & 3) * v_rowb + (j >> 2) * v16);
+    } else {
+#pragma unroll
+      for (int gi = 0; gi < 2; ++gi) {
+        const int key = min(chunk0 + 16 * gi + m, k_end - 1);
+        load_k(r, gi, (uint32_t)key * k_rowb + k_lane, key);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = min(chunk0 + 16 * (j >> 2) + 4 * kg + (j & 3), k_end - 1);
+        if constexpr (U8) {
+          r.vs[j] = *(const float*)(vsb + (uint32_t)key * 4u);
+          r.vz[j] = *(const int32_t*)(vzb + (uint32_t)key * 4u);
+        }
+        load_v(r, j, (uint32_t)key * v_rowb + v_lane);
       }
     }
-  }
-  if (h2o) {
+  };
+  // A operand e of the first product for tile gi
+  auto k_operand = [&](const Rows& r, int gi, int e) -> u32x4_t {
+    if constexpr (!U8) {
+      return r.k[gi][e];
+    } else if constexpr (!U4) {
+      const u32x4_t w = r.k[gi][e >> 1];
+      return (e & 1) ? dequant_words(w[2], w[3], r.kz[gi], r.ks[gi]) : dequant_words(w[0], w[1], r.kz[gi], r.ks[gi]);
+    } else {
+      const u32x4_t w = r.k[gi][0];
+      u32x2_t bytes;
+      int shift;
+      if constexpr (D == 128) {
+        bytes = (e & 1) ? u32x2_t{w[2], w[3]} : u32x2_t{w[0], w[1]};
+        shift = (e >> 1) ? 0 : 4;
+      } else {
+        bytes = u32x2_t{w[0], w[1]};
+        shift = e ? 0 : 4;
+      }
+      const u32x2_t c = u4_codes(bytes, shift);
+      return dequant_words(c[0], c[1], r.kz[gi], r.ks[gi]);
+    }
+  };
+  // A operand t of the second product: value t of each of this lane's 8 keys, in key order
+  auto v_operand = [&](const Rows& r, int t) -> u32x4_t {
+    u32x4_t a;
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const unsigned long long o = __shfl_xor(mine, off, 64);
-      mine = o < mine ? o : mine;
+    for (int jj = 0; jj < 4; ++jj) {
+      const int j0 = 2 * jj, j1 = 2 * jj + 1;
+      if constexpr (!U8) {
+        a[jj] = __builtin_amdgcn_perm(r.v[j1][t >> 1], r.v[j0][t >> 1], (t & 1) ? 0x07060302u : 0x05040100u);
+      } else {
+        uint32_t c0, c1;
+        if constexpr (!U4) {
+          c0 = (r.v[j0][t >> 2] >> (8 * (t & 3))) & 0xffu;
+          c1 = (r.v[j1][t >> 2] >> (8 * (t & 3))) & 0xffu;
+        } else {
+          const int sh = t < DPL / 2 ? 8 * t + 4 : 8 * (t - DPL / 2);
+          c0 = (r.v[j0][0] >> sh) & 0xfu;
+          c1 = (r.v[j1][0] >> sh) & 0xfu;
+        }
+        a[jj] = dequant_pair2(c0, r.vz[j0], r.vs[j0], c1, r.vz[j1], r.vs[j1]);
+      }
     }
-    if (lane == 0) wbest[wave] = mine;
-    __syncthreads();
-    if (tid == 0) {
-      unsigned long long mn = wbest[0];
-      for (int i = 1; i < WAVES; ++i) mn = wbest[i] < mn ? wbest[i] : mn;
-      if (mn != ~0ull) atomicMin(p.best + row, mn);
+    return a;
+  };
+  auto consume = [&](Rows& r, int chunk0) {
+    f32x4_t s[2];
+#pragma unroll
+    for (int gi = 0; gi < 2; ++gi) {
+      s[gi] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int e = 0; e < KJ; ++e) s[gi] = mfma_16x16x32<F16>(k_operand(r, gi, e), qb[e], s[gi]);
+    }
+    // this lane: head m, keys chunk0 + 16 gi + 4 kg + i (log2 units)
+    float sv[8];
+#pragma unroll
+    for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sv[4 * gi + i] = s[gi][i] * p.c;
+    if (chunk0 + CH > k_end) {
+#pragma unroll
+      for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (chunk0 + 16 * gi + 4 * kg + i >= k_end) sv[4 * gi + i] = -INFINITY;
+    }
+    if (lgrow && m < G && chunk0 < k_end) {
+      float* dst = lgbuf + (chunk0 - lg_base + 4 * kg) * G + m;
+#pragma unroll
+      for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[(16 * gi + i) * G] = sv[4 * gi + i];
+    }
+    float mx = sv[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
+    if (__any(mx > m_run + kRescaleSlack)) {
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));  // the head's maximum over the four lane groups
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m_run, mx);
+      const float al = fast_exp2(m_run - mn);
+      m_run = mn;
+      l_run *= al;
+#pragma unroll
+      for (int t = 0; t < DPL; ++t) acc[t] *= al;
+    }
+    float pv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      pv[i] = fast_exp2(sv[i] - m_run);
+      l_run += pv[i];
+    }
+    const u32x4_t pb = {pack_pair<F16>(pv[0], pv[1]), pack_pair<F16>(pv[2], pv[3]), pack_pair<F16>(pv[4], pv[5]), pack_pair<F16>(pv[6], pv[7])};
+#pragma unroll
+    for (int t = 0; t < DPL; ++t) acc[t] = mfma_16x16x32<F16>(v_operand(r, t), pb, acc[t]);
+  };
+
+  // Two steps in flight per wavefront: the loads of step i + 1 are issued before step i is consumed.
+  const int nsteps = (k_end - k_begin + CH * WAVES - 1) / (CH * WAVES);
+  const int stride = CH * WAVES;
+  int chunk = k_begin + wave * CH;
+  constexpr int FLUSH_STEPS = LGK / (CH * WAVES);
+  static_assert(LGK % (CH * WAVES) == 0 && FLUSH_STEPS >= 2 && FLUSH_STEPS % 2 == 0, "the loop below advances two steps at a time");
+  Rows ra, rb;
+  issue(ra, chunk);
+  for (int i = 0; i < nsteps; i += 2) {
+    issue(rb, chunk + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(ra, chunk);
+    __builtin_amdgcn_sched_barrier(0);  // the loads below reuse the registers consumed above
+    issue(ra, chunk + 2 * stride);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(rb, chunk + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    chunk += 2 * stride;
+    if (lgrow && !p.resident && ((i + 2) % FLUSH_STEPS == 0 || i + 2 >= nsteps)) {
+      __syncthreads();
+      flush_logits<G, LGK, CH>(lgbuf, lgrow, lg_base, k_end, tid);
+      lg_base += LGK;
+      __syncthreads();
     }
   }
-  if (tid == 0) p.split_done[(int64_t)row * p.num_splits + split] = 1u;
+
+  // ---- this wavefront's partial: sums over the four lane groups of a head, outputs by d ----------------------------
+  float l = l_run;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (m < G) {
+#pragma unroll
+    for (int t = 0; t < DPL; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][m][dmap(t, 4 * kg + i)] = acc[t][i];
+    if (kg == 0) {
+      rml[wave][m][0] = m_run;
+      rml[wave][m][1] = l;
+    }
+  }
+  finish_split<D, G, LGK, CH>(p, hh, h2o, lgbuf, red, rml, lgrow, lg_base, k_begin, k_end);
 }
 
 // Before the split kernel: no split of a row has arrived, no row has a lowest-score slot yet.
@@ -673,7 +1012,7 @@ Tuning& tuning() {
 Plan make_plan(const kvx_sdpa_args& a, bool fused_h2o) {
   Plan pl;
   const int gr = a.Hq / a.Hkv;
-  pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : 8));
+  pl.G = gr <= 1 ? 1 : (gr <= 2 ? 2 : (gr <= 4 ? 4 : (gr <= 8 ? 8 : 16)));
   // One full round of workgroups (two per compute unit, what the registers allow) over the whole grid:
   // rows * kv_len / (2 CUs) keys per split, at least 256; with weights at most what the LDS holds of a split's
   // logits (a split that waits for its row holds its place, so the device then runs several rounds) and, LDS
@@ -749,12 +1088,19 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
   }
   const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
   const int h2o = hh != nullptr;
+  // quantised stores and groups of 8 heads or more: both products on the matrix cores
   if constexpr (D <= 128) {
-    if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
-    else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (G >= 8 && kv == KVX_KV_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (G >= 8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
   }
-  if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
-  else if (kv == KVX_KV_BF16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+  if constexpr (G <= 8) {
+    if (kv_is_plain(kv) && (D > 128 || G < 8)) {
+      if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+      else hipLaunchKernelGGL((decode_split_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    }
+  }
   KVX_HIP(hipGetLastError());
   return kv == KVX_KV_F16 ? launch_tail<D, true, G>(p, hh, st) : launch_tail<D, false, G>(p, hh, st);
 }
@@ -766,8 +1112,11 @@ int launch_d(const DecodeParams& p, int G, int kv, const kvx_h2o_args* hh, hipSt
     case 2: return launch_dg<D, 2>(p, kv, hh, st);
     case 4: return launch_dg<D, 4>(p, kv, hh, st);
     case 8: return launch_dg<D, 8>(p, kv, hh, st);
+    case 16:
+      if constexpr (D <= 128) return launch_dg<D, 16>(p, kv, hh, st);
+      break;
   }
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: %d query heads per KV head (at most 16; at most 8 with head size 256)", p.Gr);
 }
 
 }  // namespace
@@ -811,7 +1160,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.poll_sleep = tuning().poll_sleep.load();
   p.B = a.B; p.Hq = a.Hq; p.Hkv = a.Hkv; p.kv_len = a.kv_len; p.Tpad = pl.Tpad;
   p.Gr = a.Hq / a.Hkv;
-  KVX_REQUIRE(p.Gr <= 8, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 8 query heads per KV head (%d)", p.Gr);
+  KVX_REQUIRE(p.Gr <= 16, KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: more than 16 query heads per KV head (%d)", p.Gr);
+  p.qs_vec = (((uintptr_t)a.k_scale | (uintptr_t)a.k_zp | (uintptr_t)a.v_scale | (uintptr_t)a.v_zp) & 15) == 0 && a.qs_stride_b % 4 == 0 && a.qs_stride_h % 4 == 0;
   p.num_splits = pl.num_splits; p.keys_per_split = pl.keys_per_split;
   p.c = a.sm_scale * kLog2e;
   p.q_sb = a.q_stride_b; p.q_sh = a.q_stride_h;

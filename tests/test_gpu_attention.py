@@ -196,6 +196,9 @@ DECODE_CASES = [
     (1, 28, 4, 3000, 128, 2),
     (1, 5, 1, 513, 64, 1),
     (2, 12, 2, 260, 128, 0),
+    (1, 32, 2, 3000, 128, 0),      # 16 and 12 heads per KV head: both products on the matrix cores, 16 head columns
+    (2, 24, 2, 700, 64, 0),
+    (1, 16, 1, 1100, 64, 2),
 ]
 
 
@@ -341,6 +344,8 @@ TYPED_CASES = [
     (torch.bfloat16, 1, 8, 2, 128, 1024, 256, 896, True, 0),
     (torch.bfloat16, 2, 4, 1, 33, 200, 256, 167, False, 1),
     (torch.bfloat16, 1, 4, 2, 300, 300, 256, 0, False, 2),  # square causal prefill
+    (torch.float16, 1, 16, 2, 40, 900, 128, 1000, True, 0),  # 8 heads per KV head: the decode step multiplies on the matrix cores
+    (torch.float16, 1, 16, 1, 20, 450, 64, 500, False, 0),
 ]
 
 

@@ -419,6 +419,9 @@ def test_attention_over_uint8_cache(kvx, gpu):
     (2, 6, 2, 600, 128, 600, False, False),
     (1, 5, 1, 300, 64, 256, True, True),
     (1, 8, 2, 12000, 128, 11000, True, False),
+    (1, 16, 1, 2100, 128, 2000, False, True),   # 16 heads per KV head over the 8-bit store
+    (1, 12, 1, 900, 64, 900, True, False),
+    (2, 32, 4, 5000, 128, 5000, False, True),   # 8 heads per KV head, 8-bit store, several splits per row
 ])
 def test_fused_decode_h2o_matches_separate_calls(kvx, gpu, decode_route, B, Hq, Hkv, T, D, limit, normalize, quantized):
     """kvx_sdpa_decode_h2o == kvx_sdpa_decode (with weights) followed by kvx_h2o_update_select(k=1),

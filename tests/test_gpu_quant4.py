@@ -141,7 +141,8 @@ def test_blocks_over_heads_store_feeds_attention(gpu):
     torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,q_len,T,D", [(1, 8, 2, 96, 2048 + 40, 128), (2, 4, 4, 33, 515, 64), (1, 8, 1, 1, 3000, 128)])
+@pytest.mark.parametrize("B,Hq,Hkv,q_len,T,D", [(1, 8, 2, 96, 2048 + 40, 128), (2, 4, 4, 33, 515, 64), (1, 8, 1, 1, 3000, 128),
+                                                 (1, 16, 1, 1, 1500, 64), (2, 8, 4, 1, 4100, 128)])
 def test_attention_over_4bit_cache(kvx, gpu, B, Hq, Hkv, q_len, T, D):
     """Attention output, score-sums (prefill kernel + score-sum kernel) and single-token decode over the
     4-bit store, the nibbles unpacked and dequantised inside the kernels, against the oracle run on
