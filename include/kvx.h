@@ -55,10 +55,13 @@ enum kvx_kv_dtype {
                       keys_values/kvcache/quantize/pytorch.py:143-154,467-478 would, i.e. to bf16 */
   KVX_KV_F16 = 3,  /* float16 rows; q and o are then float16 as well (the reference's extension takes float16 and
                       bfloat16, keys_values/csrc/bindings.cpp:207, keys_values/attention/flashinfer_wrapper.py:311-319).
-                      Every other value of this enum goes with bfloat16 q and o. */
-  KVX_KV_U4 = 2    /* the 4-bit store of the same quantiser ("torch-quantized4"): rows of D/2 bytes, byte j =
+                      KVX_KV_BF16, KVX_KV_U8 and KVX_KV_U4 go with bfloat16 q and o. */
+  KVX_KV_U4 = 2,   /* the 4-bit store of the same quantiser ("torch-quantized4"): rows of D/2 bytes, byte j =
                       code[j] << 4 | code[j + D/2] (keys_values/kvcache/quantize/pytorch.py:384-393,457-465),
                       same per-row state; strides of k / v count bytes */
+  KVX_KV_U8_F16 = 4, /* KVX_KV_U8 / KVX_KV_U4 for a float16 model: the rows were float16 when they were quantised, */
+  KVX_KV_U4_F16 = 5  /* they dequantise to float16 (the quantiser casts back to its source type,
+                        keys_values/kvcache/quantize/pytorch.py:333,478), and q and o are float16 */
 };
 
 /* One attention call. Unused pointers are NULL. All strides in elements. */
@@ -206,6 +209,15 @@ int kvx_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int32_
 int kvx_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows,
                          int32_t D, void* out, int64_t out_row_stride, void* stream);
 
+/* The four calls above with the number of bits (8 or 4) and the type of the rows as arguments: elem_dtype is
+ * KVX_KV_BF16 or KVX_KV_F16. The quantiser upcasts any float type to fp32 and casts the dequantised values back to
+ * the type it was built for (source_dtype, keys_values/kvcache/quantize/pytorch.py:333,478), so a float16 model's
+ * store holds codes of float16 rows and dequantises to float16. */
+int kvx_quantize_rows_typed(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, int32_t bits, int32_t elem_dtype,
+                            uint8_t* codes, float* scale, int32_t* zp, void* stream);
+int kvx_dequantize_rows_typed(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D,
+                              int32_t bits, int32_t elem_dtype, void* out, int64_t out_row_stride, void* stream);
+
 /* General form: a quantisation block is `nseg` segments of D contiguous bf16 values, segment s of block
  * (o, i) at x + o*x_stride_outer + i*x_stride_inner + s*x_stride_seg (strides in elements). With
  * nseg = n_query_groups and the segment stride that of the head axis this is blocks_over_heads=True
@@ -224,6 +236,7 @@ typedef struct kvx_block_quant_args {
   float* scale;
   int32_t* zp;
   int64_t state_stride_outer; /* elements */
+  int32_t elem_dtype;         /* type of x: KVX_KV_BF16 (0) or KVX_KV_F16 */
 } kvx_block_quant_args;
 int kvx_quantize_blocks(const kvx_block_quant_args* args, void* stream);
 int kvx_dequantize_blocks(const kvx_block_quant_args* args, void* stream);
@@ -392,7 +405,7 @@ int kvx_swiglu_rows(const void* gate_up, int64_t gate_up_row_stride, void* out, 
  * q_weight / k_weight: fp32 (D) norm weights, or both NULL for no normalisation.
  * cos / sin: fp32 tables (table_rows, D / 2), row p = cos / sin of p * theta_j (half-split
  *      convention: element d is paired with d +- D/2). Token t of the chunk sits at input_pos + t.
- * D in {64, 128}. */
+ * D in {64, 128, 256}. */
 int kvx_qk_norm_rope(void* qkv, int64_t stride_b, int64_t stride_t, int32_t B, int32_t num, int32_t Hq,
                      int32_t Hkv, int32_t D, const float* q_weight, const float* k_weight, float eps,
                      const float* cos, const float* sin, int32_t table_rows, int32_t input_pos,

@@ -9,7 +9,19 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libkvx.so")
 
 KVX_OK, KVX_ERR_INVALID, KVX_ERR_UNSUPPORTED, KVX_ERR_HIP, KVX_ERR_WORKSPACE = 0, 1, 2, 3, 4
-KVX_KV_BF16, KVX_KV_U8, KVX_KV_U4, KVX_KV_F16 = 0, 1, 2, 3
+KVX_KV_BF16, KVX_KV_U8, KVX_KV_U4, KVX_KV_F16, KVX_KV_U8_F16, KVX_KV_U4_F16 = 0, 1, 2, 3, 4, 5
+
+
+def quant_kv_dtype(num_bits: int, dtype) -> int:
+    """enum kvx_kv_dtype of a quantised store of ``num_bits`` codes whose rows were (and dequantise to) ``dtype``."""
+    f16 = dtype == torch.float16
+    if num_bits == 4:
+        return KVX_KV_U4_F16 if f16 else KVX_KV_U4
+    return KVX_KV_U8_F16 if f16 else KVX_KV_U8
+
+
+def elem_kv_dtype(dtype) -> int:
+    return KVX_KV_F16 if dtype == torch.float16 else KVX_KV_BF16
 
 
 class SdpaArgs(ctypes.Structure):
@@ -76,6 +88,7 @@ class BlockQuantArgs(ctypes.Structure):
         ("n_outer", c_int32), ("n_inner", c_int32), ("nseg", c_int32), ("D", c_int32), ("bits", c_int32),
         ("codes", c_void_p), ("codes_stride_outer", c_int64),
         ("scale", c_void_p), ("zp", c_void_p), ("state_stride_outer", c_int64),
+        ("elem_dtype", c_int32),
     ]
 
 
@@ -98,6 +111,8 @@ SYMBOLS = {
     "kvx_dequantize_rows": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
     "kvx_quantize_rows4": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "kvx_dequantize_rows4": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
+    "kvx_quantize_rows_typed": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "kvx_dequantize_rows_typed": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p]),
     "kvx_quantize_blocks": (ctypes.c_int, [POINTER(BlockQuantArgs), c_void_p]),
     "kvx_dequantize_blocks": (ctypes.c_int, [POINTER(BlockQuantArgs), c_void_p]),
     "kvx_cache_write": (ctypes.c_int, [POINTER(CacheWriteArgs), c_void_p]),

@@ -90,7 +90,7 @@ def _fill_common(a: _lib.SdpaArgs, query, key, value, scale, input_pos, token_po
         a.v_stride_b, a.v_stride_h, a.v_stride_t = value.stride(0), value.stride(1), value.stride(2)
     if quant is not None:
         # rows of D bytes: 8-bit codes; rows of D/2 bytes: the 4-bit store, two codes per byte
-        a.kv_dtype = _lib.KVX_KV_U4 if key.shape[3] * 2 == D else _lib.KVX_KV_U8
+        a.kv_dtype = _lib.quant_kv_dtype(4 if key.shape[3] * 2 == D else 8, query.dtype)  # the rows dequantise to the query's type
         for t in quant:
             if t.shape != (B, Hkv, T) or t.stride(-1) != 1 or t.stride() != quant.k_scale.stride():
                 raise ValueError("quantisation state must be (B, Hkv, T) arrays sharing strides, last axis contiguous")
@@ -114,8 +114,6 @@ def _row_len(D: int, key: torch.Tensor, quant) -> int:
 def _check_dtypes(query, key, value, quant):
     if query.dtype not in ALLOWED_DTYPES:
         raise NotImplementedError(f"query.dtype must be torch.bfloat16 or torch.float16, got {query.dtype}")
-    if quant is not None and query.dtype != torch.bfloat16:
-        raise NotImplementedError("the quantised stores dequantise to bfloat16: query.dtype must be torch.bfloat16")
     want = torch.uint8 if quant is not None else query.dtype
     for name, t in (("key", key), ("value", value)):
         if t is not None and t.dtype != want:

@@ -52,11 +52,10 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
   // batch and head indices are grid dimensions, and B * Hq rows are counted in 32 bits
   KVX_REQUIRE(a->B <= 65535 && a->Hq <= 65535 && (int64_t)a->B * a->Hq < ((int64_t)1 << 24), KVX_ERR_UNSUPPORTED,
               "%s: B=%d, Hq=%d beyond 65535 each or 2^24 together", who, a->B, a->Hq);
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4 || a->kv_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED,
-              "%s: unknown kv_dtype %d", who, a->kv_dtype);
+  KVX_REQUIRE(kv_valid(a->kv_dtype), KVX_ERR_UNSUPPORTED, "%s: unknown kv_dtype %d", who, a->kv_dtype);
   KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
               "%s: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", who, a->D);
-  const int row_elems = a->kv_dtype == KVX_KV_U4 ? a->D / 2 : a->D;  // elements of the cache's own type per row
+  const int row_elems = kv_is_u4(a->kv_dtype) ? a->D / 2 : a->D;  // elements of the cache's own type per row
   KVX_REQUIRE(a->input_pos >= 0, KVX_ERR_INVALID, "%s: input_pos=%d must be >= 0", who, a->input_pos);
   KVX_REQUIRE(a->sm_scale > 0.0f, KVX_ERR_INVALID, "%s: sm_scale must be positive", who);
   KVX_REQUIRE((int64_t)a->input_pos + a->q_len < INT32_MAX, KVX_ERR_INVALID, "%s: positions overflow int32", who);
@@ -174,58 +173,63 @@ int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
   return launch_sdpa_decode(*a, nullptr, (hipStream_t)stream);
 }
 
-int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale,
-                      int32_t* zp, void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_quantize_rows: row length %d not in {64, 128}", D);
-  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_quantize_rows: rows must be >= 0");
+static int quantize_rows_checked(const char* who, const void* x, int64_t x_row_stride, int64_t rows, int32_t D, int32_t bits, int32_t elem_dtype,
+                                 uint8_t* codes, float* scale, int32_t* zp, void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128}", who, D);
+  KVX_REQUIRE(bits == 8 || bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, bits);
+  KVX_REQUIRE(elem_dtype == KVX_KV_BF16 || elem_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED, "%s: elem_dtype %d is neither KVX_KV_BF16 nor KVX_KV_F16", who, elem_dtype);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "%s: rows must be >= 0", who);
   if (rows == 0) return KVX_OK;
-  KVX_REQUIRE(x && codes && scale && zp, KVX_ERR_INVALID, "kvx_quantize_rows: NULL pointer");
+  KVX_REQUIRE(x && codes && scale && zp, KVX_ERR_INVALID, "%s: NULL pointer", who);
   KVX_REQUIRE(aligned16(x) && mult8(x_row_stride) && x_row_stride >= D, KVX_ERR_INVALID,
-              "kvx_quantize_rows: x must be 16-byte aligned, row stride a multiple of 8 and >= D");
-  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_quantize_rows: codes must be 8-byte aligned");
-  return launch_quantize_rows(x, x_row_stride, rows, D, codes, scale, zp, (hipStream_t)stream);
+              "%s: x must be 16-byte aligned, row stride a multiple of 8 and >= D", who);
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "%s: codes must be 8-byte aligned", who);
+  return launch_quantize_rows(x, x_row_stride, rows, D, bits, elem_dtype == KVX_KV_F16, codes, scale, zp, (hipStream_t)stream);
 }
 
-int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out,
-                        int64_t out_row_stride, void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_dequantize_rows: row length %d not in {64, 128}", D);
-  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_dequantize_rows: rows must be >= 0");
+static int dequantize_rows_checked(const char* who, const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, int32_t bits,
+                                   int32_t elem_dtype, void* out, int64_t out_row_stride, void* stream) {
+  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128}", who, D);
+  KVX_REQUIRE(bits == 8 || bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, bits);
+  KVX_REQUIRE(elem_dtype == KVX_KV_BF16 || elem_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED, "%s: elem_dtype %d is neither KVX_KV_BF16 nor KVX_KV_F16", who, elem_dtype);
+  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "%s: rows must be >= 0", who);
   if (rows == 0) return KVX_OK;
-  KVX_REQUIRE(codes && scale && zp && out, KVX_ERR_INVALID, "kvx_dequantize_rows: NULL pointer");
+  KVX_REQUIRE(codes && scale && zp && out, KVX_ERR_INVALID, "%s: NULL pointer", who);
   KVX_REQUIRE(aligned16(out) && mult8(out_row_stride) && out_row_stride >= D, KVX_ERR_INVALID,
-              "kvx_dequantize_rows: out must be 16-byte aligned, row stride a multiple of 8 and >= D");
-  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_dequantize_rows: codes must be 8-byte aligned");
-  return launch_dequantize_rows(codes, scale, zp, rows, D, out, out_row_stride, (hipStream_t)stream);
+              "%s: out must be 16-byte aligned, row stride a multiple of 8 and >= D", who);
+  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "%s: codes must be 8-byte aligned", who);
+  return launch_dequantize_rows(codes, scale, zp, rows, D, bits, elem_dtype == KVX_KV_F16, out, out_row_stride, (hipStream_t)stream);
 }
 
-int kvx_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale, int32_t* zp,
-                       void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_quantize_rows4: row length %d not in {64, 128}", D);
-  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_quantize_rows4: rows must be >= 0");
-  if (rows == 0) return KVX_OK;
-  KVX_REQUIRE(x && codes && scale && zp, KVX_ERR_INVALID, "kvx_quantize_rows4: NULL pointer");
-  KVX_REQUIRE(aligned16(x) && mult8(x_row_stride) && x_row_stride >= D, KVX_ERR_INVALID,
-              "kvx_quantize_rows4: x must be 16-byte aligned, row stride a multiple of 8 and >= D");
-  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_quantize_rows4: codes must be 8-byte aligned");
-  return launch_quantize_rows4(x, x_row_stride, rows, D, codes, scale, zp, (hipStream_t)stream);
+int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale, int32_t* zp, void* stream) {
+  return quantize_rows_checked("kvx_quantize_rows", x, x_row_stride, rows, D, 8, KVX_KV_BF16, codes, scale, zp, stream);
 }
-
-int kvx_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out,
-                         int64_t out_row_stride, void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_dequantize_rows4: row length %d not in {64, 128}", D);
-  KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "kvx_dequantize_rows4: rows must be >= 0");
-  if (rows == 0) return KVX_OK;
-  KVX_REQUIRE(codes && scale && zp && out, KVX_ERR_INVALID, "kvx_dequantize_rows4: NULL pointer");
-  KVX_REQUIRE(aligned16(out) && mult8(out_row_stride) && out_row_stride >= D, KVX_ERR_INVALID,
-              "kvx_dequantize_rows4: out must be 16-byte aligned, row stride a multiple of 8 and >= D");
-  KVX_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 7) == 0, KVX_ERR_INVALID, "kvx_dequantize_rows4: codes must be 8-byte aligned");
-  return launch_dequantize_rows4(codes, scale, zp, rows, D, out, out_row_stride, (hipStream_t)stream);
+int kvx_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out, int64_t out_row_stride,
+                        void* stream) {
+  return dequantize_rows_checked("kvx_dequantize_rows", codes, scale, zp, rows, D, 8, KVX_KV_BF16, out, out_row_stride, stream);
+}
+int kvx_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, uint8_t* codes, float* scale, int32_t* zp, void* stream) {
+  return quantize_rows_checked("kvx_quantize_rows4", x, x_row_stride, rows, D, 4, KVX_KV_BF16, codes, scale, zp, stream);
+}
+int kvx_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, void* out, int64_t out_row_stride,
+                         void* stream) {
+  return dequantize_rows_checked("kvx_dequantize_rows4", codes, scale, zp, rows, D, 4, KVX_KV_BF16, out, out_row_stride, stream);
+}
+int kvx_quantize_rows_typed(const void* x, int64_t x_row_stride, int64_t rows, int32_t D, int32_t bits, int32_t elem_dtype, uint8_t* codes,
+                            float* scale, int32_t* zp, void* stream) {
+  return quantize_rows_checked("kvx_quantize_rows_typed", x, x_row_stride, rows, D, bits, elem_dtype, codes, scale, zp, stream);
+}
+int kvx_dequantize_rows_typed(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, int32_t bits,
+                              int32_t elem_dtype, void* out, int64_t out_row_stride, void* stream) {
+  return dequantize_rows_checked("kvx_dequantize_rows_typed", codes, scale, zp, rows, D, bits, elem_dtype, out, out_row_stride, stream);
 }
 
 static int check_blocks(const kvx_block_quant_args* a, const char* who) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "%s: args is NULL", who);
   KVX_REQUIRE(a->n_outer >= 0 && a->n_inner >= 0 && a->nseg > 0 && a->D > 0, KVX_ERR_INVALID, "%s: bad sizes", who);
   KVX_REQUIRE(a->bits == 8 || a->bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, a->bits);
+  KVX_REQUIRE(a->elem_dtype == KVX_KV_BF16 || a->elem_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED, "%s: elem_dtype %d is neither KVX_KV_BF16 nor KVX_KV_F16",
+              who, a->elem_dtype);
   KVX_REQUIRE(a->D % 16 == 0 && (int64_t)a->nseg * a->D <= 8192, KVX_ERR_UNSUPPORTED,
               "%s: D = %d must be a multiple of 16 and the block (nseg * D = %lld) at most 8192 values", who, a->D,
               (long long)a->nseg * a->D);
@@ -253,8 +257,7 @@ int kvx_dequantize_blocks(const kvx_block_quant_args* a, void* stream) {
 int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");
-  KVX_REQUIRE(a->kv_dtype == KVX_KV_BF16 || a->kv_dtype == KVX_KV_U8 || a->kv_dtype == KVX_KV_U4 || a->kv_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED,
-              "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
+  KVX_REQUIRE(kv_valid(a->kv_dtype), KVX_ERR_UNSUPPORTED, "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
   KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
               "kvx_cache_write: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a->D);
   KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
@@ -370,7 +373,7 @@ int kvx_qk_norm_rope(void* qkv, int64_t stride_b, int64_t stride_t, int32_t B, i
                      int32_t input_pos, void* stream) {
   KVX_REQUIRE(B >= 0 && num >= 0 && Hq > 0 && Hkv > 0, KVX_ERR_INVALID, "kvx_qk_norm_rope: B=%d num=%d Hq=%d Hkv=%d", B, num, Hq, Hkv);
   if (B == 0 || num == 0) return KVX_OK;
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "kvx_qk_norm_rope: head size %d not in {64, 128}", D);
+  KVX_REQUIRE(D == 64 || D == 128 || D == 256, KVX_ERR_UNSUPPORTED, "kvx_qk_norm_rope: head size %d not in {64, 128, 256}", D);
   KVX_REQUIRE(qkv && cos && sin, KVX_ERR_INVALID, "kvx_qk_norm_rope: NULL pointer");
   KVX_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), KVX_ERR_INVALID, "kvx_qk_norm_rope: give both norm weights or none");
   KVX_REQUIRE(input_pos >= 0 && (int64_t)input_pos + num <= table_rows, KVX_ERR_INVALID,

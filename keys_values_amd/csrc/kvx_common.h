@@ -52,14 +52,10 @@ size_t score_sum_workspace(const kvx_sdpa_args& a);
 int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* fused_h2o, hipStream_t st);
 size_t sdpa_decode_workspace(const kvx_sdpa_args& a, bool fused_h2o);
 void set_decode_tuning(int resident, int spin_limit, int poll_sleep);
-int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,
+int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, int bits, bool f16, uint8_t* codes, float* scale,
                          int32_t* zp, hipStream_t st);
-int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
+int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, int bits, bool f16, void* out,
                            int64_t out_row_stride, hipStream_t st);
-int launch_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale, int32_t* zp,
-                          hipStream_t st);
-int launch_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
-                            int64_t out_row_stride, hipStream_t st);
 int launch_quantize_blocks(const kvx_block_quant_args& a, hipStream_t st);
 int launch_dequantize_blocks(const kvx_block_quant_args& a, hipStream_t st);
 int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st);
@@ -98,6 +94,23 @@ typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
 // plain rows of the query's own type (no codes)
 constexpr bool kv_is_plain(int kv) { return kv == KVX_KV_BF16 || kv == KVX_KV_F16; }
+// q, o and the (dequantised) rows are float16, else bfloat16
+constexpr bool kv_elem_f16(int kv) { return kv == KVX_KV_F16 || kv == KVX_KV_U8_F16 || kv == KVX_KV_U4_F16; }
+// two codes per byte
+constexpr bool kv_is_u4(int kv) { return kv == KVX_KV_U4 || kv == KVX_KV_U4_F16; }
+constexpr bool kv_valid(int kv) { return kv >= KVX_KV_BF16 && kv <= KVX_KV_U4_F16; }
+
+// the two halves of a packed pair of the element type as fp32
+template <bool F16>
+__device__ __forceinline__ float elem_lo(uint32_t packed) {
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2_t, packed)[0];
+  else return __uint_as_float(packed << 16);
+}
+template <bool F16>
+__device__ __forceinline__ float elem_hi(uint32_t packed) {
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2_t, packed)[1];
+  else return __uint_as_float(packed & 0xffff0000u);
+}
 
 // D = A B + C on one 32x32x16 tile, operands as four dwords of eight 16-bit values
 template <bool F16>
@@ -110,7 +123,9 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16(u32x4_t a, u32x4_t b, f32x16_t
 template <bool F16>
 __device__ __forceinline__ uint32_t pack_pair(float a, float b) {
   if constexpr (F16) {
-    const f16x2_t r = __builtin_convertvector(f32x2_t{a, b}, f16x2_t);
+    // two scalar conversions (round to nearest even): a conversion of the pair as a vector trips the instruction
+    // selector when packed fp32 arithmetic is switched off and one operand is a negation
+    const f16x2_t r = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, r);
   } else {
     return pack_bf16(a, b);
@@ -159,24 +174,26 @@ __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, i
   zp = 0 - (int32_t)__builtin_rintf(mn / s);
 }
 
-// bf16( (float)((int)code - zp) * scale ), two codes -> packed dword.
+// elem( (float)((int)code - zp) * scale ), two codes -> packed dword of the element type (bf16, or fp16 with F16).
+template <bool F16 = false>
 __device__ __forceinline__ uint32_t dequant_pair(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
   float a = (float)((int32_t)c0 - zp) * scale;
   float b = (float)((int32_t)c1 - zp) * scale;
-  return pack_bf16(a, b);
+  return pack_pair<F16>(a, b);
 }
 
-// 8 byte-sized codes (two dwords) -> 8 bf16 (four dwords). (Forming code - zp in fp32 from
+// 8 byte-sized codes (two dwords) -> 8 values of the element type (four dwords). (Forming code - zp in fp32 from
 // byte-to-float conversions is exact for |zp| < 2^24 but measured no faster than this integer form; forming it
 // in packed fp16 (bytes 0x64, code = 1024 + code; v_pk_add_f16 of -(1024 + zp); v_fma_mix_f32 by the scale) gives
 // the same bits with one instruction less per value for small zero points and measured 5 - 7 % slower in the
 // decode and prefill kernels.)
+template <bool F16 = false>
 __device__ __forceinline__ u32x4_t dequant_words(uint32_t c0, uint32_t c1, int32_t zp, float scale) {
   u32x4_t r;
-  r[0] = dequant_pair(c0 & 0xff, (c0 >> 8) & 0xff, zp, scale);
-  r[1] = dequant_pair((c0 >> 16) & 0xff, c0 >> 24, zp, scale);
-  r[2] = dequant_pair(c1 & 0xff, (c1 >> 8) & 0xff, zp, scale);
-  r[3] = dequant_pair((c1 >> 16) & 0xff, c1 >> 24, zp, scale);
+  r[0] = dequant_pair<F16>(c0 & 0xff, (c0 >> 8) & 0xff, zp, scale);
+  r[1] = dequant_pair<F16>((c0 >> 16) & 0xff, c0 >> 24, zp, scale);
+  r[2] = dequant_pair<F16>(c1 & 0xff, (c1 >> 8) & 0xff, zp, scale);
+  r[3] = dequant_pair<F16>((c1 >> 16) & 0xff, c1 >> 24, zp, scale);
   return r;
 }
 

@@ -289,7 +289,10 @@ int launch_qk_norm_rope(void* qkv, int64_t sb, int64_t stt, int B, int num, int 
   const float factor = 1.0f / sqrtf((float)D);
   const int rpb = NT / (D / 8);
   const unsigned grid = (unsigned)((total + rpb - 1) / rpb);
-  if (D == 128)
+  if (D == 256)
+    hipLaunchKernelGGL(qk_norm_rope_kernel<256>, dim3(grid), dim3(NT), 0, st, (uint16_t*)qkv, sb, stt, B, num, Hq, Hkv, qw, kw, eps, factor,
+                       cos_t, sin_t, input_pos);
+  else if (D == 128)
     hipLaunchKernelGGL(qk_norm_rope_kernel<128>, dim3(grid), dim3(NT), 0, st, (uint16_t*)qkv, sb, stt, B, num, Hq, Hkv, qw, kw, eps, factor,
                        cos_t, sin_t, input_pos);
   else

@@ -70,12 +70,12 @@ __device__ __forceinline__ uint32_t codes4_u4(float x0, float x1, float x2, floa
   return __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_rintf(x3 * inv) + zf, 15.0f), 3, w);
 }
 
-template <int LPR>
+template <int LPR, bool F16>
 __device__ __forceinline__ void row_extremes(u32x4_t raw, float (&x)[8], float& mn, float& mx) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    x[2 * e] = bf16_lo(raw[e]);
-    x[2 * e + 1] = bf16_hi(raw[e]);
+    x[2 * e] = elem_lo<F16>(raw[e]);
+    x[2 * e + 1] = elem_hi<F16>(raw[e]);
   }
   mn = x[0];
   mx = x[0];
@@ -93,13 +93,13 @@ __device__ __forceinline__ void row_extremes(u32x4_t raw, float (&x)[8], float& 
 // all lanes of a row hold its extremes, so lane c of a quad works out the scale and zero point of row
 // c only, and the others fetch 1 / scale and the zero point from it with a quad broadcast. Returns the
 // codes of row i in c[i] (bytes), and in (scale, zp) the state of row (lane & 3).
-template <int LPR, int BITS>
+template <int LPR, int BITS, bool F16>
 __device__ __forceinline__ void quantize_rows_in_flight(const u32x4_t (&raw)[ROWS_PER_THREAD], u32x2_t (&c)[ROWS_PER_THREAD], float& scale,
                                                         int32_t& zp) {
   static_assert(ROWS_PER_THREAD == 4, "one row per lane of a quad");
   float x[ROWS_PER_THREAD][8], mn[ROWS_PER_THREAD], mx[ROWS_PER_THREAD];
 #pragma unroll
-  for (int i = 0; i < ROWS_PER_THREAD; ++i) row_extremes<LPR>(raw[i], x[i], mn[i], mx[i]);
+  for (int i = 0; i < ROWS_PER_THREAD; ++i) row_extremes<LPR, F16>(raw[i], x[i], mn[i], mx[i]);
   const int mine = (int)(__lane_id() & 3u);
   const float my_mn = mine == 0 ? mn[0] : mine == 1 ? mn[1] : mine == 2 ? mn[2] : mn[3];
   const float my_mx = mine == 0 ? mx[0] : mine == 1 ? mx[1] : mine == 2 ? mx[2] : mx[3];
@@ -129,13 +129,13 @@ __device__ __forceinline__ void quantize_rows_in_flight(const u32x4_t (&raw)[ROW
 
 // Quantise the 8 values of this lane's share of a row; every lane of the row returns the same
 // scale / zero point.
-template <int LPR>
+template <int LPR, bool F16>
 __device__ __forceinline__ u32x2_t quantize8(u32x4_t raw, float& scale, int32_t& zp) {
   float x[8];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    x[2 * e] = bf16_lo(raw[e]);
-    x[2 * e + 1] = bf16_hi(raw[e]);
+    x[2 * e] = elem_lo<F16>(raw[e]);
+    x[2 * e + 1] = elem_hi<F16>(raw[e]);
   }
   float mn = x[0], mx = x[0];
 #pragma unroll
@@ -157,7 +157,7 @@ __device__ __forceinline__ u32x2_t quantize8(u32x4_t raw, float& scale, int32_t&
   return out;
 }
 
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
                                                                  int64_t rows, uint8_t* __restrict__ codes,
                                                                  float* __restrict__ scale, int32_t* __restrict__ zp) {
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t*
   u32x2_t c[ROWS_PER_THREAD];
   float s;
   int32_t z;
-  quantize_rows_in_flight<LPR, 8>(raw, c, s, z);  // executed by all lanes: the DPP exchanges need them
+  quantize_rows_in_flight<LPR, 8, F16>(raw, c, s, z);  // executed by all lanes: the DPP exchanges need them
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows_kernel(const uint16_t*
   }
 }
 
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t* __restrict__ codes,
                                                                    const float* __restrict__ scale,
                                                                    const int32_t* __restrict__ zp, int64_t rows,
@@ -212,20 +212,20 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_rows_kernel(const uint8_t
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
     if (r >= rows) continue;
-    *(u32x4_t*)(out + r * out_row_stride + col * 8) = dequant_words(c[i][0], c[i][1], z[i], s[i]);
+    *(u32x4_t*)(out + r * out_row_stride + col * 8) = dequant_words<F16>(c[i][0], c[i][1], z[i], s[i]);
   }
 }
 
 // ---- 4-bit rows -------------------------------------------------------------------------------
 
 // Codes of the lane's 8 values as bytes (0..15), same layout as quantize8.
-template <int LPR>
+template <int LPR, bool F16>
 __device__ __forceinline__ u32x2_t quantize4(u32x4_t raw, float& scale, int32_t& zp) {
   float x[8];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    x[2 * e] = bf16_lo(raw[e]);
-    x[2 * e + 1] = bf16_hi(raw[e]);
+    x[2 * e] = elem_lo<F16>(raw[e]);
+    x[2 * e + 1] = elem_hi<F16>(raw[e]);
   }
   float mn = x[0], mx = x[0];
 #pragma unroll
@@ -249,7 +249,7 @@ __device__ __forceinline__ u32x2_t quantize4(u32x4_t raw, float& scale, int32_t&
 
 // Element d shares its byte with element d + D/2 (high nibble = first half of the row): the lanes of
 // the first half fetch their partner's codes from the lane LPR/2 away and store 8 packed bytes.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(NTHREADS) void quantize_rows4_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride, int64_t rows,
                                                                   uint8_t* __restrict__ codes, float* __restrict__ scale,
                                                                   int32_t* __restrict__ zp) {
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows4_kernel(const uint16_t
   u32x2_t c[ROWS_PER_THREAD];
   float s;
   int32_t z;
-  quantize_rows_in_flight<LPR, 4>(raw, c, s, z);  // executed by all lanes: the reductions and the exchanges need them
+  quantize_rows_in_flight<LPR, 4, F16>(raw, c, s, z);  // executed by all lanes: the reductions and the exchanges need them
 #pragma unroll
   for (int i = 0; i < ROWS_PER_THREAD; ++i) {
     const int64_t r = row0 + (int64_t)i * RPB;
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_rows4_kernel(const uint16_t
 }
 
 // One lane per 8 packed bytes: the high nibbles are elements col*8.., the low nibbles D/2 + col*8...
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(NTHREADS) void dequantize_rows4_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ scale,
                                                                     const int32_t* __restrict__ zp, int64_t rows,
                                                                     uint16_t* __restrict__ out, int64_t out_row_stride) {
@@ -297,8 +297,8 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_rows4_kernel(const uint8_
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const uint32_t w = c[e >> 1] >> ((e & 1) * 16);
-    hi[e] = dequant_pair((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
-    lo[e] = dequant_pair(w & 0xf, (w >> 8) & 0xf, z, s);
+    hi[e] = dequant_pair<F16>((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
+    lo[e] = dequant_pair<F16>(w & 0xf, (w >> 8) & 0xf, z, s);
   }
   *(u32x4_t*)(out + r * out_row_stride + col * 8) = hi;
   *(u32x4_t*)(out + r * out_row_stride + D / 2 + col * 8) = lo;
@@ -317,16 +317,17 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+template <bool F16>
 __device__ __forceinline__ u32x2_t codes_of_chunk(u32x4_t raw, float inv, float zf, float qmax) {
   u32x2_t out;
 #pragma unroll
   for (int h = 0; h < 2; ++h)
-    out[h] = quant_code(bf16_lo(raw[2 * h]), inv, zf, qmax) | (quant_code(bf16_hi(raw[2 * h]), inv, zf, qmax) << 8) |
-             (quant_code(bf16_lo(raw[2 * h + 1]), inv, zf, qmax) << 16) | (quant_code(bf16_hi(raw[2 * h + 1]), inv, zf, qmax) << 24);
+    out[h] = quant_code(elem_lo<F16>(raw[2 * h]), inv, zf, qmax) | (quant_code(elem_hi<F16>(raw[2 * h]), inv, zf, qmax) << 8) |
+             (quant_code(elem_lo<F16>(raw[2 * h + 1]), inv, zf, qmax) << 16) | (quant_code(elem_hi<F16>(raw[2 * h + 1]), inv, zf, qmax) << 24);
   return out;
 }
 
-template <int BITS>
+template <int BITS, bool F16>
 __global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_block_quant_args a) {
   const int lane = threadIdx.x & 63;
   const int64_t blk = (int64_t)blockIdx.x * (NTHREADS / 64) + (threadIdx.x >> 6);
@@ -341,9 +342,9 @@ __global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_blo
     const u32x4_t raw = chunk(c);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      mn = fminf(mn, fminf(bf16_lo(raw[e]), bf16_hi(raw[e])));
-      mx = fmaxf(mx, fmaxf(bf16_lo(raw[e]), bf16_hi(raw[e])));
-      bad = __builtin_isunordered(bf16_lo(raw[e]), bf16_hi(raw[e])) ? 1.0f : bad;
+      mn = fminf(mn, fminf(elem_lo<F16>(raw[e]), elem_hi<F16>(raw[e])));
+      mx = fmaxf(mx, fmaxf(elem_lo<F16>(raw[e]), elem_hi<F16>(raw[e])));
+      bad = __builtin_isunordered(elem_lo<F16>(raw[e]), elem_hi<F16>(raw[e])) ? 1.0f : bad;
     }
   }
   mn = wave_min(mn);
@@ -356,11 +357,11 @@ __global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_blo
   const float inv = 1.0f / s, zf = (float)z;
   uint8_t* out = a.codes + outer * a.codes_stride_outer + inner * ((int64_t)nchunks * BITS);  // nchunks * 8 values * BITS / 8 bytes
   if constexpr (BITS == 8) {
-    for (int c = lane; c < nchunks; c += 64) *(u32x2_t*)(out + c * 8) = codes_of_chunk(chunk(c), inv, zf, qmax);
+    for (int c = lane; c < nchunks; c += 64) *(u32x2_t*)(out + c * 8) = codes_of_chunk<F16>(chunk(c), inv, zf, qmax);
   } else {
     const int half = nchunks / 2;
     for (int c = lane; c < half; c += 64) {
-      const u32x2_t hi = codes_of_chunk(chunk(c), inv, zf, qmax), lo = codes_of_chunk(chunk(c + half), inv, zf, qmax);
+      const u32x2_t hi = codes_of_chunk<F16>(chunk(c), inv, zf, qmax), lo = codes_of_chunk<F16>(chunk(c + half), inv, zf, qmax);
       *(u32x2_t*)(out + c * 8) = u32x2_t{(hi[0] << 4) | lo[0], (hi[1] << 4) | lo[1]};
     }
   }
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(NTHREADS) void quantize_blocks_kernel(const kvx_blo
   }
 }
 
-template <int BITS>
+template <int BITS, bool F16>
 __global__ __launch_bounds__(NTHREADS) void dequantize_blocks_kernel(const kvx_block_quant_args a) {
   const int lane = threadIdx.x & 63;
   const int64_t blk = (int64_t)blockIdx.x * (NTHREADS / 64) + (threadIdx.x >> 6);
@@ -387,10 +388,10 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_blocks_kernel(const kvx_b
     for (int c = lane; c < nchunks; c += 64) {
       const u32x2_t cc = *(const u32x2_t*)(in + c * 8);
       u32x4_t o;
-      o[0] = dequant_pair(cc[0] & 0xff, (cc[0] >> 8) & 0xff, z, s);
-      o[1] = dequant_pair((cc[0] >> 16) & 0xff, cc[0] >> 24, z, s);
-      o[2] = dequant_pair(cc[1] & 0xff, (cc[1] >> 8) & 0xff, z, s);
-      o[3] = dequant_pair((cc[1] >> 16) & 0xff, cc[1] >> 24, z, s);
+      o[0] = dequant_pair<F16>(cc[0] & 0xff, (cc[0] >> 8) & 0xff, z, s);
+      o[1] = dequant_pair<F16>((cc[0] >> 16) & 0xff, cc[0] >> 24, z, s);
+      o[2] = dequant_pair<F16>(cc[1] & 0xff, (cc[1] >> 8) & 0xff, z, s);
+      o[3] = dequant_pair<F16>((cc[1] >> 16) & 0xff, cc[1] >> 24, z, s);
       *chunk_ptr(c) = o;
     }
   } else {
@@ -401,8 +402,8 @@ __global__ __launch_bounds__(NTHREADS) void dequantize_blocks_kernel(const kvx_b
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const uint32_t w = cc[e >> 1] >> ((e & 1) * 16);
-        hi[e] = dequant_pair((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
-        lo[e] = dequant_pair(w & 0xf, (w >> 8) & 0xf, z, s);
+        hi[e] = dequant_pair<F16>((w >> 4) & 0xf, (w >> 12) & 0xf, z, s);
+        lo[e] = dequant_pair<F16>(w & 0xf, (w >> 8) & 0xf, z, s);
       }
       *chunk_ptr(c) = hi;
       *chunk_ptr(c + half) = lo;
@@ -428,33 +429,25 @@ __device__ __forceinline__ float row_norm(u32x4_t raw) {
   float ss = 0.0f;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    float a, b;
-    if constexpr (F16) {
-      const f16x2_t hv = __builtin_bit_cast(f16x2_t, (uint32_t)raw[e]);
-      a = (float)hv[0];
-      b = (float)hv[1];
-    } else {
-      a = bf16_lo(raw[e]);
-      b = bf16_hi(raw[e]);
-    }
+    const float a = elem_lo<F16>(raw[e]), b = elem_hi<F16>(raw[e]);
     ss += a * a;
     ss += b * b;
   }
   return sqrtf(row_sum<LPR>(ss));
 }
 
-// |x - dq(q(x))|_2 of a row: the dequantised value and the difference are rounded to bf16, the norm
+// |x - dq(q(x))|_2 of a row: the dequantised value and the difference are rounded to the rows' type, the norm
 // accumulates in fp32 (keys_values/kvcache/quantize/pytorch.py:530-548).
-template <int LPR>
+template <int LPR, bool F16>
 __device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, float scale, int32_t zp) {
   float ss = 0.0f;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const uint32_t cw = codes[e >> 1];
     const int sh = (e & 1) * 16;
-    const uint32_t dq = dequant_pair((cw >> sh) & 0xff, (cw >> (sh + 8)) & 0xff, zp, scale);
-    const uint32_t diff = pack_bf16(bf16_lo(raw[e]) - bf16_lo(dq), bf16_hi(raw[e]) - bf16_hi(dq));
-    const float a = bf16_lo(diff), b = bf16_hi(diff);
+    const uint32_t dq = dequant_pair<F16>((cw >> sh) & 0xff, (cw >> (sh + 8)) & 0xff, zp, scale);
+    const uint32_t diff = pack_pair<F16>(elem_lo<F16>(raw[e]) - elem_lo<F16>(dq), elem_hi<F16>(raw[e]) - elem_hi<F16>(dq));
+    const float a = elem_lo<F16>(diff), b = elem_hi<F16>(diff);
     ss += a * a;
     ss += b * b;
   }
@@ -469,7 +462,8 @@ __device__ __forceinline__ float row_quant_error(u32x4_t raw, u32x2_t codes, flo
 template <int D, int KV>
 __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_write_args a) {
   constexpr bool U8 = !kv_is_plain(KV);  // a quantised store: codes + row state
-  constexpr bool U4 = KV == KVX_KV_U4;    // two codes per byte: only the lanes of the first half of a row store
+  constexpr bool U4 = kv_is_u4(KV);       // two codes per byte: only the lanes of the first half of a row store
+  constexpr bool F16 = kv_elem_f16(KV);   // the rows are float16
   constexpr int LPR = D / 8;
   const int64_t gid = (int64_t)blockIdx.x * NTHREADS + threadIdx.x;
   const int col = (int)(gid % LPR);
@@ -505,9 +499,9 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
   auto put = [&](const u32x4_t& krow, const u32x4_t& vrow, int target, bool doit, bool want_err) -> float {
     float s1, s2, err = 0.0f;
     int32_t z1, z2;
-    u32x2_t kc = U4 ? quantize4<LPR>(krow, s1, z1) : quantize8<LPR>(krow, s1, z1);
-    u32x2_t vc = U4 ? quantize4<LPR>(vrow, s2, z2) : quantize8<LPR>(vrow, s2, z2);
-    if (want_err) err = row_quant_error<LPR>(krow, kc, s1, z1) + row_quant_error<LPR>(vrow, vc, s2, z2);  // uniform branch
+    u32x2_t kc = U4 ? quantize4<LPR, F16>(krow, s1, z1) : quantize8<LPR, F16>(krow, s1, z1);
+    u32x2_t vc = U4 ? quantize4<LPR, F16>(vrow, s2, z2) : quantize8<LPR, F16>(vrow, s2, z2);
+    if (want_err) err = row_quant_error<LPR, F16>(krow, kc, s1, z1) + row_quant_error<LPR, F16>(vrow, vc, s2, z2);  // uniform branch
     if constexpr (U4) {  // byte j = code[j] << 4 | code[j + D/2]: the partner lane holds the low nibbles
       kc = u32x2_t{(kc[0] << 4) | (uint32_t)__shfl_xor(kc[0], LPR / 2, 64), (kc[1] << 4) | (uint32_t)__shfl_xor(kc[1], LPR / 2, 64)};
       vc = u32x2_t{(vc[0] << 4) | (uint32_t)__shfl_xor(vc[0], LPR / 2, 64), (vc[1] << 4) | (uint32_t)__shfl_xor(vc[1], LPR / 2, 64)};
@@ -546,8 +540,8 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
           kq = u4_codes(kq, col < LPR / 2 ? 4 : 0);
           vq = u4_codes(vq, col < LPR / 2 ? 4 : 0);
         }
-        krow = dequant_words(kq[0], kq[1], a.k_zp[qs_row + ring], a.k_scale[qs_row + ring]);
-        vrow = dequant_words(vq[0], vq[1], a.v_zp[qs_row + ring], a.v_scale[qs_row + ring]);
+        krow = dequant_words<F16>(kq[0], kq[1], a.k_zp[qs_row + ring], a.k_scale[qs_row + ring]);
+        vrow = dequant_words<F16>(vq[0], vq[1], a.v_zp[qs_row + ring], a.v_scale[qs_row + ring]);
       }
       put(krow, vrow, slot, mv, false);
     }
@@ -569,7 +563,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
     qerr = put(kr, vr, wslot, ok, a.q_errors != nullptr);
   }
   float vnorm = 0.0f;
-  if (a.v_norm) vnorm = row_norm<LPR, KV == KVX_KV_F16>(vr);  // uniform branch: every lane takes part in the reduction
+  if (a.v_norm) vnorm = row_norm<LPR, F16>(vr);  // uniform branch: every lane takes part in the reduction
   if (live && col == 0 && a.replay_log) {  // the slot as consumed, valid or not: the log mirrors index
     const int64_t lp = a.log_pos + j;
     a.replay_log[(lp / a.log_blocksize) * a.log_stride_block + b * a.log_stride_b + hh * a.log_stride_h + lp % a.log_blocksize] =
@@ -585,64 +579,60 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
 
 }  // namespace
 
-int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale,
+// D in {64, 128}, bits in {8, 4}, f16: the rows are float16 (else bfloat16)
+template <int D, bool F16>
+int launch_quantize_rows_t(const void* x, int64_t x_row_stride, int64_t rows, int bits, uint8_t* codes, float* scale, int32_t* zp, hipStream_t st) {
+  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
+  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
+  if (bits == 8) hipLaunchKernelGGL((quantize_rows_kernel<D, F16>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  else hipLaunchKernelGGL((quantize_rows4_kernel<D, F16>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, int bits, bool f16, uint8_t* codes, float* scale,
                          int32_t* zp, hipStream_t st) {
   if (rows == 0) return KVX_OK;
-  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
-  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
-  if (D == 128)
-    hipLaunchKernelGGL((quantize_rows_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
-  else
-    hipLaunchKernelGGL((quantize_rows_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
+  if (D == 128) return f16 ? launch_quantize_rows_t<128, true>(x, x_row_stride, rows, bits, codes, scale, zp, st)
+                           : launch_quantize_rows_t<128, false>(x, x_row_stride, rows, bits, codes, scale, zp, st);
+  return f16 ? launch_quantize_rows_t<64, true>(x, x_row_stride, rows, bits, codes, scale, zp, st)
+             : launch_quantize_rows_t<64, false>(x, x_row_stride, rows, bits, codes, scale, zp, st);
+}
+
+template <int D, bool F16>
+int launch_dequantize_rows_t(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int bits, void* out,
+                             int64_t out_row_stride, hipStream_t st) {
+  if (bits == 8) {
+    const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
+    const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
+    hipLaunchKernelGGL((dequantize_rows_kernel<D, F16>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  } else {
+    const int64_t lanes = rows * (D / 16);
+    const unsigned grid = (unsigned)((lanes + NTHREADS - 1) / NTHREADS);
+    hipLaunchKernelGGL((dequantize_rows4_kernel<D, F16>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
+  }
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
 
-int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
-                           int64_t out_row_stride, hipStream_t st) {
+int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, int bits, bool f16,
+                           void* out, int64_t out_row_stride, hipStream_t st) {
   if (rows == 0) return KVX_OK;
-  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
-  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
-  if (D == 128)
-    hipLaunchKernelGGL((dequantize_rows_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
-  else
-    hipLaunchKernelGGL((dequantize_rows_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
-  KVX_HIP(hipGetLastError());
-  return KVX_OK;
-}
-
-int launch_quantize_rows4(const void* x, int64_t x_row_stride, int64_t rows, int D, uint8_t* codes, float* scale, int32_t* zp,
-                          hipStream_t st) {
-  if (rows == 0) return KVX_OK;
-  const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
-  const unsigned grid = (unsigned)((rows + rpb - 1) / rpb);
-  if (D == 128)
-    hipLaunchKernelGGL((quantize_rows4_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
-  else
-    hipLaunchKernelGGL((quantize_rows4_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, (const uint16_t*)x, x_row_stride, rows, codes, scale, zp);
-  KVX_HIP(hipGetLastError());
-  return KVX_OK;
-}
-
-int launch_dequantize_rows4(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, void* out,
-                            int64_t out_row_stride, hipStream_t st) {
-  if (rows == 0) return KVX_OK;
-  const int64_t lanes = rows * (D / 16);
-  const unsigned grid = (unsigned)((lanes + NTHREADS - 1) / NTHREADS);
-  if (D == 128)
-    hipLaunchKernelGGL((dequantize_rows4_kernel<128>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
-  else
-    hipLaunchKernelGGL((dequantize_rows4_kernel<64>), dim3(grid), dim3(NTHREADS), 0, st, codes, scale, zp, rows, (uint16_t*)out, out_row_stride);
-  KVX_HIP(hipGetLastError());
-  return KVX_OK;
+  if (D == 128) return f16 ? launch_dequantize_rows_t<128, true>(codes, scale, zp, rows, bits, out, out_row_stride, st)
+                           : launch_dequantize_rows_t<128, false>(codes, scale, zp, rows, bits, out, out_row_stride, st);
+  return f16 ? launch_dequantize_rows_t<64, true>(codes, scale, zp, rows, bits, out, out_row_stride, st)
+             : launch_dequantize_rows_t<64, false>(codes, scale, zp, rows, bits, out, out_row_stride, st);
 }
 
 int launch_quantize_blocks(const kvx_block_quant_args& a, hipStream_t st) {
   const int64_t blocks = (int64_t)a.n_outer * a.n_inner;
   if (blocks == 0) return KVX_OK;
   const unsigned grid = (unsigned)((blocks + NTHREADS / 64 - 1) / (NTHREADS / 64));
-  if (a.bits == 8) hipLaunchKernelGGL((quantize_blocks_kernel<8>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  else hipLaunchKernelGGL((quantize_blocks_kernel<4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  const bool f16 = a.elem_dtype == KVX_KV_F16;
+  if (a.bits == 8 && f16) hipLaunchKernelGGL((quantize_blocks_kernel<8, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else if (a.bits == 8) hipLaunchKernelGGL((quantize_blocks_kernel<8, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else if (f16) hipLaunchKernelGGL((quantize_blocks_kernel<4, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else hipLaunchKernelGGL((quantize_blocks_kernel<4, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
@@ -651,8 +641,28 @@ int launch_dequantize_blocks(const kvx_block_quant_args& a, hipStream_t st) {
   const int64_t blocks = (int64_t)a.n_outer * a.n_inner;
   if (blocks == 0) return KVX_OK;
   const unsigned grid = (unsigned)((blocks + NTHREADS / 64 - 1) / (NTHREADS / 64));
-  if (a.bits == 8) hipLaunchKernelGGL((dequantize_blocks_kernel<8>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  else hipLaunchKernelGGL((dequantize_blocks_kernel<4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  const bool f16 = a.elem_dtype == KVX_KV_F16;
+  if (a.bits == 8 && f16) hipLaunchKernelGGL((dequantize_blocks_kernel<8, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else if (a.bits == 8) hipLaunchKernelGGL((dequantize_blocks_kernel<8, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else if (f16) hipLaunchKernelGGL((dequantize_blocks_kernel<4, true>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else hipLaunchKernelGGL((dequantize_blocks_kernel<4, false>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  KVX_HIP(hipGetLastError());
+  return KVX_OK;
+}
+
+template <int D>
+int launch_cache_write_d(const kvx_cache_write_args& a, unsigned grid, hipStream_t st) {
+  switch (a.kv_dtype) {
+    case KVX_KV_F16: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
+    case KVX_KV_BF16: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
+    default:
+      if constexpr (D <= 128) {  // quantised stores: head sizes 64 and 128 (checked by the caller)
+        if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
+        else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
+        else if (a.kv_dtype == KVX_KV_U4_F16) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
+        else hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
+      }
+  }
   KVX_HIP(hipGetLastError());
   return KVX_OK;
 }
@@ -661,22 +671,9 @@ int launch_cache_write(const kvx_cache_write_args& a, hipStream_t st) {
   const int64_t total = (int64_t)a.B * a.Hkv * a.num * (a.D / 8);
   if (total == 0) return KVX_OK;
   const unsigned grid = (unsigned)((total + NTHREADS - 1) / NTHREADS);
-  if (a.D == 256) {  // plain rows only (checked by the caller)
-    if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<256, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else hipLaunchKernelGGL((cache_write_kernel<256, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  } else if (a.D == 128) {
-    if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else hipLaunchKernelGGL((cache_write_kernel<128, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  } else {
-    if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else if (a.kv_dtype == KVX_KV_F16) hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-    else hipLaunchKernelGGL((cache_write_kernel<64, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  }
-  KVX_HIP(hipGetLastError());
-  return KVX_OK;
+  if (a.D == 256) return launch_cache_write_d<256>(a, grid, st);
+  if (a.D == 128) return launch_cache_write_d<128>(a, grid, st);
+  return launch_cache_write_d<64>(a, grid, st);
 }
 
 }  // namespace kvx

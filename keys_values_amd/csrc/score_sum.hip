@@ -177,7 +177,7 @@ struct QLoader {
 template <int D, int KV, int W, bool QSPLIT>
 __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(const ScoreParams p) {
   constexpr int BK = NW * W;  // keys per workgroup
-  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q and k
+  constexpr bool F16 = kv_elem_f16(KV);  // element type of q and k
   __shared__ Smem<D> sm;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -211,13 +211,13 @@ __global__ __launch_bounds__(64 * W, D <= 128 ? 2 : 1) void score_sum_kernel(con
 #pragma unroll
       for (int j = 0; j < D / 16; ++j) {
         u32x2_t cc;
-        if constexpr (KV == KVX_KV_U4) {  // chunk 2j + h of the row: one nibble of 8 bytes
+        if constexpr (kv_is_u4(KV)) {  // chunk 2j + h of the row: one nibble of 8 bytes
           cc = ok ? *(const u32x2_t*)(kp + u4_byte_off<D>(2 * j + h)) : u32x2_t{0, 0};
           cc = u4_codes(cc, u4_shift<D>(2 * j + h));
         } else {
           cc = ok ? *(const u32x2_t*)(kp + 16 * j + 8 * h) : u32x2_t{0, 0};
         }
-        kf[nt][j] = dequant_words(cc[0], cc[1], zp, sc);
+        kf[nt][j] = dequant_words<F16>(cc[0], cc[1], zp, sc);
       }
     }
   }
@@ -499,15 +499,15 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   p.k_sb = a.k_stride_b; p.k_sh = a.k_stride_h; p.k_st = a.k_stride_t;
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
-  if (a.D == 128) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, pl.splits, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, pl.splits, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, pl.splits, st) : launch_t<128, KVX_KV_BF16>(p, pl.splits, st);
-  }
-  if (a.D == 64) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, pl.splits, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, pl.splits, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, pl.splits, st) : launch_t<64, KVX_KV_BF16>(p, pl.splits, st);
+  if (a.D == 128 || a.D == 64) {
+    switch (a.kv_dtype) {
+      case KVX_KV_BF16: return a.D == 128 ? launch_t<128, KVX_KV_BF16>(p, pl.splits, st) : launch_t<64, KVX_KV_BF16>(p, pl.splits, st);
+      case KVX_KV_F16: return a.D == 128 ? launch_t<128, KVX_KV_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_F16>(p, pl.splits, st);
+      case KVX_KV_U8: return a.D == 128 ? launch_t<128, KVX_KV_U8>(p, pl.splits, st) : launch_t<64, KVX_KV_U8>(p, pl.splits, st);
+      case KVX_KV_U4: return a.D == 128 ? launch_t<128, KVX_KV_U4>(p, pl.splits, st) : launch_t<64, KVX_KV_U4>(p, pl.splits, st);
+      case KVX_KV_U8_F16: return a.D == 128 ? launch_t<128, KVX_KV_U8_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_U8_F16>(p, pl.splits, st);
+      case KVX_KV_U4_F16: return a.D == 128 ? launch_t<128, KVX_KV_U4_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_U4_F16>(p, pl.splits, st);
+    }
   }
   if (a.D == 256 && kv_is_plain(a.kv_dtype))
     return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, pl.splits, st) : launch_t<256, KVX_KV_BF16>(p, pl.splits, st);

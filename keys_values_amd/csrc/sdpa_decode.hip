@@ -70,7 +70,6 @@ struct DecodeParams {
   int64_t q_sb, q_sh, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, qs_sb, qs_sh;
 };
 
-__device__ __forceinline__ u32x4_t dq8(uint32_t c0, uint32_t c1, int32_t zp, float scale) { return dequant_words(c0, c1, zp, scale); }
 
 // Sum over the LPR lanes that share a row. Every lane of the group ends with the same bits: each
 // step adds two values that the partner lane adds in the other order.
@@ -254,7 +253,7 @@ __device__ __forceinline__ void finish_split(const DecodeParams& p, const kvx_h2
 
 template <int D, int G, int KV>
 __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
-  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q, k, v, o
+  constexpr bool F16 = kv_elem_f16(KV);  // element type of q, k, v, o
   constexpr int LPR = D / 8;     // lanes per row: a lane owns 8 consecutive d
   constexpr int RPI = 64 / LPR;  // rows per load instruction of a wavefront
   constexpr int U = 4;           // load instructions per step and tensor (even: rows pair up for dot2)
@@ -280,15 +279,12 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 #pragma unroll
     for (int e = 0; e < 4; ++e) qv[g][e] = t[e];
   }
-  // Rows are addressed as a uniform base plus a 32-bit byte offset (the host checks the range).
-  constexpr bool U8 = !kv_is_plain(KV);  // codes + row state (8-bit or 4-bit store)
-  constexpr bool U4 = KV == KVX_KV_U4;
-  constexpr int ES = U8 ? 1 : 2;
-  const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
-  const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * ES;
-  const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES, lane_off = U4 ? u4_byte_off<D>(dc) : 8 * dc * ES;
-  const int nib = u4_shift<D>(dc);  // 4-bit store: which nibble holds this lane's 8 values
-  const int64_t qs_off = b * p.qs_sb + kvh * p.qs_sh;
+  // Rows are addressed as a uniform base plus a 32-bit byte offset (the host checks the range). Plain rows only:
+  // quantised stores take decode_mfma_kernel.
+  static_assert(kv_is_plain(KV), "plain 16-bit rows");
+  const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * 2;
+  const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * 2;
+  const uint32_t k_rowb = (uint32_t)p.k_st * 2, v_rowb = (uint32_t)p.v_st * 2, lane_off = 16 * dc;
   float* lgrow = p.logits ? p.logits + ((int64_t)b * p.Hkv + kvh) * p.Tpad * G : nullptr;
   int lg_base = k_begin;  // first key of the logits gathered in LDS
 
@@ -304,36 +300,18 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
 
   struct Rows {
     u32x4_t k[U], v[U];
-    float ks[U], vs[U];
-    int32_t kz[U], vz[U];
   };
   // Rows past the end re-read the last valid row; their logits become -inf below.
   auto issue = [&](Rows& r, int chunk0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(chunk0 + u * RPI + kk, k_end - 1);
-      if constexpr (!U8) {
-        r.k[u] = __builtin_nontemporal_load((const u32x4_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
-      } else {
-        u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
-        if constexpr (U4) c = u4_codes(c, nib);
-        r.k[u] = u32x4_t{c[0], c[1], 0, 0};
-        r.ks[u] = p.k_scale[qs_off + key];
-        r.kz[u] = p.k_zp[qs_off + key];
-      }
+      r.k[u] = __builtin_nontemporal_load((const u32x4_t*)(kbase + ((uint32_t)key * k_rowb + lane_off)));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(chunk0 + u * RPI + kk, k_end - 1);
-      if constexpr (!U8) {
-        r.v[u] = __builtin_nontemporal_load((const u32x4_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
-      } else {
-        u32x2_t c = __builtin_nontemporal_load((const u32x2_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
-        if constexpr (U4) c = u4_codes(c, nib);
-        r.v[u] = u32x4_t{c[0], c[1], 0, 0};
-        r.vs[u] = p.v_scale[qs_off + key];
-        r.vz[u] = p.v_zp[qs_off + key];
-      }
+      r.v[u] = __builtin_nontemporal_load((const u32x4_t*)(vbase + ((uint32_t)key * v_rowb + lane_off)));
     }
   };
   auto consume = [&](Rows& r, int chunk0) {
@@ -341,8 +319,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     float s[U][G];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      u32x4_t kx = r.k[u];
-      if constexpr (U8) kx = dq8(kx[0], kx[1], r.kz[u], r.ks[u]);
+      const u32x4_t kx = r.k[u];
       const bool valid = chunk0 + u * RPI + kk < k_end;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -399,11 +376,7 @@ __global__ __launch_bounds__(NTHREADS) void decode_split_kernel(const DecodePara
     // O += p V, two rows per dot2
 #pragma unroll
     for (int u = 0; u < U; u += 2) {
-      u32x4_t xa = r.v[u], xb = r.v[u + 1];
-      if constexpr (U8) {
-        xa = dq8(xa[0], xa[1], r.vz[u], r.vs[u]);
-        xb = dq8(xb[0], xb[1], r.vz[u + 1], r.vs[u + 1]);
-      }
+      const u32x4_t xa = r.v[u], xb = r.v[u + 1];
       uint32_t pg[G];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -496,16 +469,17 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c
   else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
-// bf16( (float)((int)code - zp) * scale ) for two codes with their own row state (two keys)
+// elem( (float)((int)code - zp) * scale ) for two codes with their own row state (two keys)
+template <bool F16>
 __device__ __forceinline__ uint32_t dequant_pair2(uint32_t c0, int32_t zp0, float sc0, uint32_t c1, int32_t zp1, float sc1) {
-  return pack_bf16((float)((int32_t)c0 - zp0) * sc0, (float)((int32_t)c1 - zp1) * sc1);
+  return pack_pair<F16>((float)((int32_t)c0 - zp0) * sc0, (float)((int32_t)c1 - zp1) * sc1);
 }
 
 template <int D, int G, int KV>
 __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
-  constexpr bool F16 = KV == KVX_KV_F16;
+  constexpr bool F16 = kv_elem_f16(KV);
   constexpr bool U8 = !kv_is_plain(KV);  // codes + row state (8-bit or 4-bit store)
-  constexpr bool U4 = KV == KVX_KV_U4;
+  constexpr bool U4 = kv_is_u4(KV);
   constexpr int KJ = D / 32;   // matrix instructions of the first product per 16-key tile
   constexpr int DPL = D / 16;  // d rows per lane = matrix instructions of the second product per 32-key block
   constexpr int CH = 32;       // keys per wavefront and step
@@ -662,7 +636,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
       return r.k[gi][e];
     } else if constexpr (!U4) {
       const u32x4_t w = r.k[gi][e >> 1];
-      return (e & 1) ? dequant_words(w[2], w[3], r.kz[gi], r.ks[gi]) : dequant_words(w[0], w[1], r.kz[gi], r.ks[gi]);
+      return (e & 1) ? dequant_words<F16>(w[2], w[3], r.kz[gi], r.ks[gi]) : dequant_words<F16>(w[0], w[1], r.kz[gi], r.ks[gi]);
     } else {
       const u32x4_t w = r.k[gi][0];
       u32x2_t bytes;
@@ -675,7 +649,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
         shift = e ? 0 : 4;
       }
       const u32x2_t c = u4_codes(bytes, shift);
-      return dequant_words(c[0], c[1], r.kz[gi], r.ks[gi]);
+      return dequant_words<F16>(c[0], c[1], r.kz[gi], r.ks[gi]);
     }
   };
   // A operand t of the second product: value t of each of this lane's 8 keys, in key order
@@ -696,7 +670,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
           c0 = (r.v[j0][0] >> sh) & 0xfu;
           c1 = (r.v[j1][0] >> sh) & 0xfu;
         }
-        a[jj] = dequant_pair2(c0, r.vz[j0], r.vs[j0], c1, r.vz[j1], r.vs[j1]);
+        a[jj] = dequant_pair2<F16>(c0, r.vz[j0], r.vs[j0], c1, r.vz[j1], r.vs[j1]);
       }
     }
     return a;
@@ -1092,6 +1066,8 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
   if constexpr (D <= 128) {
     if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (kv == KVX_KV_U4_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U4_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if (kv == KVX_KV_U8_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U8_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (G >= 8 && kv == KVX_KV_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (G >= 8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
   }
@@ -1102,7 +1078,7 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
     }
   }
   KVX_HIP(hipGetLastError());
-  return kv == KVX_KV_F16 ? launch_tail<D, true, G>(p, hh, st) : launch_tail<D, false, G>(p, hh, st);
+  return kv_elem_f16(kv) ? launch_tail<D, true, G>(p, hh, st) : launch_tail<D, false, G>(p, hh, st);
 }
 
 template <int D>

@@ -87,8 +87,6 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(lds_ptr_t p) {
   return __builtin_bit_cast(u32x2_t, t);
 }
 
-// 8 codes (two dwords) -> 8 bf16 (four dwords)
-__device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp, float scale) { return dequant_words(c0, c1, zp, scale); }
 
 // Tile loader. A wavefront instruction covers RPW = 64 / CPR whole rows; wavefront w of the
 // workgroup takes row groups w, w + 4, ... of the 64-row tile (NI groups each for K and for V).
@@ -97,7 +95,7 @@ __device__ __forceinline__ u32x4_t dequant8(uint32_t c0, uint32_t c1, int32_t zp
 template <int D, int KV>
 struct Loader {
   static constexpr bool U8 = !kv_is_plain(KV);  // codes through registers (8-bit or 4-bit store)
-  static constexpr bool U4 = KV == KVX_KV_U4;
+  static constexpr bool U4 = kv_is_u4(KV);
   static constexpr int CPR = D / 8;
   static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
   static constexpr int NWAVES = nwaves(KV);
@@ -267,8 +265,8 @@ struct Loader {
         const int r = row_of(i);
         u32x2_t c = IS_K ? kc[i] : vc[i];
         if constexpr (U4) c = u4_codes(c, IS_K ? shk : shv);
-        if (IS_K) sm.k[buf][r][lane % CPR] = dequant8(c[0], c[1], kzr[i], ksr[i]);
-        else sm.v[buf][r][lane % CPR] = dequant8(c[0], c[1], vzr[i], vsr[i]);
+        if (IS_K) sm.k[buf][r][lane % CPR] = dequant_words<kv_elem_f16(KV)>(c[0], c[1], kzr[i], ksr[i]);
+        else sm.v[buf][r][lane % CPR] = dequant_words<kv_elem_f16(KV)>(c[0], c[1], vzr[i], vsr[i]);
       }
     }
     if (IS_K && tid < BN) {
@@ -281,7 +279,7 @@ struct Loader {
 
 template <int D, int KV>
 __global__ __launch_bounds__(64 * nwaves(KV), (kv_is_plain(KV) && D <= 128) ? 2 : 1) void sdpa_prefill_kernel(const PrefillParams p) {
-  constexpr bool F16 = KV == KVX_KV_F16;  // element type of q, k, v, o
+  constexpr bool F16 = kv_elem_f16(KV);  // element type of q, k, v, o
   constexpr int BM = 32 * nwaves(KV);  // rows per workgroup
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;  // k-steps of the first product
@@ -705,7 +703,7 @@ int launch_t(PrefillParams& p, hipStream_t st) {
   if (p.num_splits > 1) {
     constexpr int ROWS = 256 / (D / 4);
     const int64_t total_rows = (int64_t)p.B * p.Hkv * p.R;
-    hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D, KV == KVX_KV_F16>), dim3((unsigned)((total_rows + ROWS - 1) / ROWS)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D, kv_elem_f16(KV)>), dim3((unsigned)((total_rows + ROWS - 1) / ROWS)), dim3(256), 0, st, p);
     KVX_HIP(hipGetLastError());
   }
   return KVX_OK;
@@ -732,15 +730,15 @@ int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {
     p.part_o = (float*)a.workspace;
     p.part_ml = p.part_o + rows * (size_t)a.D;
   }
-  if (a.D == 128) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<128, KVX_KV_U4>(p, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<128, KVX_KV_F16>(p, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<128, KVX_KV_BF16>(p, st);
-  }
-  if (a.D == 64) {
-    if (a.kv_dtype == KVX_KV_U4) return launch_t<64, KVX_KV_U4>(p, st);
-    if (a.kv_dtype == KVX_KV_F16) return launch_t<64, KVX_KV_F16>(p, st);
-    return a.kv_dtype == KVX_KV_U8 ? launch_t<64, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
+  if (a.D == 128 || a.D == 64) {
+    switch (a.kv_dtype) {
+      case KVX_KV_BF16: return a.D == 128 ? launch_t<128, KVX_KV_BF16>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
+      case KVX_KV_F16: return a.D == 128 ? launch_t<128, KVX_KV_F16>(p, st) : launch_t<64, KVX_KV_F16>(p, st);
+      case KVX_KV_U8: return a.D == 128 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_U8>(p, st);
+      case KVX_KV_U4: return a.D == 128 ? launch_t<128, KVX_KV_U4>(p, st) : launch_t<64, KVX_KV_U4>(p, st);
+      case KVX_KV_U8_F16: return a.D == 128 ? launch_t<128, KVX_KV_U8_F16>(p, st) : launch_t<64, KVX_KV_U8_F16>(p, st);
+      case KVX_KV_U4_F16: return a.D == 128 ? launch_t<128, KVX_KV_U4_F16>(p, st) : launch_t<64, KVX_KV_U4_F16>(p, st);
+    }
   }
   if (a.D == 256 && kv_is_plain(a.kv_dtype))
     return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, st) : launch_t<256, KVX_KV_BF16>(p, st);

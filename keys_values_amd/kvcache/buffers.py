@@ -67,9 +67,9 @@ class QuantizedKeysAndValues(KeysAndValues):
 
     def _dequantize(self, codes, scale, zp) -> torch.Tensor:
         b, h, t, _ = codes.shape
-        out = torch.empty((b, h, t, self.head_size), dtype=torch.bfloat16, device=codes.device)
+        out = torch.empty((b, h, t, self.head_size), dtype=self.dtype, device=codes.device)
         _dequantize_rows(codes, scale, zp, out, self.num_bits)
-        return out if self.dtype == torch.bfloat16 else out.to(self.dtype)
+        return out
 
     def keys(self) -> torch.Tensor:
         return self._dequantize(self.key_codes, self.quant.k_scale, self.quant.k_zp)
@@ -82,7 +82,11 @@ def _dequantize_rows(codes, scale, zp, out, num_bits: int):
     """codes (b, h, t, row bytes) strided over t only at the slot axis, state (b, h, t), out (b, h, t, D)
     contiguous: one launch per (b, h) run of contiguous slots."""
     lib = _lib.load()
-    fn = lib.kvx_dequantize_rows4 if num_bits == 4 else lib.kvx_dequantize_rows
+    elem = _lib.elem_kv_dtype(out.dtype)
+
+    def fn(c, s, z, rows, dd, o, stride, stream):  # the rows dequantise to the type of `out`
+        return lib.kvx_dequantize_rows_typed(c, s, z, rows, dd, num_bits, elem, o, stride, stream)
+
     b, h, t, row = codes.shape
     d = out.shape[-1]
     dev = codes.device
@@ -181,8 +185,6 @@ class HipKVCacheBuffers(KVCacheBuffers):
             raise NotImplementedError(f"head_size = {params.head_size} not in {sizes}")
         if self.dtype is not None and self.dtype not in (torch.bfloat16, torch.float16):
             raise NotImplementedError(f"dtype {self.dtype}: the kernels take bfloat16 or float16 rows")
-        if num_bits is not None and self.dtype not in (None, torch.bfloat16):
-            raise NotImplementedError("the quantised store dequantises to bfloat16")
         self.num_bits = num_bits
         self.k = self.v = None
         self.k_scale = self.k_zp = self.v_scale = self.v_zp = None
@@ -214,7 +216,7 @@ class HipKVCacheBuffers(KVCacheBuffers):
         if device.type != "cuda":
             raise RuntimeError(f"HipKVCacheBuffers live on a ROCm device, not on {device}: there is no CPU path")
         if self.dtype is None:
-            if dtype not in (torch.bfloat16, torch.float16) or (self.quantized and dtype != torch.bfloat16):
+            if dtype not in (torch.bfloat16, torch.float16):
                 raise NotImplementedError(f"dtype {dtype} is not served by this store")
             self.dtype = dtype
         batch_size = self.batch_size
@@ -281,7 +283,7 @@ class HipKVCacheBuffers(KVCacheBuffers):
             value = value.contiguous()
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, d, self.cache_length
-        a.kv_dtype = {None: _lib.KVX_KV_F16 if self.dtype == torch.float16 else _lib.KVX_KV_BF16, 8: _lib.KVX_KV_U8, 4: _lib.KVX_KV_U4}[self.num_bits]
+        a.kv_dtype = _lib.elem_kv_dtype(self.dtype) if self.num_bits is None else _lib.quant_kv_dtype(self.num_bits, self.dtype)
         a.index, a.index_stride_b, a.index_stride_h = index.data_ptr(), index.stride(0), index.stride(1)
         a.key, a.key_stride_b, a.key_stride_h, a.key_stride_t = key.data_ptr(), key.stride(0), key.stride(1), key.stride(2)
         a.value, a.value_stride_b, a.value_stride_h, a.value_stride_t = value.data_ptr(), value.stride(0), value.stride(1), value.stride(2)

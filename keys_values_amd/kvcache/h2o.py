@@ -54,15 +54,16 @@ DEFAULT_DEQUANTIZE_CHUNK_ROWS = 2048
 _dequant_buffers = {}
 
 
-def _dequant_scratch(device, numel: int):
-    """Two bf16 buffers of ``numel`` elements, grow-only, shared by the caches of one device and stream
-    (launches on a stream are ordered: a layer's attention has read them before the next layer's
+def _dequant_scratch(device, numel: int, dtype: torch.dtype = torch.bfloat16):
+    """Two 16-bit buffers of ``numel`` elements of ``dtype``, grow-only, shared by the caches of one device and
+    stream (launches on a stream are ordered: a layer's attention has read them before the next layer's
     dequantisation overwrites them)."""
     key = (str(device), torch.cuda.current_stream(device).cuda_stream)
     buf = _dequant_buffers.get(key)
     if buf is None or buf.numel() < 2 * numel:
-        buf = torch.empty(2 * numel, dtype=torch.bfloat16, device=device)
+        buf = torch.empty(2 * numel, dtype=torch.int16, device=device)
         _dequant_buffers[key] = buf
+    buf = buf.view(dtype)
     return buf[:numel], buf[numel : 2 * numel]
 
 
@@ -126,8 +127,6 @@ class H2OKVCache:
             raise ValueError(f"combination_constant = {combination_constant}, must be in [0, 1]")
         if params.dtype not in (None, torch.bfloat16, torch.float16):
             raise NotImplementedError(f"cache dtype {params.dtype}: the kernels take bfloat16 or float16")
-        if quantized and params.dtype == torch.float16:
-            raise NotImplementedError("the quantised stores dequantise to bfloat16")
         if params.head_size not in (ops.QUANTIZED_HEAD_SIZES if quantized else ops.ALLOWED_HEAD_SIZES):
             raise NotImplementedError(f"head_size = {params.head_size} not in {ops.QUANTIZED_HEAD_SIZES if quantized else ops.ALLOWED_HEAD_SIZES}")
         if params.n_head % params.n_query_groups != 0:
@@ -408,9 +407,13 @@ class H2OKVCache:
         scratch by one launch per tensor (all slots of the first ``b`` batch entries: they are contiguous)."""
         h, length, d = self.n_query_groups, self.cache_length, self.head_size
         rows = b * h * length
-        kd, vd = _dequant_scratch(self.device, rows * d)
+        kd, vd = _dequant_scratch(self.device, rows * d, self.dtype)
         lib = _lib.load()
-        fn = lib.kvx_dequantize_rows4 if self.num_bits == 4 else lib.kvx_dequantize_rows
+        bits, elem = self.num_bits, _lib.elem_kv_dtype(self.dtype)
+
+        def fn(c, s, z, n, dd, o, stride, stream):
+            return lib.kvx_dequantize_rows_typed(c, s, z, n, dd, bits, elem, o, stride, stream)
+
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
             if b == self.max_batch_size:  # K and V are adjacent in the store and in the scratch: one launch
@@ -457,8 +460,7 @@ class H2OKVCache:
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, self.head_size, self.cache_length
         a.input_pos = input_pos
-        a.kv_dtype = ((_lib.KVX_KV_U4 if self.num_bits == 4 else _lib.KVX_KV_U8) if self.quantized
-                      else (_lib.KVX_KV_F16 if self.dtype == torch.float16 else _lib.KVX_KV_BF16))
+        a.kv_dtype = _lib.quant_kv_dtype(self.num_bits, self.dtype) if self.quantized else _lib.elem_kv_dtype(self.dtype)
         a.index = index.data_ptr()
         a.index_stride_b, a.index_stride_h = index.stride(0), index.stride(1)
         a.key = key.data_ptr()

@@ -34,8 +34,8 @@ class RowQuantizer:
             raise ValueError(f"shape = {shape}, must be 4D and all positive")
         if num_bits not in (4, 8):  # keys_values/kvcache/quantize/pytorch.py:191-192
             raise ValueError(f"num_bits = {num_bits}, must be 4 or 8")
-        if source_dtype != torch.bfloat16:
-            raise NotImplementedError(f"source_dtype = {source_dtype}: the kernels take bfloat16 rows")
+        if source_dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"source_dtype = {source_dtype}: the kernels take bfloat16 or float16 rows")
         if shape[3] % 16 != 0:
             raise NotImplementedError(f"head_size = {shape[3]} must be a multiple of 16")
         self.shape = tuple(shape)
@@ -107,7 +107,7 @@ class RowQuantizer:
         else:  # block (b * Hkv + h, t)
             a.n_outer, a.n_inner, a.nseg = b * hkv, num, 1
             a.x_stride_outer, a.x_stride_inner, a.x_stride_seg = x.stride(1), x.stride(2), 0
-        a.D, a.bits = d, self.num_bits
+        a.D, a.bits, a.elem_dtype = d, self.num_bits, _lib.elem_kv_dtype(self.source_dtype)
         a.codes = buffer[0, start].data_ptr()
         a.codes_stride_outer = buffer.stride(0)
         a.scale, a.zp = scales[0, start:].data_ptr(), zps[0, start:].data_ptr()
@@ -143,9 +143,9 @@ class RowQuantizer:
             st = _lib.stream_ptr(dev)
             if not self.blocks_over_heads and d in (64, 128) and start == 0 and end == length and values.is_contiguous():
                 # the whole store in one pass of the row kernels (16 or 8 lanes per row)
-                fn = lib.kvx_quantize_rows if self.num_bits == 8 else lib.kvx_quantize_rows4
-                _lib.check(fn(values.data_ptr(), d, b * hkv * length, d, self.quant_buffer.data_ptr(),
-                              self.quant_scales.data_ptr(), self.quant_zero_points.data_ptr(), st))
+                _lib.check(lib.kvx_quantize_rows_typed(values.data_ptr(), d, b * hkv * length, d, self.num_bits,
+                                                       _lib.elem_kv_dtype(self.source_dtype), self.quant_buffer.data_ptr(),
+                                                       self.quant_scales.data_ptr(), self.quant_zero_points.data_ptr(), st))
                 return
             x = self._kernel_view(values)
             a = self._block_args(x, start, self.quant_buffer, self.quant_scales, self.quant_zero_points)

@@ -55,6 +55,31 @@ def test_quantize_rows_bit_exact(kvx, gpu, rows, D):
     assert torch.equal(out.cpu(), O.dequantize_rows(c_ref, s_ref, z_ref, torch.bfloat16)), "dequantised rows differ"
 
 
+@pytest.mark.parametrize("bits,rows,D", [(8, 1000, 128), (8, 77, 64), (4, 1000, 128), (4, 5, 64)])
+def test_quantize_rows_of_float16_bit_exact(kvx, gpu, bits, rows, D):
+    """The typed entry points on float16 rows (a float16 model's store): the quantiser upcasts to fp32 and casts the
+    dequantised values back to the rows' type (keys_values/kvcache/quantize/pytorch.py:333,478)."""
+    x = outlier_rows(5, rows, D).to(torch.float16)
+    x[0] = 0.0
+    x[1] = -3.5
+    x[2] = torch.linspace(100.0, 101.0, D).to(torch.float16)
+    c_ref, s_ref, z_ref = O.quantize_rows(x, bits)
+    xg = x.to(gpu)
+    st = _lib.stream_ptr(gpu)
+    codes = torch.empty((rows, D * bits // 8), dtype=torch.uint8, device=gpu)
+    sc = torch.empty(rows, dtype=torch.float32, device=gpu)
+    zp = torch.empty(rows, dtype=torch.int32, device=gpu)
+    _lib.check(kvx.kvx_quantize_rows_typed(xg.data_ptr(), D, rows, D, bits, _lib.KVX_KV_F16, codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), st))
+    out = torch.empty((rows, D), dtype=torch.float16, device=gpu)
+    _lib.check(kvx.kvx_dequantize_rows_typed(codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), rows, D, bits, _lib.KVX_KV_F16, out.data_ptr(), D, st))
+    torch.cuda.synchronize()
+    assert torch.equal(sc.cpu(), s_ref) and torch.equal(zp.cpu(), z_ref), "row state differs"
+    assert torch.equal(codes.cpu(), O.compress4(c_ref) if bits == 4 else c_ref), "codes differ"
+    assert torch.equal(out.cpu(), O.dequantize_rows(c_ref, s_ref, z_ref, torch.float16)), "dequantised rows differ"
+    with pytest.raises(NotImplementedError):
+        _lib.check(kvx.kvx_quantize_rows_typed(xg.data_ptr(), D, rows, D, bits, _lib.KVX_KV_U8, codes.data_ptr(), sc.data_ptr(), zp.data_ptr(), st))
+
+
 @pytest.mark.parametrize("bits", [8, 4])
 def test_quantize_row_with_nan(kvx, gpu, bits):
     """torch.aminmax gives NaN extremes for a row that holds a NaN (keys_values/kvcache/quantize/pytorch.py:90),
@@ -309,8 +334,8 @@ def _sets_equal_away_from_ties(n_gpu, n_ref, scores_ref, k):
                 ), f"selection differs away from a tie at ({b},{h}): {sorted(diff)}"
 
 
-@pytest.mark.parametrize("quantized", [False, True])
-def test_h2o_cache_steps_vs_oracle(gpu, quantized):
+@pytest.mark.parametrize("quantized,dtype,bits", [(False, torch.bfloat16, 8), (True, torch.bfloat16, 8), (True, torch.float16, 8), (True, torch.float16, 4)])
+def test_h2o_cache_steps_vs_oracle(gpu, quantized, dtype, bits):
     """Prefill that fills the cache, then chunked steps: initial rule, evict-write, attention with
     scattered positions, score accumulation, selection (configuration 1 shapes: 8/2 heads, D 64,
     1024 slots, 128-token chunks). With the uint8 store every row is quantised once, when written,
@@ -319,13 +344,14 @@ def test_h2o_cache_steps_vs_oracle(gpu, quantized):
     B, Hq, Hkv, L, D, chunk = 1, 8, 2, 1024, 64, 128
     gen = torch.Generator().manual_seed(0)
     total = L + 4 * chunk
-    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
-    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
-    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
-    ks_o = O.dequantize_rows(*O.quantize_rows(ks)) if quantized else ks
-    vs_o = O.dequantize_rows(*O.quantize_rows(vs)) if quantized else vs
-    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=torch.bfloat16, max_chunk_size=chunk)
-    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, quantized=quantized, device=gpu)
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(dtype)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(dtype)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(dtype)
+    ks_o = O.dequantize_rows(*O.quantize_rows(ks, bits), dtype) if quantized else ks
+    vs_o = O.dequantize_rows(*O.quantize_rows(vs, bits), dtype) if quantized else vs
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=dtype, max_chunk_size=chunk)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq, dtype), max_chunk_size=chunk, quantized=quantized, num_bits=bits, device=gpu)
+    codes_of = O.uncompress4 if bits == 4 else (lambda c: c)
     ref.prefill(qs[:, :, :L], ks_o[:, :, :L], vs_o[:, :, :L])
     # the first chunk attends over the keys/values as given, not over the store (kvcache/base.py:567-571)
     o_ref, _ = O.sdpa_in_blocks(qs[:, :, :L], ks[:, :, :L], vs[:, :, :L], 1 / math.sqrt(D), 0, None, return_attn_weights=False)
@@ -347,12 +373,25 @@ def test_h2o_cache_steps_vs_oracle(gpu, quantized):
         assert rel_err(o.float().cpu().view(B, chunk, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
         torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
         if quantized:
-            assert torch.equal(O.dequantize_rows(cache.k.cpu(), cache.k_scale.cpu(), cache.k_zp.cpu()), ref.k)
-            assert torch.equal(O.dequantize_rows(cache.v.cpu(), cache.v_scale.cpu(), cache.v_zp.cpu()), ref.v)
+            assert torch.equal(O.dequantize_rows(codes_of(cache.k.cpu()), cache.k_scale.cpu(), cache.k_zp.cpu(), dtype), ref.k)
+            assert torch.equal(O.dequantize_rows(codes_of(cache.v.cpu()), cache.v_scale.cpu(), cache.v_zp.cpu(), dtype), ref.v)
         else:
             assert torch.equal(cache.k.cpu(), ref.k) and torch.equal(cache.v.cpu(), ref.v)
         _sets_equal_away_from_ties(cache._next_index[:B].cpu().long(), ref.next_index, ref.scores, chunk)
         pos += chunk
+    if quantized:  # single-token steps over the quantised store (the fused decode + H2O call)
+        extra = torch.Generator().manual_seed(99)
+        for _ in range(3):
+            q1 = torch.randn(B, Hq, 1, D, generator=extra).to(dtype)
+            k1 = torch.randn(B, Hkv, 1, D, generator=extra).to(dtype)
+            v1 = torch.randn(B, Hkv, 1, D, generator=extra).to(dtype)
+            k1o, v1o = O.dequantize_rows(*O.quantize_rows(k1, bits), dtype), O.dequantize_rows(*O.quantize_rows(v1, bits), dtype)
+            o_ref, w_ref, index = ref.forward(q1, k1o, v1o)
+            cache.set_next_positions(index)
+            o = cache.forward(q1.to(gpu), k1.to(gpu), v1.to(gpu))
+            assert o.dtype == dtype
+            assert rel_err(o.float().cpu().view(B, 1, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+            torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(8, 2), (6, 2), (7, 1)])

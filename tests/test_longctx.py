@@ -329,7 +329,7 @@ def test_swiglu_kernel(gpu, rows, dim):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("B,num,Hq,Hkv,D,norm,input_pos", [(1, 64, 8, 2, 64, True, 0), (2, 100, 32, 8, 128, True, 4000), (1, 33, 4, 4, 128, False, 77)])
+@pytest.mark.parametrize("B,num,Hq,Hkv,D,norm,input_pos", [(1, 64, 8, 2, 64, True, 0), (2, 100, 32, 8, 128, True, 4000), (1, 33, 4, 4, 128, False, 77), (2, 19, 4, 2, 256, True, 300)])
 def test_qk_norm_rope_kernel(gpu, B, num, Hq, Hkv, D, norm, input_pos):
     from keys_values_amd.longctx import ops
 
