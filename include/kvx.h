@@ -11,7 +11,7 @@
  *
  * Conventions
  *   B      batch size                 Hq     query heads          Hkv   key/value heads
- *   G      Hq / Hkv (group size)      D      head size (64, 128 or 256; quantised stores: 64 or 128)
+ *   G      Hq / Hkv (group size)      D      head size (64, 128 or 256)
  *   q_len  queries per call           kv_len cache slots visible to the call
  *   Tensors are addressed as base + b*stride_b + h*stride_h + t*stride_t + d with the head
  *   dimension contiguous; strides are in ELEMENTS of the tensor's own type. This covers both the
@@ -191,7 +191,7 @@ void kvx_decode_tuning(int resident, int spin_limit, int poll_sleep);
  * bit-for-bit as TorchBasicQuantizer._quantize with MyPerChannelMinMaxObserver._calculate_qparams and
  * quantize_per_channel (keys_values/kvcache/quantize/pytorch.py:100-139,312-355).
  * x: bf16, `rows` rows of D elements, row r at x + r*x_row_stride. codes: uint8 rows*D contiguous.
- * scale / zp: one per row, contiguous. D in {64, 128}. */
+ * scale / zp: one per row, contiguous. D in {64, 128, 256}. */
 int kvx_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int32_t D,
                       uint8_t* codes, float* scale, int32_t* zp, void* stream);
 

@@ -22,7 +22,7 @@ import torch
 from .. import _lib
 
 ALLOWED_HEAD_SIZES = (64, 128, 256)  # keys_values/attention/flashinfer_wrapper.py:276
-QUANTIZED_HEAD_SIZES = (64, 128)    # the kernels that read codes
+QUANTIZED_HEAD_SIZES = ALLOWED_HEAD_SIZES  # the kernels that read codes take the same sizes
 ALLOWED_DTYPES = (torch.bfloat16, torch.float16)  # keys_values/attention/flashinfer_wrapper.py:311-319
 
 

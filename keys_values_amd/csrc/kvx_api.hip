@@ -53,8 +53,7 @@ int check_sdpa_common(const kvx_sdpa_args* a, const char* who, bool need_v_o) {
   KVX_REQUIRE(a->B <= 65535 && a->Hq <= 65535 && (int64_t)a->B * a->Hq < ((int64_t)1 << 24), KVX_ERR_UNSUPPORTED,
               "%s: B=%d, Hq=%d beyond 65535 each or 2^24 together", who, a->B, a->Hq);
   KVX_REQUIRE(kv_valid(a->kv_dtype), KVX_ERR_UNSUPPORTED, "%s: unknown kv_dtype %d", who, a->kv_dtype);
-  KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
-              "%s: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", who, a->D);
+  KVX_REQUIRE(a->D == 64 || a->D == 128 || a->D == 256, KVX_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128, 256}", who, a->D);
   const int row_elems = kv_is_u4(a->kv_dtype) ? a->D / 2 : a->D;  // elements of the cache's own type per row
   KVX_REQUIRE(a->input_pos >= 0, KVX_ERR_INVALID, "%s: input_pos=%d must be >= 0", who, a->input_pos);
   KVX_REQUIRE(a->sm_scale > 0.0f, KVX_ERR_INVALID, "%s: sm_scale must be positive", who);
@@ -175,7 +174,7 @@ int kvx_sdpa_decode(const kvx_sdpa_args* a, void* stream) {
 
 static int quantize_rows_checked(const char* who, const void* x, int64_t x_row_stride, int64_t rows, int32_t D, int32_t bits, int32_t elem_dtype,
                                  uint8_t* codes, float* scale, int32_t* zp, void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128}", who, D);
+  KVX_REQUIRE(D == 64 || D == 128 || D == 256, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128, 256}", who, D);
   KVX_REQUIRE(bits == 8 || bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, bits);
   KVX_REQUIRE(elem_dtype == KVX_KV_BF16 || elem_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED, "%s: elem_dtype %d is neither KVX_KV_BF16 nor KVX_KV_F16", who, elem_dtype);
   KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "%s: rows must be >= 0", who);
@@ -189,7 +188,7 @@ static int quantize_rows_checked(const char* who, const void* x, int64_t x_row_s
 
 static int dequantize_rows_checked(const char* who, const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int32_t D, int32_t bits,
                                    int32_t elem_dtype, void* out, int64_t out_row_stride, void* stream) {
-  KVX_REQUIRE(D == 64 || D == 128, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128}", who, D);
+  KVX_REQUIRE(D == 64 || D == 128 || D == 256, KVX_ERR_UNSUPPORTED, "%s: row length %d not in {64, 128, 256}", who, D);
   KVX_REQUIRE(bits == 8 || bits == 4, KVX_ERR_UNSUPPORTED, "%s: bits = %d, must be 4 or 8", who, bits);
   KVX_REQUIRE(elem_dtype == KVX_KV_BF16 || elem_dtype == KVX_KV_F16, KVX_ERR_UNSUPPORTED, "%s: elem_dtype %d is neither KVX_KV_BF16 nor KVX_KV_F16", who, elem_dtype);
   KVX_REQUIRE(rows >= 0, KVX_ERR_INVALID, "%s: rows must be >= 0", who);
@@ -258,8 +257,7 @@ int kvx_cache_write(const kvx_cache_write_args* a, void* stream) {
   KVX_REQUIRE(a != nullptr, KVX_ERR_INVALID, "kvx_cache_write: args is NULL");
   KVX_REQUIRE(a->B > 0 && a->Hkv > 0 && a->num > 0 && a->cache_len > 0, KVX_ERR_INVALID, "kvx_cache_write: sizes must be positive");
   KVX_REQUIRE(kv_valid(a->kv_dtype), KVX_ERR_UNSUPPORTED, "kvx_cache_write: unknown kv_dtype %d", a->kv_dtype);
-  KVX_REQUIRE(a->D == 64 || a->D == 128 || (a->D == 256 && kv_is_plain(a->kv_dtype)), KVX_ERR_UNSUPPORTED,
-              "kvx_cache_write: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a->D);
+  KVX_REQUIRE(a->D == 64 || a->D == 128 || a->D == 256, KVX_ERR_UNSUPPORTED, "kvx_cache_write: head size %d not in {64, 128, 256}", a->D);
   KVX_REQUIRE(a->num <= a->cache_len, KVX_ERR_INVALID, "kvx_cache_write: num=%d exceeds cache_len=%d", a->num, a->cache_len);
   KVX_REQUIRE(a->index && a->key && a->value && a->k_cache && a->v_cache, KVX_ERR_INVALID, "kvx_cache_write: NULL pointer");
   KVX_REQUIRE(a->token_pos || a->grace_num == 0, KVX_ERR_INVALID, "kvx_cache_write: the ring move needs token_pos");

@@ -15,14 +15,15 @@ namespace {
 constexpr int NTHREADS = 256;
 constexpr int ROWS_PER_THREAD = 4;  // independent rows in flight per lane
 
-// Reductions over the LPR (8 or 16) adjacent lanes holding one row; every lane gets the result.
+// Reductions over the LPR (8, 16 or 32) adjacent lanes holding one row; every lane gets the result.
 template <int LPR>
 __device__ __forceinline__ float row_max(float v) {
   v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)));   // quad_perm [1,0,3,2]
   v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)));   // quad_perm [2,3,0,1]
   v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)));  // row_half_mirror
-  if constexpr (LPR == 16)
+  if constexpr (LPR >= 16)
     v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)));  // row_mirror
+  if constexpr (LPR == 32) v = fmaxf(v, __shfl_xor(v, 16, 64));  // the other DPP row of the group
   return v;
 }
 template <int LPR>
@@ -30,8 +31,9 @@ __device__ __forceinline__ float row_min(float v) {
   v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)));
   v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)));
   v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)));
-  if constexpr (LPR == 16)
+  if constexpr (LPR >= 16)
     v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)));
+  if constexpr (LPR == 32) v = fminf(v, __shfl_xor(v, 16, 64));
   return v;
 }
 
@@ -579,7 +581,7 @@ __global__ __launch_bounds__(NTHREADS) void cache_write_kernel(const kvx_cache_w
 
 }  // namespace
 
-// D in {64, 128}, bits in {8, 4}, f16: the rows are float16 (else bfloat16)
+// D in {64, 128, 256}, bits in {8, 4}, f16: the rows are float16 (else bfloat16)
 template <int D, bool F16>
 int launch_quantize_rows_t(const void* x, int64_t x_row_stride, int64_t rows, int bits, uint8_t* codes, float* scale, int32_t* zp, hipStream_t st) {
   const int rpb = (NTHREADS / (D / 8)) * ROWS_PER_THREAD;
@@ -593,6 +595,8 @@ int launch_quantize_rows_t(const void* x, int64_t x_row_stride, int64_t rows, in
 int launch_quantize_rows(const void* x, int64_t x_row_stride, int64_t rows, int D, int bits, bool f16, uint8_t* codes, float* scale,
                          int32_t* zp, hipStream_t st) {
   if (rows == 0) return KVX_OK;
+  if (D == 256) return f16 ? launch_quantize_rows_t<256, true>(x, x_row_stride, rows, bits, codes, scale, zp, st)
+                           : launch_quantize_rows_t<256, false>(x, x_row_stride, rows, bits, codes, scale, zp, st);
   if (D == 128) return f16 ? launch_quantize_rows_t<128, true>(x, x_row_stride, rows, bits, codes, scale, zp, st)
                            : launch_quantize_rows_t<128, false>(x, x_row_stride, rows, bits, codes, scale, zp, st);
   return f16 ? launch_quantize_rows_t<64, true>(x, x_row_stride, rows, bits, codes, scale, zp, st)
@@ -618,6 +622,8 @@ int launch_dequantize_rows_t(const uint8_t* codes, const float* scale, const int
 int launch_dequantize_rows(const uint8_t* codes, const float* scale, const int32_t* zp, int64_t rows, int D, int bits, bool f16,
                            void* out, int64_t out_row_stride, hipStream_t st) {
   if (rows == 0) return KVX_OK;
+  if (D == 256) return f16 ? launch_dequantize_rows_t<256, true>(codes, scale, zp, rows, bits, out, out_row_stride, st)
+                           : launch_dequantize_rows_t<256, false>(codes, scale, zp, rows, bits, out, out_row_stride, st);
   if (D == 128) return f16 ? launch_dequantize_rows_t<128, true>(codes, scale, zp, rows, bits, out, out_row_stride, st)
                            : launch_dequantize_rows_t<128, false>(codes, scale, zp, rows, bits, out, out_row_stride, st);
   return f16 ? launch_dequantize_rows_t<64, true>(codes, scale, zp, rows, bits, out, out_row_stride, st)
@@ -655,13 +661,10 @@ int launch_cache_write_d(const kvx_cache_write_args& a, unsigned grid, hipStream
   switch (a.kv_dtype) {
     case KVX_KV_F16: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_F16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
     case KVX_KV_BF16: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_BF16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
-    default:
-      if constexpr (D <= 128) {  // quantised stores: head sizes 64 and 128 (checked by the caller)
-        if (a.kv_dtype == KVX_KV_U4) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a);
-        else if (a.kv_dtype == KVX_KV_U8) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a);
-        else if (a.kv_dtype == KVX_KV_U4_F16) hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-        else hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8_F16>), dim3(grid), dim3(NTHREADS), 0, st, a);
-      }
+    case KVX_KV_U4: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
+    case KVX_KV_U8: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
+    case KVX_KV_U4_F16: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U4_F16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
+    default: hipLaunchKernelGGL((cache_write_kernel<D, KVX_KV_U8_F16>), dim3(grid), dim3(NTHREADS), 0, st, a); break;
   }
   KVX_HIP(hipGetLastError());
   return KVX_OK;

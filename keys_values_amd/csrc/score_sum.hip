@@ -499,19 +499,21 @@ int launch_score_sum(const kvx_sdpa_args& a, hipStream_t st) {
   p.k_sb = a.k_stride_b; p.k_sh = a.k_stride_h; p.k_st = a.k_stride_t;
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   p.tp_sb = a.tp_stride_b; p.tp_sh = a.tp_stride_h;
-  if (a.D == 128 || a.D == 64) {
+#define KVX_SCORE_SUM_CASE(KV) \
+  case KV: \
+    return a.D == 256 ? launch_t<256, KV>(p, pl.splits, st) : a.D == 128 ? launch_t<128, KV>(p, pl.splits, st) : launch_t<64, KV>(p, pl.splits, st);
+  if (a.D == 256 || a.D == 128 || a.D == 64) {
     switch (a.kv_dtype) {
-      case KVX_KV_BF16: return a.D == 128 ? launch_t<128, KVX_KV_BF16>(p, pl.splits, st) : launch_t<64, KVX_KV_BF16>(p, pl.splits, st);
-      case KVX_KV_F16: return a.D == 128 ? launch_t<128, KVX_KV_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_F16>(p, pl.splits, st);
-      case KVX_KV_U8: return a.D == 128 ? launch_t<128, KVX_KV_U8>(p, pl.splits, st) : launch_t<64, KVX_KV_U8>(p, pl.splits, st);
-      case KVX_KV_U4: return a.D == 128 ? launch_t<128, KVX_KV_U4>(p, pl.splits, st) : launch_t<64, KVX_KV_U4>(p, pl.splits, st);
-      case KVX_KV_U8_F16: return a.D == 128 ? launch_t<128, KVX_KV_U8_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_U8_F16>(p, pl.splits, st);
-      case KVX_KV_U4_F16: return a.D == 128 ? launch_t<128, KVX_KV_U4_F16>(p, pl.splits, st) : launch_t<64, KVX_KV_U4_F16>(p, pl.splits, st);
+      KVX_SCORE_SUM_CASE(KVX_KV_BF16)
+      KVX_SCORE_SUM_CASE(KVX_KV_F16)
+      KVX_SCORE_SUM_CASE(KVX_KV_U8)
+      KVX_SCORE_SUM_CASE(KVX_KV_U4)
+      KVX_SCORE_SUM_CASE(KVX_KV_U8_F16)
+      KVX_SCORE_SUM_CASE(KVX_KV_U4_F16)
     }
   }
-  if (a.D == 256 && kv_is_plain(a.kv_dtype))
-    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, pl.splits, st) : launch_t<256, KVX_KV_BF16>(p, pl.splits, st);
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
+#undef KVX_SCORE_SUM_CASE
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_score_sum: head size %d not in {64, 128, 256}", a.D);
 }
 
 }  // namespace kvx

@@ -476,20 +476,21 @@ __device__ __forceinline__ uint32_t dequant_pair2(uint32_t c0, int32_t zp0, floa
 }
 
 template <int D, int G, int KV>
-__global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
+__global__ __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) void decode_mfma_kernel(const DecodeParams p, const kvx_h2o_args hh, const int h2o) {
   constexpr bool F16 = kv_elem_f16(KV);
   constexpr bool U8 = !kv_is_plain(KV);  // codes + row state (8-bit or 4-bit store)
   constexpr bool U4 = kv_is_u4(KV);
   constexpr int KJ = D / 32;   // matrix instructions of the first product per 16-key tile
   constexpr int DPL = D / 16;  // d rows per lane = matrix instructions of the second product per 32-key block
   constexpr int CH = 32;       // keys per wavefront and step
-  constexpr int KR = U4 ? 1 : (U8 ? D / 64 : KJ);                          // 16-byte loads per key of K
-  constexpr int VW = U4 ? 1 : (U8 ? (DPL + 3) / 4 : DPL / 2);              // dwords per key of V
+  constexpr int NL4 = D >= 128 ? D / 128 : 1;                              // 4-bit rows: 16-byte loads per key of K
+  constexpr int KR = U4 ? NL4 : (U8 ? D / 64 : KJ);                        // 16-byte loads per key of K
+  constexpr int VW = U4 ? (DPL + 7) / 8 : (U8 ? (DPL + 3) / 4 : DPL / 2);  // dwords per key of V
   constexpr int LGK = logit_floats(G, D) / G;
   __shared__ __align__(16) float lgbuf[LGK * G];  // [key][head]
   __shared__ float red[WAVES][G][D];
   __shared__ float rml[WAVES][G][2];
-  static_assert(D == 64 || D == 128, "head sizes 64 and 128");
+  static_assert(D == 64 || D == 128 || (D == 256 && U8), "plain rows of 256 values take the vector-ALU kernel");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -503,6 +504,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
   auto kslice = [&](int e) -> int {
     if constexpr (!U8) return 8 * (kg + 4 * e);
     else if constexpr (U4 && D == 64) return 8 * kg + 32 * e;
+    else if constexpr (U4) return 16 * kg + 8 * (e & 1) + 64 * ((e >> 1) % NL4) + (D / 2) * (e / (2 * NL4));
     else return 16 * kg + 8 * (e & 1) + 64 * (e >> 1);
   };
   // d of row `mrow` of matrix instruction t of the second product
@@ -521,7 +523,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
   const uint8_t* kbase = (const uint8_t*)p.k + (b * p.k_sb + kvh * p.k_sh) * ES;
   const uint8_t* vbase = (const uint8_t*)p.v + (b * p.v_sb + kvh * p.v_sh) * ES;
   const uint32_t k_rowb = (uint32_t)p.k_st * ES, v_rowb = (uint32_t)p.v_st * ES;
-  const uint32_t k_lane = U4 ? (D == 128 ? 16 * kg : 8 * kg) : 16 * kg;    // + 64 r for the r-th load of the row
+  const uint32_t k_lane = (U4 && D == 64) ? 8 * kg : 16 * kg;              // + 64 r for the r-th load of the row
   const uint32_t v_lane = (uint32_t)m * (U4 ? DPL / 2 : (U8 ? DPL : 2 * DPL));
   const int64_t qs_off = b * p.qs_sb + kvh * p.qs_sh;
   const char* ksb = (const char*)(p.k_scale + qs_off);
@@ -567,24 +569,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
   };
   auto load_v = [&](Rows& r, int j, uint32_t off) {
     const uint8_t* row = vbase + off;
-    if constexpr (!U8) {
-      if constexpr (D == 128) {
-        const u32x4_t x = __builtin_nontemporal_load((const u32x4_t*)row);
-        r.v[j][0] = x[0]; r.v[j][1] = x[1]; r.v[j][2] = x[2]; r.v[j][3] = x[3];
-      } else {
-        const u32x2_t x = __builtin_nontemporal_load((const u32x2_t*)row);
-        r.v[j][0] = x[0]; r.v[j][1] = x[1];
-      }
-    } else if constexpr (!U4) {
-      if constexpr (D == 128) {
-        const u32x2_t x = __builtin_nontemporal_load((const u32x2_t*)row);
-        r.v[j][0] = x[0]; r.v[j][1] = x[1];
-      } else {
-        r.v[j][0] = __builtin_nontemporal_load((const uint32_t*)row);
-      }
+    constexpr int BYTES = U4 ? DPL / 2 : (U8 ? DPL : 2 * DPL);  // this lane's share of the row
+    if constexpr (BYTES == 16) {
+      const u32x4_t x = __builtin_nontemporal_load((const u32x4_t*)row);
+      r.v[j][0] = x[0]; r.v[j][1] = x[1]; r.v[j][2] = x[2]; r.v[j][3] = x[3];
+    } else if constexpr (BYTES == 8) {
+      const u32x2_t x = __builtin_nontemporal_load((const u32x2_t*)row);
+      r.v[j][0] = x[0]; r.v[j][1] = x[1];
+    } else if constexpr (BYTES == 4) {
+      r.v[j][0] = __builtin_nontemporal_load((const uint32_t*)row);
     } else {
-      if constexpr (D == 128) r.v[j][0] = __builtin_nontemporal_load((const uint32_t*)row);
-      else r.v[j][0] = (uint32_t)__builtin_nontemporal_load((const uint16_t*)row);
+      static_assert(BYTES == 2, "4-bit rows of 64 values");
+      r.v[j][0] = (uint32_t)__builtin_nontemporal_load((const uint16_t*)row);
     }
   };
   auto issue = [&](Rows& r, int chunk0) {
@@ -638,12 +634,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
       const u32x4_t w = r.k[gi][e >> 1];
       return (e & 1) ? dequant_words<F16>(w[2], w[3], r.kz[gi], r.ks[gi]) : dequant_words<F16>(w[0], w[1], r.kz[gi], r.ks[gi]);
     } else {
-      const u32x4_t w = r.k[gi][0];
+      const u32x4_t w = r.k[gi][D >= 128 ? (e >> 1) % NL4 : 0];
       u32x2_t bytes;
       int shift;
-      if constexpr (D == 128) {
+      if constexpr (D >= 128) {
         bytes = (e & 1) ? u32x2_t{w[2], w[3]} : u32x2_t{w[0], w[1]};
-        shift = (e >> 1) ? 0 : 4;
+        shift = (e / (2 * NL4)) ? 0 : 4;
       } else {
         bytes = u32x2_t{w[0], w[1]};
         shift = e ? 0 : 4;
@@ -666,9 +662,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void decode_mfma_kernel(const DecodePa
           c0 = (r.v[j0][t >> 2] >> (8 * (t & 3))) & 0xffu;
           c1 = (r.v[j1][t >> 2] >> (8 * (t & 3))) & 0xffu;
         } else {
-          const int sh = t < DPL / 2 ? 8 * t + 4 : 8 * (t - DPL / 2);
-          c0 = (r.v[j0][0] >> sh) & 0xfu;
-          c1 = (r.v[j1][0] >> sh) & 0xfu;
+          const int tb = t < DPL / 2 ? t : t - DPL / 2;  // byte of this lane's share; first half of the row: high nibble
+          const int sh = 8 * (tb & 3) + (t < DPL / 2 ? 4 : 0);
+          c0 = (r.v[j0][tb >> 2] >> sh) & 0xfu;
+          c1 = (r.v[j1][tb >> 2] >> sh) & 0xfu;
         }
         a[jj] = dequant_pair2<F16>(c0, r.vz[j0], r.vs[j0], c1, r.vz[j1], r.vs[j1]);
       }
@@ -1063,13 +1060,15 @@ int launch_dg(const DecodeParams& p, int kv, const kvx_h2o_args* hh, hipStream_t
   const kvx_h2o_args h2 = hh ? *hh : kvx_h2o_args{};
   const int h2o = hh != nullptr;
   // quantised stores and groups of 8 heads or more: both products on the matrix cores
-  if constexpr (D <= 128) {
+  {
     if (kv == KVX_KV_U4) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U4>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (kv == KVX_KV_U8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U8>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (kv == KVX_KV_U4_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U4_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
     else if (kv == KVX_KV_U8_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_U8_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
-    else if (G >= 8 && kv == KVX_KV_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
-    else if (G >= 8) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    else if constexpr (D <= 128 && G >= 8) {
+      if (kv == KVX_KV_F16) hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_F16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+      else hipLaunchKernelGGL((decode_mfma_kernel<D, G, KVX_KV_BF16>), grid, dim3(NTHREADS), 0, st, p, h2, h2o);
+    }
   }
   if constexpr (G <= 8) {
     if (kv_is_plain(kv) && (D > 128 || G < 8)) {
@@ -1147,8 +1146,8 @@ int launch_sdpa_decode(const kvx_sdpa_args& a, const kvx_h2o_args* hh, hipStream
   p.qs_sb = a.qs_stride_b; p.qs_sh = a.qs_stride_h;
   if (a.D == 128) return launch_d<128>(p, pl.G, a.kv_dtype, hh, st);
   if (a.D == 64) return launch_d<64>(p, pl.G, a.kv_dtype, hh, st);
-  if (a.D == 256 && kv_is_plain(a.kv_dtype)) return launch_d<256>(p, pl.G, a.kv_dtype, hh, st);
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
+  if (a.D == 256) return launch_d<256>(p, pl.G, a.kv_dtype, hh, st);
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_decode: head size %d not in {64, 128, 256}", a.D);
 }
 
 }  // namespace kvx

@@ -31,8 +31,9 @@ constexpr float kSlackLog2 = 8.0f;  // see the running-maximum update in the ker
 
 // Wavefronts per workgroup, 32 rows each. The uint8 cache takes 8: a tile is dequantised once per
 // workgroup, so twice the rows halve that vector work per row (-13 % kernel time); for bf16 tiles the
-// two sizes run alike and the smaller one leaves more workgroups for short chunks.
-constexpr int nwaves(int kv) { return kv_is_plain(kv) ? 4 : 8; }  // kv: enum kvx_kv_dtype
+// two sizes run alike and the smaller one leaves more workgroups for short chunks. At head size 256 the
+// output accumulators (128 registers) leave no room for two wavefronts per SIMD: four for every store.
+constexpr int nwaves(int kv, int D) { return (kv_is_plain(kv) || D > 128) ? 4 : 8; }  // kv: enum kvx_kv_dtype
 constexpr int BN = 64;   // keys per tile
 
 struct PrefillParams {
@@ -98,10 +99,13 @@ struct Loader {
   static constexpr bool U4 = kv_is_u4(KV);
   static constexpr int CPR = D / 8;
   static constexpr int RPW = 64 / CPR;        // rows per wavefront instruction: 4 (D=128), 8 (D=64)
-  static constexpr int NWAVES = nwaves(KV);
+  static constexpr int NWAVES = nwaves(KV, D);
   static constexpr int NTHREADS = 64 * NWAVES;
   static constexpr int NI = BN / RPW / NWAVES;     // instructions per wavefront per operand: 4 / 2
   static constexpr int ESZ = U8 ? 1 : 2;
+  // row groups of one wavefront are NWAVES RPW rows apart: with a multiple of 16 the XOR keys, and so
+  // the source chunks, are the same for all of them (not for D = 256 with four wavefronts: 8 rows)
+  static constexpr bool SAME_CHUNK = (NWAVES * RPW) % 16 == 0;
   const char* kbase;
   const char* vbase;
   const float* ks;
@@ -109,12 +113,10 @@ struct Loader {
   const float* vs;
   const int32_t* vz;
   const int32_t* tp;
-  uint32_t koff, voff;          // byte offset of this lane's chunk of row group 0 inside a tile (source side swizzled)
   int64_t k_tile_bytes, v_tile_bytes, k_st, v_st;
-  int64_t k_step, v_step;       // bytes between this wavefront's consecutive row groups (NWAVES RPW rows)
   int wave, lane, kv_len, rl;
   int cgk[NI], cgv[NI];         // the source chunk that belongs at this lane's LDS position, per row group
-  int shk, shv;                 // 4-bit store: nibble of this lane's K / V chunk (4 = high)
+  int shk[SAME_CHUNK ? 1 : NI], shv[SAME_CHUNK ? 1 : NI];  // 4-bit store: nibble of this lane's K / V chunk (4 = high)
   uint32_t lds_k, lds_v;        // LDS addresses of the K and V buffers (wavefront-uniform)
   uint32_t lds_kw, lds_vw;      // the same plus this wavefront's row-group offset
   uint32_t koffs[NI], voffs[NI];  // byte offset of this lane's chunk of row group i inside a tile
@@ -146,21 +148,16 @@ struct Loader {
     tp = p.tp ? p.tp + b * p.tp_sb + kvh * p.tp_sh : nullptr;
     k_tile_bytes = (int64_t)BN * p.k_st * ESZ;
     v_tile_bytes = (int64_t)BN * p.v_st * ESZ;
-    // row groups of one wavefront are NWAVES RPW rows apart: a multiple of 16 (the XOR keys and with them the
-    // source chunks are then the same for all of them) except for D = 256 with four wavefronts (8 rows apart)
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int r = row_of(i);
       cgk[i] = (lane % CPR) ^ swz_k<CPR>(r);  // the chunk that belongs at LDS position lane % CPR of row r
       cgv[i] = (lane % CPR) ^ swz_v<CPR>(r);
+      if (i == 0 || !SAME_CHUNK) {
+        shk[SAME_CHUNK ? 0 : i] = u4_shift<D>(cgk[i]);
+        shv[SAME_CHUNK ? 0 : i] = u4_shift<D>(cgv[i]);
+      }
     }
-    const int r0 = row_of(0);
-    koff = (uint32_t)(r0 * p.k_st * ESZ + chunk_off(cgk[0]));
-    voff = (uint32_t)(r0 * p.v_st * ESZ + chunk_off(cgv[0]));
-    shk = u4_shift<D>(cgk[0]);  // quantised stores: D <= 128, all row groups share their chunk
-    shv = u4_shift<D>(cgv[0]);
-    k_step = (int64_t)NWAVES * RPW * p.k_st * ESZ;
-    v_step = (int64_t)NWAVES * RPW * p.v_st * ESZ;
     lds_kw = lds_k + (uint32_t)(wave * RPW * CPR * 16);
     lds_vw = lds_v + (uint32_t)(wave * RPW * CPR * 16);
 #pragma unroll
@@ -195,8 +192,6 @@ struct Loader {
     }
     const char* base = IS_K ? kbase : vbase;
     const int64_t st = IS_K ? k_st : v_st;
-    const int64_t step = IS_K ? k_step : v_step;
-    const uint32_t off0 = IS_K ? koff : voff;
     const char* tb = base + tile * (IS_K ? k_tile_bytes : v_tile_bytes);
     if (key0 + BN <= kv_len) {
 #pragma unroll
@@ -206,7 +201,7 @@ struct Loader {
           dma16(tb, IS_K ? koffs[i] : voffs[i], dst);
         } else {
           const int key = key0 + row_of(i);
-          const u32x2_t c = *(const u32x2_t*)(tb + i * step + off0);
+          const u32x2_t c = *(const u32x2_t*)(tb + (IS_K ? koffs[i] : voffs[i]));
           if (IS_K) { kc[i] = c; ksr[i] = ks[key]; kzr[i] = kz[key]; }
           else { vc[i] = c; vsr[i] = vs[key]; vzr[i] = vz[key]; }
         }
@@ -264,7 +259,7 @@ struct Loader {
       for (int i = 0; i < NI; ++i) {
         const int r = row_of(i);
         u32x2_t c = IS_K ? kc[i] : vc[i];
-        if constexpr (U4) c = u4_codes(c, IS_K ? shk : shv);
+        if constexpr (U4) c = u4_codes(c, IS_K ? shk[SAME_CHUNK ? 0 : i] : shv[SAME_CHUNK ? 0 : i]);
         if (IS_K) sm.k[buf][r][lane % CPR] = dequant_words<kv_elem_f16(KV)>(c[0], c[1], kzr[i], ksr[i]);
         else sm.v[buf][r][lane % CPR] = dequant_words<kv_elem_f16(KV)>(c[0], c[1], vzr[i], vsr[i]);
       }
@@ -278,9 +273,9 @@ struct Loader {
 };
 
 template <int D, int KV>
-__global__ __launch_bounds__(64 * nwaves(KV), (kv_is_plain(KV) && D <= 128) ? 2 : 1) void sdpa_prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(64 * nwaves(KV, D), (kv_is_plain(KV) && D <= 128) ? 2 : 1) void sdpa_prefill_kernel(const PrefillParams p) {
   constexpr bool F16 = kv_elem_f16(KV);  // element type of q, k, v, o
-  constexpr int BM = 32 * nwaves(KV);  // rows per workgroup
+  constexpr int BM = 32 * nwaves(KV, D);  // rows per workgroup
   constexpr int CPR = D / 8;
   constexpr int KS = D / 16;  // k-steps of the first product
   constexpr int DT = D / 32;  // d tiles of the second product
@@ -673,7 +668,7 @@ void fill_params(PrefillParams& p, const kvx_sdpa_args& a) {
   p.R = a.q_len * p.G;
   p.input_pos = a.input_pos;
   p.num_tiles = (a.kv_len + BN - 1) / BN;
-  const int bm = 32 * nwaves(a.kv_dtype);
+  const int bm = 32 * nwaves(a.kv_dtype, a.D);
   p.m_blocks = (p.R + bm - 1) / bm;
   p.num_splits = pick_splits(a, p.m_blocks, p.num_tiles);
   p.tiles_per_split = (p.num_tiles + p.num_splits - 1) / p.num_splits;
@@ -698,7 +693,7 @@ size_t partial_bytes(const PrefillParams& p, int D) {
 template <int D, int KV>
 int launch_t(PrefillParams& p, hipStream_t st) {
   dim3 grid(p.B * p.Hkv, p.m_blocks, p.num_splits);
-  hipLaunchKernelGGL((sdpa_prefill_kernel<D, KV>), grid, dim3(64 * nwaves(KV)), 0, st, p);
+  hipLaunchKernelGGL((sdpa_prefill_kernel<D, KV>), grid, dim3(64 * nwaves(KV, D)), 0, st, p);
   KVX_HIP(hipGetLastError());
   if (p.num_splits > 1) {
     constexpr int ROWS = 256 / (D / 4);
@@ -730,19 +725,20 @@ int launch_sdpa_prefill(const kvx_sdpa_args& a, hipStream_t st) {
     p.part_o = (float*)a.workspace;
     p.part_ml = p.part_o + rows * (size_t)a.D;
   }
-  if (a.D == 128 || a.D == 64) {
+#define KVX_PREFILL_CASE(KV) \
+  case KV: return a.D == 256 ? launch_t<256, KV>(p, st) : a.D == 128 ? launch_t<128, KV>(p, st) : launch_t<64, KV>(p, st);
+  if (a.D == 256 || a.D == 128 || a.D == 64) {
     switch (a.kv_dtype) {
-      case KVX_KV_BF16: return a.D == 128 ? launch_t<128, KVX_KV_BF16>(p, st) : launch_t<64, KVX_KV_BF16>(p, st);
-      case KVX_KV_F16: return a.D == 128 ? launch_t<128, KVX_KV_F16>(p, st) : launch_t<64, KVX_KV_F16>(p, st);
-      case KVX_KV_U8: return a.D == 128 ? launch_t<128, KVX_KV_U8>(p, st) : launch_t<64, KVX_KV_U8>(p, st);
-      case KVX_KV_U4: return a.D == 128 ? launch_t<128, KVX_KV_U4>(p, st) : launch_t<64, KVX_KV_U4>(p, st);
-      case KVX_KV_U8_F16: return a.D == 128 ? launch_t<128, KVX_KV_U8_F16>(p, st) : launch_t<64, KVX_KV_U8_F16>(p, st);
-      case KVX_KV_U4_F16: return a.D == 128 ? launch_t<128, KVX_KV_U4_F16>(p, st) : launch_t<64, KVX_KV_U4_F16>(p, st);
+      KVX_PREFILL_CASE(KVX_KV_BF16)
+      KVX_PREFILL_CASE(KVX_KV_F16)
+      KVX_PREFILL_CASE(KVX_KV_U8)
+      KVX_PREFILL_CASE(KVX_KV_U4)
+      KVX_PREFILL_CASE(KVX_KV_U8_F16)
+      KVX_PREFILL_CASE(KVX_KV_U4_F16)
     }
   }
-  if (a.D == 256 && kv_is_plain(a.kv_dtype))
-    return a.kv_dtype == KVX_KV_F16 ? launch_t<256, KVX_KV_F16>(p, st) : launch_t<256, KVX_KV_BF16>(p, st);
-  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_prefill: head size %d not in {64, 128, 256} (quantised stores: {64, 128})", a.D);
+#undef KVX_PREFILL_CASE
+  return set_error(KVX_ERR_UNSUPPORTED, "kvx_sdpa_prefill: head size %d not in {64, 128, 256}", a.D);
 }
 
 }  // namespace kvx

@@ -141,7 +141,7 @@ class RowQuantizer:
         dev = self.device
         with torch.cuda.device(dev):
             st = _lib.stream_ptr(dev)
-            if not self.blocks_over_heads and d in (64, 128) and start == 0 and end == length and values.is_contiguous():
+            if not self.blocks_over_heads and d in (64, 128, 256) and start == 0 and end == length and values.is_contiguous():
                 # the whole store in one pass of the row kernels (16 or 8 lanes per row)
                 _lib.check(lib.kvx_quantize_rows_typed(values.data_ptr(), d, b * hkv * length, d, self.num_bits,
                                                        _lib.elem_kv_dtype(self.source_dtype), self.quant_buffer.data_ptr(),

@@ -334,14 +334,15 @@ def _sets_equal_away_from_ties(n_gpu, n_ref, scores_ref, k):
                 ), f"selection differs away from a tie at ({b},{h}): {sorted(diff)}"
 
 
-@pytest.mark.parametrize("quantized,dtype,bits", [(False, torch.bfloat16, 8), (True, torch.bfloat16, 8), (True, torch.float16, 8), (True, torch.float16, 4)])
-def test_h2o_cache_steps_vs_oracle(gpu, quantized, dtype, bits):
+@pytest.mark.parametrize("quantized,dtype,bits,D", [(False, torch.bfloat16, 8, 64), (True, torch.bfloat16, 8, 64), (True, torch.float16, 8, 64),
+                                                     (True, torch.float16, 4, 64), (True, torch.bfloat16, 8, 256), (True, torch.float16, 4, 256)])
+def test_h2o_cache_steps_vs_oracle(gpu, quantized, dtype, bits, D):
     """Prefill that fills the cache, then chunked steps: initial rule, evict-write, attention with
     scattered positions, score accumulation, selection (configuration 1 shapes: 8/2 heads, D 64,
     1024 slots, 128-token chunks). With the uint8 store every row is quantised once, when written,
     so the oracle is fed the dequantised rows: what the reference's attention reads from its
     dequantised working buffer (keys_values/kvcache/quant_buffers.py:776-793)."""
-    B, Hq, Hkv, L, D, chunk = 1, 8, 2, 1024, 64, 128
+    B, Hq, Hkv, L, chunk = 1, 8, 2, 1024, 128
     gen = torch.Generator().manual_seed(0)
     total = L + 4 * chunk
     qs = torch.randn(B, Hq, total, D, generator=gen).to(dtype)
