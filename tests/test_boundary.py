@@ -68,8 +68,8 @@ def test_validation_answers_without_a_gpu(kvx):
     a.Hq = 8
     a.D = 512
     assert kvx.kvx_sdpa_prefill(ctypes.byref(a), None) == _lib.KVX_ERR_UNSUPPORTED
-    a.D, a.kv_dtype = 256, _lib.KVX_KV_U8  # heads of 256 only with plain rows
-    assert kvx.kvx_sdpa_prefill(ctypes.byref(a), None) == _lib.KVX_ERR_UNSUPPORTED
+    a.D, a.kv_dtype = 128, 17  # not a store type
+    assert kvx.kvx_sdpa_prefill(ctypes.byref(a), None) == _lib.KVX_ERR_UNSUPPORTED and b"kv_dtype" in kvx.kvx_last_error()
     a.kv_dtype = _lib.KVX_KV_BF16
     h = _lib.H2OArgs()
     h.B, h.Hkv, h.kv_len, h.limit, h.k = 1, 1, 16, 16, 17
