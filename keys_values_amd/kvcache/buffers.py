@@ -11,6 +11,8 @@ bfloat16 or float16 rows, or as 8-bit / 4-bit codes with per-row scale and zero 
 ``QuantizedKVCacheBuffers`` with a ``TorchBasicQuantizer``, keys_values/kvcache/quant_buffers.py:361-804,
 without its dequantised working copy: the codes stay resident, rows are quantised when written and
 ``write_back`` has nothing left to do). Slot writes go through ``kvx_cache_write``; there is no CPU path.
+With ``blocks_over_heads=True`` the quantisation blocks are the slots over all heads, held by two
+``RowQuantizer`` stores and served by the quantiser's block kernels.
 """
 import ctypes
 from dataclasses import dataclass
@@ -20,6 +22,7 @@ import torch
 
 from .. import _lib
 from ..attention import ops
+from .quantize import RowQuantizer
 
 PositionsType = Union[torch.Tensor, Tuple[int, int]]
 
@@ -174,12 +177,34 @@ class KVCacheBuffers:
 _STORE_BITS = {"default": None, "torch-quantized8": 8, "torch-quantized4": 4}
 
 
+class BlockQuantizedKeysAndValues(KeysAndValues):
+    """The first ``length`` slots of a store whose quantisation blocks run over the heads, dequantised on demand."""
+
+    def __init__(self, quantizer_k, quantizer_v, batch_size: int, length: int):
+        self._qk, self._qv, self._b, self._t = quantizer_k, quantizer_v, batch_size, length
+
+    def keys(self) -> torch.Tensor:
+        return self._qk.dequantize(0, self._t)[: self._b]
+
+    def values(self) -> torch.Tensor:
+        return self._qv.dequantize(0, self._t)[: self._b]
+
+
 class HipKVCacheBuffers(KVCacheBuffers):
-    def __init__(self, params: KVCacheBuffersParams, cache_length: int, allocate_buffers: bool = False, num_bits: Optional[int] = None):
-        """``num_bits``: None for plain rows, 8 or 4 for the quantised store."""
+    def __init__(self, params: KVCacheBuffersParams, cache_length: int, allocate_buffers: bool = False, num_bits: Optional[int] = None,
+                 blocks_over_heads: bool = False):
+        """``num_bits``: None for plain rows, 8 or 4 for the quantised store. ``blocks_over_heads``: one quantisation
+        block per slot over all heads (keys_values/kvcache/quant_buffers.py:849-870) instead of one per (head, slot)
+        row; ignored by the plain store. A slot written for some heads only is requantised as a whole from the
+        dequantised rows of the others, as the reference's write-back of its dequantised working buffer does
+        (keys_values/kvcache/quant_buffers.py:368-375). This form is served by the block kernels of the quantiser;
+        the attention kernels read the one-block-per-row store only, so a cache on top of it attends over the rows
+        that ``get_keys_values`` dequantises."""
         super().__init__(params, cache_length)
         if num_bits not in (None, 4, 8):
             raise ValueError(f"num_bits = {num_bits}, must be None, 4 or 8")
+        self.blocks_over_heads = bool(blocks_over_heads) and num_bits is not None
+        self._qk = self._qv = None  # the two block stores (blocks over the heads only)
         sizes = ops.ALLOWED_HEAD_SIZES if num_bits is None else ops.QUANTIZED_HEAD_SIZES
         if params.head_size not in sizes:
             raise NotImplementedError(f"head_size = {params.head_size} not in {sizes}")
@@ -227,7 +252,17 @@ class HipKVCacheBuffers(KVCacheBuffers):
         if batch_size is None:
             return
         b, h, length = batch_size, self.n_query_groups, self.cache_length
-        if self.quantized:
+        if self.blocks_over_heads:
+            shape = (b, h, length, self.head_size)
+            self._qk = RowQuantizer(shape, self.dtype, self.num_bits, True, allocate_buffers=True, device=device)
+            self._qv = RowQuantizer(shape, self.dtype, self.num_bits, True, allocate_buffers=True, device=device)
+            for q in (self._qk, self._qv):
+                q.quant_buffer.zero_()
+            # the same names as the row store; shapes (b, length, h * row bytes) and (b, length)
+            self.k, self.v = self._qk.quant_buffer, self._qv.quant_buffer
+            self.k_scale, self.v_scale = self._qk.quant_scales, self._qv.quant_scales
+            self.k_zp, self.v_zp = self._qk.quant_zero_points, self._qv.quant_zero_points
+        elif self.quantized:
             self.k = torch.zeros((b, h, length, self._row_bytes()), dtype=torch.uint8, device=device)
             self.v = torch.zeros_like(self.k)
             self.k_scale = torch.zeros((b, h, length), dtype=torch.float32, device=device)
@@ -240,6 +275,7 @@ class HipKVCacheBuffers(KVCacheBuffers):
 
     def _deallocate(self):
         self.k = self.v = None
+        self._qk = self._qv = None
         self.k_scale = self.k_zp = self.v_scale = self.v_zp = None
 
     def _require_buffers(self):
@@ -274,6 +310,10 @@ class HipKVCacheBuffers(KVCacheBuffers):
         b, h, num, d = key.shape
         if (b, h, d) != (self.batch_size, self.n_query_groups, self.head_size) or key.shape != value.shape:
             raise ValueError(f"key.shape = {tuple(key.shape)}, value.shape = {tuple(value.shape)} do not fit the buffers")
+        if self.blocks_over_heads:
+            if not isinstance(positions, torch.Tensor):
+                self._check_positions(positions, num)
+            return self._set_block_slots(positions, key.to(device=self.device, dtype=self.dtype), value.to(device=self.device, dtype=self.dtype))
         index = self._check_positions(positions, num)
         key = key.to(device=self.device, dtype=self.dtype)
         value = value.to(device=self.device, dtype=self.dtype)
@@ -296,8 +336,63 @@ class HipKVCacheBuffers(KVCacheBuffers):
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
 
+    # -- blocks over the heads ------------------------------------------------------------------------------
+
+    def _gathered(self, q: "RowQuantizer", blocks: torch.Tensor) -> "RowQuantizer":
+        """A scratch store holding copies of the blocks ``blocks`` (flat batch * cache_length + slot indices)."""
+        n = blocks.numel()
+        tmp = RowQuantizer((1, self.n_query_groups, n, self.head_size), self.dtype, self.num_bits, True, allocate_buffers=True, device=self.device)
+        tmp.quant_buffer[0] = q.quant_buffer.view(-1, q.quant_buffer.shape[-1])[blocks]
+        tmp.quant_scales[0] = q.quant_scales.view(-1)[blocks]
+        tmp.quant_zero_points[0] = q.quant_zero_points.view(-1)[blocks]
+        return tmp
+
+    def _flat_blocks(self, index: torch.Tensor) -> torch.Tensor:
+        b = index.shape[0]
+        return (torch.arange(b, device=index.device).view(b, 1, 1) * self.cache_length + index.long()).reshape(-1)
+
+    def _set_block_slots(self, positions: PositionsType, key: torch.Tensor, value: torch.Tensor):
+        b, h, num, d = key.shape
+        for q in (self._qk, self._qv):
+            q.allocate_buffers(b)  # the batch size of this fill
+        if not isinstance(positions, torch.Tensor):  # every head writes the same slots: whole blocks are replaced
+            self._qk.quantize(positions[0], positions[1], key)
+            self._qv.quantize(positions[0], positions[1], value)
+            return
+        index = self._check_positions(positions, num)
+        blocks, where = torch.unique(self._flat_blocks(index), return_inverse=True)
+        heads = torch.arange(h, device=self.device).view(1, h, 1).expand(b, h, num).reshape(-1)
+        for q, new in ((self._qk, key), (self._qv, value)):
+            tmp = self._gathered(q, blocks)
+            rows = tmp.dequantize(0, blocks.numel())  # (1, h, n, d): the other heads' rows as the store holds them
+            rows[0, heads, where] = new.reshape(-1, d)
+            tmp.quantize(0, blocks.numel(), rows)
+            q.quant_buffer.view(-1, q.quant_buffer.shape[-1])[blocks] = tmp.quant_buffer[0]
+            q.quant_scales.view(-1)[blocks] = tmp.quant_scales[0]
+            q.quant_zero_points.view(-1)[blocks] = tmp.quant_zero_points[0]
+
+    def _get_block_slots(self, positions: PositionsType) -> Tuple[torch.Tensor, torch.Tensor]:
+        b, h = self.batch_size, self.n_query_groups
+        if not isinstance(positions, torch.Tensor):
+            start, end = positions
+            if not (0 <= start < end <= self.cache_length):
+                raise ValueError(f"positions = {positions} must be a range inside [0, {self.cache_length}]")
+            return self._qk.dequantize(start, end)[:b], self._qv.dequantize(start, end)[:b]
+        index = self._check_positions(positions)
+        num = index.shape[2]
+        blocks = self._flat_blocks(index)  # one block per (batch, head, position): the head's row is picked below
+        heads = torch.arange(h, device=self.device).view(1, h, 1).expand(b, h, num).reshape(-1)
+        each = torch.arange(blocks.numel(), device=self.device)
+        out = []
+        for q in (self._qk, self._qv):
+            rows = self._gathered(q, blocks).dequantize(0, blocks.numel())
+            out.append(rows[0, heads, each].view(b, h, num, self.head_size))
+        return out[0], out[1]
+
     def get_slots(self, positions: PositionsType) -> Tuple[torch.Tensor, torch.Tensor]:
         self._require_buffers()
+        if self.blocks_over_heads:
+            return self._get_block_slots(positions)
         b = self.batch_size
         if isinstance(positions, torch.Tensor):
             index = self._check_positions(positions).to(torch.int64)
@@ -325,6 +420,8 @@ class HipKVCacheBuffers(KVCacheBuffers):
         if not self.buffers_are_allocated or self.batch_size is None or self.current_length is None:
             return None
         b, t = self.batch_size, self.current_length
+        if self.blocks_over_heads:
+            return BlockQuantizedKeysAndValues(self._qk, self._qv, b, t)
         if not self.quantized:
             return DefaultKeysAndValues(self.k[:b, :, :t], self.v[:b, :, :t])
         return QuantizedKeysAndValues(self.k[:b, :, :t], self.v[:b, :, :t], self._quant_state(t), self.head_size, self.num_bits, self.dtype)
@@ -360,12 +457,13 @@ class HipKVCacheBuffers(KVCacheBuffers):
             raise IndexError("Argument 'cache_length' is missing")
         num_bits = kwargs.get("num_bits")
         rows = params.max_batch_size * params.n_query_groups * int(cache_length)
+        states = params.max_batch_size * int(cache_length) if kwargs.get("blocks_over_heads") else rows  # scale + zero point each
         if num_bits is None:
             if params.dtype is None:
                 raise ValueError("params.dtype must be provided")
             parts = {"buffers": 2 * rows * params.head_size * 8 * torch.empty((), dtype=params.dtype).element_size()}
         else:
-            parts = {"buffers": 2 * rows * params.head_size * num_bits, "quant_state": 2 * rows * 64}
+            parts = {"buffers": 2 * rows * params.head_size * num_bits, "quant_state": 2 * states * 64}
         return sum(parts.values()), parts
 
 

@@ -96,7 +96,15 @@ class H2OKVCache:
         replay_log_blocksize: Optional[int] = None,
         overlap_select: bool = False,
         dequantize_chunk_rows: Optional[int] = DEFAULT_DEQUANTIZE_CHUNK_ROWS,
+        blocks_over_heads: bool = False,
     ):
+        if blocks_over_heads and quantized:
+            # keys_values/kvcache/quant_buffers.py:849-870. This class keeps rows, positions and scores in one store
+            # that its kernels read and write in place, one quantisation block per (head, slot) row; blocks that
+            # run over the heads are requantised as a whole whenever one head's row changes.
+            raise NotImplementedError(
+                "blocks_over_heads=True is served by HipKVCacheBuffers / create_kv_cache_buffers (the buffer interface "
+                "of the reference's cache classes), not by the fused H2O store")
         # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
         # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
         self.dequantize_chunk_rows = dequantize_chunk_rows

@@ -93,3 +93,77 @@ def test_buffers_before_prefill_raise_a_clear_error(gpu):
         bufs.set_slots((0, 4), x, x)
     with pytest.raises(IndexError):
         bufs.get_slots((0, 4))
+
+
+def _oracle_blocks(x, bits):
+    """Codes, scales and zero points of the slots of x (B, Hkv, n, D), one block per slot over the heads."""
+    return O.quantize_store(x, bits, True)
+
+
+@pytest.mark.parametrize("bits,dtype", [(8, torch.bfloat16), (4, torch.bfloat16), (8, torch.float16)])
+def test_buffers_with_blocks_over_heads(gpu, bits, dtype):
+    """The store whose quantisation blocks run over the heads (keys_values/kvcache/quant_buffers.py:849-870),
+    through the buffer interface: a prefill leaves what the reference's quantiser leaves
+    (keys_values/kvcache/quantize/pytorch.py:235-245,312-355); a write to slots that differ per head requantises each
+    touched slot from the new rows and the dequantised rows of the other heads, which is what the reference's
+    write-back of its dequantised working buffer does to it (keys_values/kvcache/quant_buffers.py:368-375); reads
+    return the dequantised rows. Bit-exact against the oracle."""
+    B, Hkv, L, D, num = 2, 4, 96, 64, 5
+    gen = torch.Generator().manual_seed(bits)
+    params = KVCacheBuffersParams(B, Hkv, D, gpu, dtype)
+    buf = create_kv_cache_buffers(f"torch-quantized{bits}", params, L, blocks_over_heads=True)
+    assert buf.blocks_over_heads
+    k0 = torch.randn(B, Hkv, L, D, generator=gen).to(dtype)
+    v0 = (torch.randn(B, Hkv, L, D, generator=gen) * 3).to(dtype)
+    buf.prefill(k0.to(gpu), v0.to(gpu))
+    shape = (B, Hkv, L, D)
+    state = {}
+    for name, x, codes, sc, zp in (("k", k0, buf.k, buf.k_scale, buf.k_zp), ("v", v0, buf.v, buf.v_scale, buf.v_zp)):
+        c_ref, s_ref, z_ref = _oracle_blocks(x, bits)
+        assert tuple(codes.shape) == (B, L, Hkv * D * bits // 8) and tuple(sc.shape) == (B, L)
+        assert torch.equal(codes.cpu(), c_ref) and torch.equal(sc.cpu(), s_ref) and torch.equal(zp.cpu(), z_ref), name
+        state[name] = O.dequantize_store(c_ref, s_ref, z_ref, shape, bits, True, dtype).contiguous()
+        state[name + "_codes"] = (c_ref, s_ref, z_ref)
+    kv = buf.get_keys_values()
+    assert torch.equal(kv.keys().cpu(), state["k"]) and torch.equal(kv.values().cpu(), state["v"])
+    # slots that differ per head (and overlap between heads), two rounds
+    for rnd in range(2):
+        pos = torch.stack([torch.stack([torch.randperm(L, generator=gen)[:num] for _ in range(Hkv)]) for _ in range(B)]).to(torch.int32)
+        old, shared = pos[0, 1, 0].item(), pos[0, 0, 0].item()  # two heads write the same slot
+        pos[0, 1][pos[0, 1] == shared] = old
+        pos[0, 1, 0] = shared
+        k1 = torch.randn(B, Hkv, num, D, generator=gen).to(dtype)
+        v1 = torch.randn(B, Hkv, num, D, generator=gen).to(dtype)
+        buf.set_slots(pos.to(gpu), k1.to(gpu), v1.to(gpu))
+        for name, new, codes, sc, zp in (("k", k1, buf.k, buf.k_scale, buf.k_zp), ("v", v1, buf.v, buf.v_scale, buf.v_zp)):
+            work = state[name].clone()  # the dequantised working buffer
+            gi = pos.long().unsqueeze(-1).expand(-1, -1, -1, D)
+            work.scatter_(2, gi, new)
+            touched = torch.zeros(B, L, dtype=torch.bool)
+            for b in range(B):
+                touched[b, pos[b].reshape(-1).long()] = True
+            c_all, s_all, z_all = _oracle_blocks(work, bits)
+            got_c, got_s, got_z = codes.cpu(), sc.cpu(), zp.cpu()
+            assert torch.equal(got_c[touched], c_all[touched]) and torch.equal(got_s[touched], s_all[touched]) and torch.equal(got_z[touched], z_all[touched])
+            # untouched slots keep their codes: nothing else was requantised
+            old_c, old_s, old_z = state[name + "_codes"]
+            assert torch.equal(got_c[~touched], old_c[~touched]) and torch.equal(got_s[~touched], old_s[~touched]) and torch.equal(got_z[~touched], old_z[~touched])
+            state[name + "_codes"] = (got_c, got_s, got_z)
+            state[name] = O.dequantize_store(got_c, got_s, got_z, shape, bits, True, dtype).contiguous()
+        kk, vv = buf.get_slots(pos.to(gpu))
+        gi = pos.long().unsqueeze(-1).expand(-1, -1, -1, D)
+        assert torch.equal(kk.cpu(), state["k"].gather(2, gi)) and torch.equal(vv.cpu(), state["v"].gather(2, gi))
+        kk, vv = buf.get_slots((7, 19))
+        assert torch.equal(kk.cpu(), state["k"][:, :, 7:19]) and torch.equal(vv.cpu(), state["v"][:, :, 7:19])
+    # a range write replaces whole blocks
+    k2 = torch.randn(B, Hkv, 8, D, generator=gen).to(dtype)
+    buf.set_slots((16, 24), k2.to(gpu), k2.to(gpu))
+    c_ref, s_ref, z_ref = _oracle_blocks(k2, bits)
+    assert torch.equal(buf.k[:, 16:24].cpu(), c_ref) and torch.equal(buf.v_scale[:, 16:24].cpu(), s_ref)
+
+
+def test_h2o_cache_names_the_route_for_blocks_over_heads(gpu):
+    from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
+
+    with pytest.raises(NotImplementedError, match="HipKVCacheBuffers"):
+        H2OKVCache(KVCacheParams(1, 2, 64, 64, 4), quantized=True, blocks_over_heads=True, device=gpu)
