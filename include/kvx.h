@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define KVX_VERSION 102 /* major*10000 + minor*100 + patch */
+#define KVX_VERSION 103 /* major*10000 + minor*100 + patch */
 
 enum kvx_status {
   KVX_OK = 0,

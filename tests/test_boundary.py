@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(kvx):
     assert sorted(_lib.SYMBOLS) == names, "ctypes table and header disagree"
     for n in names:
         assert hasattr(kvx, n), f"libkvx.so does not export {n}"
-    assert kvx.kvx_version() == 102
+    assert kvx.kvx_version() == 103
 
 
 def test_struct_layouts_match_c(tmp_path):
