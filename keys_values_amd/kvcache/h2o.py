@@ -28,9 +28,18 @@ the Q-Hitter combination with the quantisation error (``QuantizedH2OKVCache`` /
 keys_values/kvcache/factory.py:50-66. With ``switch_replay_logging(True)`` the cache records the token
 chunks and the slot every later token went to (keys_values/kvcache/attn_weights.py:43-204,939-966).
 
-Not covered (raises): fp32 caches, bitsandbytes stores, quantisation blocks over heads in the cache object.
+With ``blocks_over_heads=True`` (keys_values/kvcache/quant_buffers.py:849-870) a quantisation block is a slot
+over all heads. The cache then works the way the reference's quantised buffers do
+(keys_values/kvcache/quant_buffers.py:361-804): the codes live in two block stores, the kernels run on a
+dequantised working buffer shared by the caches of a device and stream (a cache that finds the buffer holding
+another cache's rows dequantises its own store into it first), and after every slot write the touched slots are
+quantised again as whole blocks from the working rows and read back, so that the buffer always holds what the
+codes say. Every policy variant but the Q-Hitter combination runs on it.
+
+Not covered (raises): fp32 caches, bitsandbytes stores.
 """
 import ctypes
+import weakref
 from dataclasses import dataclass
 from typing import Optional
 
@@ -38,6 +47,7 @@ import torch
 
 from .. import _lib
 from ..attention import ops
+from .quantize import RowQuantizer
 from .replay import DEFAULT_REPLAY_LOG_BLOCKSIZE, AttnWeightsReplayLog, ReplayArena
 
 DEFAULT_KEEP_INITIAL_FRACTION = 0.05  # keys_values/kvcache/attn_weights.py:322
@@ -52,19 +62,28 @@ EAGER_SELECT = 4096
 DEFAULT_DEQUANTIZE_CHUNK_ROWS = 2048
 
 _dequant_buffers = {}
+_dequant_owner = {}  # per buffer: the cache whose rows it holds as that cache's working buffer (blocks over heads), else None
 
 
-def _dequant_scratch(device, numel: int, dtype: torch.dtype = torch.bfloat16):
+def _dequant_scratch(device, numel: int, dtype: torch.dtype = torch.bfloat16, owner=None):
     """Two 16-bit buffers of ``numel`` elements of ``dtype``, grow-only, shared by the caches of one device and
     stream (launches on a stream are ordered: a layer's attention has read them before the next layer's
-    dequantisation overwrites them)."""
+    dequantisation overwrites them). ``owner``: the cache that is about to use them as its working buffer; the third
+    value returned says whether they still hold that cache's rows from its last use. Any other use takes the
+    buffers away from their owner."""
     key = (str(device), torch.cuda.current_stream(device).cuda_stream)
     buf = _dequant_buffers.get(key)
-    if buf is None or buf.numel() < 2 * numel:
+    fresh = buf is None or buf.numel() < 2 * numel
+    if fresh:
         buf = torch.empty(2 * numel, dtype=torch.int16, device=device)
         _dequant_buffers[key] = buf
+    before = _dequant_owner.get(key)
+    held = (not fresh) and owner is not None and before is not None and before[0]() is owner and before[1] == numel
+    if before is not None and before[0]() is not None and before[0]() is not owner:
+        before[0]().wait_for_selection()  # its second stream may still be reading the rows
+    _dequant_owner[key] = (weakref.ref(owner), numel) if owner is not None else None
     buf = buf.view(dtype)
-    return buf[:numel], buf[numel : 2 * numel]
+    return buf[:numel], buf[numel : 2 * numel], held
 
 
 @dataclass(frozen=True)
@@ -98,13 +117,10 @@ class H2OKVCache:
         dequantize_chunk_rows: Optional[int] = DEFAULT_DEQUANTIZE_CHUNK_ROWS,
         blocks_over_heads: bool = False,
     ):
-        if blocks_over_heads and quantized:
-            # keys_values/kvcache/quant_buffers.py:849-870. This class keeps rows, positions and scores in one store
-            # that its kernels read and write in place, one quantisation block per (head, slot) row; blocks that
-            # run over the heads are requantised as a whole whenever one head's row changes.
-            raise NotImplementedError(
-                "blocks_over_heads=True is served by HipKVCacheBuffers / create_kv_cache_buffers (the buffer interface "
-                "of the reference's cache classes), not by the fused H2O store")
+        # blocks_over_heads (quantised stores only): one quantisation block per slot over all heads; see the module text
+        self.blocks_over_heads = bool(blocks_over_heads) and quantized
+        if self.blocks_over_heads and q_hitter:
+            raise NotImplementedError("the quantisation-error policy is served with one block per (head, slot) row only")
         # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
         # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
         self.dequantize_chunk_rows = dequantize_chunk_rows
@@ -170,10 +186,18 @@ class H2OKVCache:
         b, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
         kv_dtype = torch.uint8 if quantized else self.dtype
         row = d // 2 if (quantized and num_bits == 4) else d  # the 4-bit store packs two codes per byte
-        # K and V (and their row states) are the two halves of one allocation each: one launch can walk both
-        self._kv = torch.zeros((2, b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
-        self.k, self.v = self._kv[0], self._kv[1]
-        if quantized:
+        if self.blocks_over_heads:
+            # the codes; k and v are bound to the shared working buffer by every forward (_bind_working)
+            self.block_store_k = RowQuantizer((b, h, length, d), self.dtype, num_bits, True, allocate_buffers=True, device=self.device)
+            self.block_store_v = RowQuantizer((b, h, length, d), self.dtype, num_bits, True, allocate_buffers=True, device=self.device)
+            for q in (self.block_store_k, self.block_store_v):
+                q.quant_buffer.zero_()
+            self.k = self.v = None
+        else:
+            # K and V (and their row states) are the two halves of one allocation each: one launch can walk both
+            self._kv = torch.zeros((2, b, h, length, row), dtype=kv_dtype, device=self.device)  # buffers.py:462-464
+            self.k, self.v = self._kv[0], self._kv[1]
+        if quantized and not self.blocks_over_heads:
             self._kv_scale = torch.zeros((2, b, h, length), dtype=torch.float32, device=self.device)
             self._kv_zp = torch.zeros((2, b, h, length), dtype=torch.int32, device=self.device)
             self.k_scale, self.v_scale = self._kv_scale[0], self._kv_scale[1]
@@ -292,7 +316,7 @@ class H2OKVCache:
         self._log_chunks.append(token_idx.detach().clone())  # keys_values/kvcache/base.py:844-855
 
     def _quant_state(self, T: int) -> Optional[ops.QuantState]:
-        if not self.quantized:
+        if not self.quantized or self.blocks_over_heads:  # blocks over heads: the kernels read the working buffer
             return None
         b = self.batch_size
         return ops.QuantState(self.k_scale[:b, :, :T], self.k_zp[:b, :, :T], self.v_scale[:b, :, :T], self.v_zp[:b, :, :T])
@@ -347,6 +371,8 @@ class H2OKVCache:
             raise ValueError(f"shapes {tuple(query.shape)}, {tuple(key.shape)} do not fit the cache")
         input_pos = self._input_pos
         self.wait_for_selection()
+        if self.blocks_over_heads:
+            self._bind_working(fresh=input_pos == 0)
         if input_pos == 0:
             out = self._prefill_step(query, key, value)
             self._log_token_chunk(token_idx, num, prefill=True)
@@ -364,7 +390,9 @@ class H2OKVCache:
         if index is None:
             raise IndexError("Cache needs to be initialized with 'prefill' before being used")
         self._log_token_chunk(token_idx, num, prefill=False)
-        self._write(index, key, value, input_pos)
+        ring = self._write(index, key, value, input_pos)
+        if self.blocks_over_heads:
+            self._write_back(index, ring, (self.current_length, self.current_length + num) if diff > 0 else None)
         if diff > 0:
             self.current_length += num
         self._have_next = False
@@ -410,12 +438,57 @@ class H2OKVCache:
 
     __call__ = forward
 
+    # -- blocks over the heads: working buffer and write-back (keys_values/kvcache/quant_buffers.py:473-503,732-804) --
+
+    def _bind_working(self, fresh: bool):
+        """Point k / v at the shared working buffer and make it hold this cache's rows: dequantise the block stores
+        into it unless it still holds them from this cache's last step (``fresh``: a new sequence starts, nothing
+        stored counts)."""
+        bmax, h, length, d = self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size
+        kd, vd, held = _dequant_scratch(self.device, bmax * h * length * d, self.dtype, owner=self)
+        self.k, self.v = kd.view(bmax, h, length, d), vd.view(bmax, h, length, d)
+        if fresh or held or self.batch_size is None:
+            return
+        b = self.batch_size
+        for q, work in ((self.block_store_k, self.k), (self.block_store_v, self.v)):
+            q.allocate_buffers(b)
+            q.dequantize(0, length, out=work[:b])
+
+    def _write_back(self, index: torch.Tensor, ring: Optional[torch.Tensor], span):
+        """Quantise the slots just written as whole blocks from the working rows and read them back. ``span``: the
+        slot range when every head wrote the same slots (prefill, filling); else the slots are ``index`` (batch,
+        heads, num) and the ring slots that took new tokens. A slot that several heads wrote is processed once per
+        head, with the same result every time: no host synchronisation to find the distinct ones."""
+        b, h, length, d = self.batch_size, self.n_query_groups, self.cache_length, self.head_size
+        stores = ((self.block_store_k, self.k), (self.block_store_v, self.v))
+        for q, _ in stores:
+            q.allocate_buffers(b)
+        if span is not None:
+            start, end = span
+            for q, work in stores:
+                q.quantize(start, end, work[:b, :, start:end])
+                work[:b, :, start:end] = q.dequantize(start, end)
+            return
+        slots = index.reshape(b, -1).long()
+        if ring is not None:
+            slots = torch.cat((slots, ring.long().view(1, -1).expand(b, -1)), dim=1)
+        n = slots.shape[1]
+        blocks = (torch.arange(b, device=self.device).view(b, 1) * length + slots).reshape(-1)  # flat (batch, slot) ids
+        gi = slots.view(b, 1, n, 1).expand(b, h, n, d)
+        for q, work in stores:
+            tmp = RowQuantizer((b, h, n, d), self.dtype, self.num_bits, True, allocate_buffers=True, device=self.device)
+            tmp.quantize(0, n, work[:b].gather(2, gi))
+            q.quant_buffer.view(-1, q.quant_buffer.shape[-1])[blocks] = tmp.quant_buffer.view(b * n, -1)
+            q.quant_scales.view(-1)[blocks] = tmp.quant_scales.view(-1)
+            q.quant_zero_points.view(-1)[blocks] = tmp.quant_zero_points.view(-1)
+            work[:b].scatter_(2, gi, tmp.dequantize(0, n))
+
     def _dequantized(self, b: int, T: int):
         """bf16 views (b, n_query_groups, T, head_size) of the quantised store, dequantised into the shared
         scratch by one launch per tensor (all slots of the first ``b`` batch entries: they are contiguous)."""
         h, length, d = self.n_query_groups, self.cache_length, self.head_size
         rows = b * h * length
-        kd, vd = _dequant_scratch(self.device, rows * d, self.dtype)
+        kd, vd, _ = _dequant_scratch(self.device, rows * d, self.dtype)
         lib = _lib.load()
         bits, elem = self.num_bits, _lib.elem_kv_dtype(self.dtype)
 
@@ -447,6 +520,8 @@ class H2OKVCache:
                 extra.zero_()
         self.current_length = num
         self._write(index, key, value, 0)
+        if self.blocks_over_heads:
+            self._write_back(index, None, (0, num))
         if self.grace_period > 0:  # first slot to move out once the cache is full, attn_weights.py:861-863
             self.next_grace_pos = self.cache_length - self.grace_period
         self.prefill_length = num
@@ -468,7 +543,8 @@ class H2OKVCache:
         a = _lib.CacheWriteArgs()
         a.B, a.Hkv, a.num, a.D, a.cache_len = b, h, num, self.head_size, self.cache_length
         a.input_pos = input_pos
-        a.kv_dtype = _lib.quant_kv_dtype(self.num_bits, self.dtype) if self.quantized else _lib.elem_kv_dtype(self.dtype)
+        codes = self.quantized and not self.blocks_over_heads
+        a.kv_dtype = _lib.quant_kv_dtype(self.num_bits, self.dtype) if codes else _lib.elem_kv_dtype(self.dtype)
         a.index = index.data_ptr()
         a.index_stride_b, a.index_stride_h = index.stride(0), index.stride(1)
         a.key = key.data_ptr()
@@ -479,7 +555,7 @@ class H2OKVCache:
         a.kc_stride_b, a.kc_stride_h, a.kc_stride_t = self.k.stride(0), self.k.stride(1), self.k.stride(2)
         a.v_cache = self.v.data_ptr()
         a.vc_stride_b, a.vc_stride_h, a.vc_stride_t = self.v.stride(0), self.v.stride(1), self.v.stride(2)
-        if self.quantized:
+        if codes:
             a.k_scale, a.k_zp = self.k_scale.data_ptr(), self.k_zp.data_ptr()
             a.v_scale, a.v_zp = self.v_scale.data_ptr(), self.v_zp.data_ptr()
             a.qs_stride_b, a.qs_stride_h = self.k_scale.stride(0), self.k_scale.stride(1)
@@ -509,6 +585,7 @@ class H2OKVCache:
                 self.next_grace_pos = (self.next_grace_pos - prefix + num) % gp + prefix
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().kvx_cache_write(ctypes.byref(a), _lib.stream_ptr(self.device)))
+        return ring
 
     def _h2o_args(self, full: bool, k: int = 1) -> _lib.H2OArgs:
         a = _lib.H2OArgs()

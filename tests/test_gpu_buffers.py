@@ -160,10 +160,3 @@ def test_buffers_with_blocks_over_heads(gpu, bits, dtype):
     buf.set_slots((16, 24), k2.to(gpu), k2.to(gpu))
     c_ref, s_ref, z_ref = _oracle_blocks(k2, bits)
     assert torch.equal(buf.k[:, 16:24].cpu(), c_ref) and torch.equal(buf.v_scale[:, 16:24].cpu(), s_ref)
-
-
-def test_h2o_cache_names_the_route_for_blocks_over_heads(gpu):
-    from keys_values_amd.kvcache.h2o import H2OKVCache, KVCacheParams
-
-    with pytest.raises(NotImplementedError, match="HipKVCacheBuffers"):
-        H2OKVCache(KVCacheParams(1, 2, 64, 64, 4), quantized=True, blocks_over_heads=True, device=gpu)

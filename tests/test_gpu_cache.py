@@ -655,3 +655,122 @@ def test_overlapped_score_sum_pass_equals_in_order_pass(gpu, bits, grace):
         assert torch.equal(plain.scores, beside.scores) and torch.equal(plain.token_pos, beside.token_pos)
         assert torch.equal(plain.k, beside.k) and torch.equal(plain.v, beside.v)
         pos += chunk
+
+
+def _requantise_slots(ref, slots, bits, dtype):
+    """What a write-back does to the oracle's rows: the slots ``slots`` (batch, n) of ref.k / ref.v, each a block
+    over all heads, are quantised and dequantised (keys_values/kvcache/quant_buffers.py:732-775 with blocks over
+    the heads, keys_values/kvcache/quantize/pytorch.py:235-245,334-337)."""
+    B, Hkv, L, D = ref.k.shape
+    n = slots.shape[1]
+    gi = slots.view(B, 1, n, 1).expand(B, Hkv, n, D)
+    for store in (ref.k, ref.v):
+        rows = store.gather(2, gi)
+        c, sc, z = O.quantize_store(rows, bits, True)
+        store.scatter_(2, gi, O.dequantize_store(c, sc, z, (B, Hkv, n, D), bits, True, dtype).contiguous())
+
+
+@pytest.mark.parametrize("bits,dtype,grace", [(8, torch.bfloat16, 0), (4, torch.bfloat16, 0), (8, torch.float16, 0)])
+def test_h2o_cache_with_blocks_over_heads_vs_oracle(gpu, bits, dtype, grace):
+    """The cache over a store whose quantisation blocks run over the heads: prefill that fills it, chunk steps with
+    slots that differ per head, single-token steps (the fused decode + H2O call). The oracle is the plain cache with
+    the write-back applied to the slots of every write before attention reads them; rows, positions and scores are
+    compared after every step, the block stores' codes must dequantise to the working rows."""
+    B, Hq, Hkv, L, D, chunk = 2, 8, 2, 512, 64, 64
+    gen = torch.Generator().manual_seed(bits)
+    total = L + 3 * chunk + 3
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(dtype)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(dtype)
+    vs = (torch.randn(B, Hkv, total, D, generator=gen) * 2).to(dtype)
+    ref = O.H2OCacheOracle(B, Hq, Hkv, L, D, dtype=dtype, max_chunk_size=chunk)
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq, dtype), max_chunk_size=chunk, quantized=True, num_bits=bits, blocks_over_heads=True,
+                       grace_period=grace, device=gpu)
+    assert cache.blocks_over_heads
+    # another cache of the same kind takes the working buffer in between: each must find its own rows again
+    other = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq, dtype), max_chunk_size=chunk, quantized=True, num_bits=bits, blocks_over_heads=True, device=gpu)
+
+    def check_rows():
+        b, T = cache.batch_size, cache.current_length  # the shared working buffer is undefined beyond the slots in use
+        assert torch.equal(cache.k[:b, :, :T].cpu(), ref.k[:, :, :T]) and torch.equal(cache.v[:b, :, :T].cpu(), ref.v[:, :, :T])
+        back = cache.block_store_k.dequantize(0, T)
+        assert torch.equal(back.cpu(), ref.k[:, :, :T])
+
+    first = L - chunk  # prefill leaves room for one chunk: the filling branch
+    ref.prefill(qs[:, :, :first], ks[:, :, :first], vs[:, :, :first])
+    _requantise_slots(ref, torch.arange(first).view(1, -1).expand(B, -1), bits, dtype)
+    o = cache.forward(qs[:, :, :first].to(gpu), ks[:, :, :first].to(gpu), vs[:, :, :first].to(gpu))
+    o_ref, _ = O.sdpa_in_blocks(qs[:, :, :first], ks[:, :, :first], vs[:, :, :first], 1 / math.sqrt(D), 0, None, return_attn_weights=False)
+    assert rel_err(o.float().cpu().view(B, first, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+    check_rows()
+    other.forward(qs[:, :, :first].to(gpu) * 0.5, vs[:, :, :first].to(gpu), ks[:, :, :first].to(gpu))
+    pos = first
+    for step, num in enumerate([chunk, chunk, chunk, 1, 1, 1]):
+        sl = slice(pos, pos + num)
+        # the oracle's step with the write-back between the slot write and the attention
+        if ref.current_length < L:
+            index = torch.arange(ref.current_length, ref.current_length + num).view(1, 1, -1).expand(B, Hkv, -1)
+            ref.current_length += num
+        elif ref.use_initial_rule:
+            n0 = min(int(0.05 * L), L - num)
+            index = torch.arange(n0, n0 + num).view(1, 1, -1).expand(B, Hkv, -1)
+            ref.use_initial_rule = False
+        else:
+            index = ref.next_index[:, :, :num]
+        index = index.contiguous().to(torch.int64)
+        if step > 0 and cache._have_next:
+            cache.set_next_positions(index)  # keep the two caches on the same slots; the GPU's own choice is checked below
+        O.cache_write(ref.k, ref.v, ref.token_pos, ref.scores, index, ks[:, :, sl], vs[:, :, sl], ref.input_pos)
+        _requantise_slots(ref, index.reshape(B, -1), bits, dtype)
+        T = ref.current_length
+        o_ref, w = O.sdpa_in_blocks(qs[:, :, sl], ref.k[:, :, :T], ref.v[:, :, :T], ref.scale, ref.input_pos, ref.token_pos[:, :, :T].to(torch.int64))
+        ref.input_pos += num
+        if T == L:
+            ref.next_index = O.h2o_update_select(ref.scores, w, T, L, chunk)
+        else:
+            ref.scores[:, :, :T] += w
+        o = cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        assert cache.input_pos == ref.input_pos and torch.equal(cache.token_pos.cpu(), ref.token_pos)
+        assert rel_err(o.float().cpu().view(B, num, Hq, D).transpose(1, 2), o_ref.float()) < 2e-2
+        torch.testing.assert_close(cache.scores.cpu(), ref.scores, rtol=2e-3, atol=1e-5)
+        check_rows()
+        if T == L and num > 1:
+            _sets_equal_away_from_ties(cache._next_index[:B].cpu().long(), ref.next_index, ref.scores, chunk)
+        if step % 2 == 0:  # the working buffer changes hands
+            other.forward(qs[:, :, sl].to(gpu), vs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu))
+        pos += num
+
+
+def test_h2o_cache_blocks_over_heads_with_grace_period(gpu):
+    """With a grace period the ring rows move between slots: both ends of every move are written back. The block
+    stores' codes must dequantise to the working rows after every step, and the cache must stay close to the
+    unquantised one (8-bit blocks: a small relative error)."""
+    B, Hq, Hkv, L, D, chunk, grace = 1, 4, 2, 256, 64, 32, 48
+    gen = torch.Generator().manual_seed(7)
+    total = L + 4 * chunk
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    vs = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    params = KVCacheParams(B, Hkv, L, D, Hq)
+    cache = H2OKVCache(params, max_chunk_size=chunk, quantized=True, num_bits=8, blocks_over_heads=True, grace_period=grace, device=gpu)
+    plain = H2OKVCache(params, max_chunk_size=chunk, grace_period=grace, device=gpu)
+    pos = 0
+    for num in [L] + [chunk] * 4:
+        sl = slice(pos, pos + num)
+        args = (qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        if plain._have_next and cache._have_next:  # both on the slots the plain cache chose for this step
+            cache.set_next_positions(plain.next_positions(num))
+        o_plain = plain.forward(*args)
+        o = cache.forward(*args)
+        torch.cuda.synchronize()
+        assert torch.equal(cache.token_pos.cpu(), plain.token_pos.cpu())
+        assert rel_err(o.float().cpu(), o_plain.float().cpu()) < 5e-2
+        assert torch.equal(cache.block_store_k.dequantize(0, L).cpu(), cache.k[:B].cpu())
+        assert torch.equal(cache.block_store_v.dequantize(0, L).cpu(), cache.v[:B].cpu())
+        assert rel_err(cache.k[:B].float().cpu(), plain.k[:B].float().cpu()) < 2e-2
+        pos += num
+
+
+def test_q_hitter_takes_blocks_per_row_only(gpu):
+    with pytest.raises(NotImplementedError, match="one block per"):
+        H2OKVCache(KVCacheParams(1, 2, 64, 64, 4), quantized=True, q_hitter=True, blocks_over_heads=True, device=gpu)
