@@ -210,7 +210,8 @@ def bench_prefill(args, torch, dev):
     if u8:
         from keys_values_amd.kvcache.h2o import _dequant_scratch
 
-        kd, vd = (t.view(B, Hkv, T, D) for t in _dequant_scratch(dev, B * Hkv * T * D))  # the cache object's own buffer
+        kd, vd, _ = _dequant_scratch(dev, B * Hkv * T * D)  # the cache object's own buffer
+        kd, vd = kd.view(B, Hkv, T, D), vd.view(B, Hkv, T, D)
         dq = lib.kvx_dequantize_rows4 if u4 else lib.kvx_dequantize_rows
 
         def step_copy():
