@@ -34,7 +34,8 @@ over all heads. The cache then works the way the reference's quantised buffers d
 dequantised working buffer shared by the caches of a device and stream (a cache that finds the buffer holding
 another cache's rows dequantises its own store into it first), and after every slot write the touched slots are
 quantised again as whole blocks from the working rows and read back, so that the buffer always holds what the
-codes say. Every policy variant but the Q-Hitter combination runs on it.
+codes say. Every policy variant runs on it; the quantisation errors of the Q-Hitter combination are those of the new
+tokens' blocks over the heads (keys_values/kvcache/quant_buffers.py:306-331).
 
 Not covered (raises): fp32 caches, bitsandbytes stores.
 """
@@ -119,8 +120,6 @@ class H2OKVCache:
     ):
         # blocks_over_heads (quantised stores only): one quantisation block per slot over all heads; see the module text
         self.blocks_over_heads = bool(blocks_over_heads) and quantized
-        if self.blocks_over_heads and q_hitter:
-            raise NotImplementedError("the quantisation-error policy is served with one block per (head, slot) row only")
         # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
         # attended to over a bf16 copy of the quantised store made once for the chunk; None = never.
         self.dequantize_chunk_rows = dequantize_chunk_rows
@@ -392,6 +391,7 @@ class H2OKVCache:
         self._log_token_chunk(token_idx, num, prefill=False)
         ring = self._write(index, key, value, input_pos)
         if self.blocks_over_heads:
+            self._block_errors(index, ring, key, value)
             self._write_back(index, ring, (self.current_length, self.current_length + num) if diff > 0 else None)
         if diff > 0:
             self.current_length += num
@@ -453,6 +453,24 @@ class H2OKVCache:
         for q, work in ((self.block_store_k, self.k), (self.block_store_v, self.v)):
             q.allocate_buffers(b)
             q.dequantize(0, length, out=work[:b])
+
+    def _block_errors(self, index: torch.Tensor, ring: Optional[torch.Tensor], key: torch.Tensor, value: torch.Tensor):
+        """Quantisation errors of the new tokens for the Q-Hitter combination (keys_values/kvcache/qh2o.py:130-160):
+        with blocks over the heads they are those of the new tokens' own blocks, one per token over all heads
+        (keys_values/kvcache/quant_buffers.py:306-331), which the row-quantising slot write cannot produce. With a
+        grace period the errors of the ring slots move out with their rows first (``index[..., :num2]``), the last
+        ``num2`` new tokens then take the ring slots (keys_values/kvcache/attn_weights.py:267-303)."""
+        if self.q_errors is None:
+            return
+        b, h, num = index.shape
+        err = self.block_store_k.quantization_error(key.to(self.dtype)) + self.block_store_v.quantization_error(value.to(self.dtype))
+        slots = index.long()
+        if ring is not None:
+            num2 = ring.numel()
+            rs = ring.long().view(1, 1, num2).expand(b, h, num2)
+            self.q_errors[:b].scatter_(2, slots[:, :, :num2], self.q_errors[:b].gather(2, rs))
+            slots = torch.cat((slots[:, :, num2:], rs), dim=2)
+        self.q_errors[:b].scatter_(2, slots, err)
 
     def _write_back(self, index: torch.Tensor, ring: Optional[torch.Tensor], span):
         """Quantise the slots just written as whole blocks from the working rows and read them back. ``span``: the
@@ -521,6 +539,7 @@ class H2OKVCache:
         self.current_length = num
         self._write(index, key, value, 0)
         if self.blocks_over_heads:
+            self._block_errors(index, None, key, value)
             self._write_back(index, None, (0, num))
         if self.grace_period > 0:  # first slot to move out once the cache is full, attn_weights.py:861-863
             self.next_grace_pos = self.cache_length - self.grace_period
@@ -563,7 +582,8 @@ class H2OKVCache:
         a.tp_stride_b, a.tp_stride_h = self.token_pos.stride(0), self.token_pos.stride(1)
         a.scores = self.scores.data_ptr()
         a.sc_stride_b, a.sc_stride_h = self.scores.stride(0), self.scores.stride(1)
-        a.v_norm, a.q_errors = _lib.ptr(self.v_norm), _lib.ptr(self.q_errors)
+        # blocks over the heads: the row-quantising write cannot give the blocks' errors (_block_errors does)
+        a.v_norm, a.q_errors = _lib.ptr(self.v_norm), (None if self.blocks_over_heads else _lib.ptr(self.q_errors))
         if self._log_on and self._log_arena is not None and input_pos >= self.cache_length:
             # keys_values/kvcache/attn_weights.py:629-633: the slots are recorded by the kernel that consumes them
             log_pos = input_pos - self.cache_length

@@ -771,6 +771,35 @@ def test_h2o_cache_blocks_over_heads_with_grace_period(gpu):
         pos += num
 
 
-def test_q_hitter_takes_blocks_per_row_only(gpu):
-    with pytest.raises(NotImplementedError, match="one block per"):
-        H2OKVCache(KVCacheParams(1, 2, 64, 64, 4), quantized=True, q_hitter=True, blocks_over_heads=True, device=gpu)
+def test_q_hitter_over_blocks_over_heads(gpu):
+    """The Q-Hitter policy on a store with blocks over the heads: the error buffer holds, at every written slot,
+    |k - dq(q(k))| + |v - dq(q(v))| of the token's row inside the block of that token over all heads
+    (keys_values/kvcache/quant_buffers.py:306-331, keys_values/kvcache/qh2o.py:130-160), and the ring slots' errors
+    move with their rows."""
+    B, Hq, Hkv, L, D, chunk, grace, bits = 1, 4, 2, 128, 64, 16, 24, 8
+    gen = torch.Generator().manual_seed(11)
+    total = L + 3 * chunk
+    qs = torch.randn(B, Hq, total, D, generator=gen).to(torch.bfloat16)
+    ks = torch.randn(B, Hkv, total, D, generator=gen).to(torch.bfloat16)
+    vs = (torch.randn(B, Hkv, total, D, generator=gen) * 3).to(torch.bfloat16)
+
+    def block_error(x):  # (B, Hkv, n, D) -> (B, Hkv, n)
+        c, sc, z = O.quantize_store(x, bits, True)
+        back = O.dequantize_store(c, sc, z, tuple(x.shape), bits, True, x.dtype)
+        return torch.linalg.vector_norm(x - back, dim=-1, dtype=torch.float32)
+
+    token_err = block_error(ks) + block_error(vs)  # per token position, as if written alone
+    cache = H2OKVCache(KVCacheParams(B, Hkv, L, D, Hq), max_chunk_size=chunk, quantized=True, num_bits=bits, blocks_over_heads=True,
+                       q_hitter=True, grace_period=grace, device=gpu)
+    pos = 0
+    for num in [L, chunk, chunk, chunk]:
+        sl = slice(pos, pos + num)
+        cache.forward(qs[:, :, sl].to(gpu), ks[:, :, sl].to(gpu), vs[:, :, sl].to(gpu))
+        torch.cuda.synchronize()
+        # every slot holds the error of the token whose position it carries
+        tp = cache.token_pos[:B].cpu().long()
+        want = token_err.gather(2, tp)
+        torch.testing.assert_close(cache.q_errors[:B].cpu(), want, rtol=1e-5, atol=1e-6)
+        pos += num
+
+
