@@ -333,6 +333,60 @@ def test_prefill_and_decode_random_shapes(gpu, case):
     torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
 
 
+def _random_cases_wide(n, seed):
+    """A second seeded mix over what later builds added: up to 16 heads per KV head, head size 256, float16 rows,
+    quantised stores of every one of them."""
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        D = rnd.choice([64, 128, 256])
+        G = rnd.choice([1, 2, 4, 6, 8] if D == 256 else [1, 3, 4, 8, 9, 12, 16])
+        Hkv = rnd.choice([1, 2])
+        T = rnd.choice([3, 64, 97, 256, 511, 1000, 1537])
+        q_len = rnd.randint(1, min(T, 100))
+        cases.append((len(cases), rnd.choice([1, 2]), G * Hkv, Hkv, q_len, T, D, rnd.choice([0, 0, 2]), rnd.choice(["contig", "scattered"]),
+                      rnd.choice(["plain", "u8", "u8", "u4"]), rnd.choice(["bf16", "f16"])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases_wide(24, 77), ids=lambda c: "-".join(str(x) for x in c))
+def test_prefill_and_decode_random_shapes_wide(gpu, case):
+    n, B, Hq, Hkv, q_len, T, D, splits, layout, store, dt = case
+    dtype = torch.bfloat16 if dt == "bf16" else torch.float16
+    q, k, v, gen = make_qkv(9000 + n, B, Hq, Hkv, q_len, T, D, dtype=dtype)
+    scale = 1.0 / math.sqrt(D)
+    if layout == "contig":
+        input_pos, tp = T - q_len, None
+    else:
+        input_pos = T + 37
+        tp = scattered_positions(gen, B, Hkv, T, input_pos, q_len)
+    quant = None
+    kg, vg = k.to(gpu), v.to(gpu)
+    if store != "plain":
+        bits = 8 if store == "u8" else 4
+        (kc, ks, kz), (vc, vs, vz) = O.quantize_rows(k, bits), O.quantize_rows(v, bits)
+        k, v = O.dequantize_rows(kc, ks, kz, dtype), O.dequantize_rows(vc, vs, vz, dtype)
+        if bits == 4:
+            kc, vc = O.compress4(kc), O.compress4(vc)
+        kg, vg = kc.to(gpu), vc.to(gpu)
+        quant = ops.QuantState(ks.to(gpu), kz.to(gpu), vs.to(gpu), vz.to(gpu))
+    o_ref, w_ref = O.sdpa_in_blocks(q, k, v, scale, input_pos, None if tp is None else tp.long())
+    out, w, lse = ops.prefill_core(q.to(gpu), kg, vg, scale, input_pos, None if tp is None else tp.to(gpu), return_weights=True,
+                                   return_lse=True, output_transposed=False, quant=quant, num_splits=splits)
+    torch.cuda.synchronize()
+    assert out.dtype == dtype
+    assert rel_err(out.float().cpu(), o_ref.float()) < 2e-2
+    torch.testing.assert_close(w.cpu(), w_ref, rtol=1e-3, atol=1e-6)
+    torch.testing.assert_close(lse.cpu(), O.lse2(q, k, scale, input_pos, None if tp is None else tp.long()), rtol=0, atol=2e-3)
+    o1_ref, w1_ref = O.sdpa_in_blocks(q[:, :, :1], k, v, scale, 10 * T + 100, None)
+    out1, w1, _ = ops.decode_core(q[:, :, :1].to(gpu), kg, vg, scale, return_weights=True, quant=quant)
+    torch.cuda.synchronize()
+    assert rel_err(out1.float().cpu().unsqueeze(2), o1_ref.float()) < 2e-2
+    torch.testing.assert_close(w1.cpu(), w1_ref, rtol=1e-3, atol=1e-6)
+
+
 # ---- float16 queries / keys / values and head size 256 (keys_values/attention/flashinfer_wrapper.py:276,311-319) ----
 
 TYPED_CASES = [
