@@ -118,6 +118,11 @@ class H2OKVCache:
         dequantize_chunk_rows: Optional[int] = DEFAULT_DEQUANTIZE_CHUNK_ROWS,
         blocks_over_heads: bool = False,
     ):
+        self._init_kwargs = dict(max_chunk_size=max_chunk_size, normalize_scores=normalize_scores, grace_period=grace_period,
+                                 quantized=quantized, num_bits=num_bits, keep_initial_fraction=keep_initial_fraction, device=device,
+                                 v_length=v_length, q_hitter=q_hitter, combination_constant=combination_constant,
+                                 replay_log_blocksize=replay_log_blocksize, overlap_select=overlap_select,
+                                 dequantize_chunk_rows=dequantize_chunk_rows, blocks_over_heads=blocks_over_heads)
         # blocks_over_heads (quantised stores only): one quantisation block per slot over all heads; see the module text
         self.blocks_over_heads = bool(blocks_over_heads) and quantized
         # dequantize_chunk_rows: a chunk with at least this many query rows (tokens x heads per KV head) is
@@ -243,6 +248,98 @@ class H2OKVCache:
         if self.current_length is None:
             raise IndexError("Cache is not initialized, call 'prefill' first")
         return self.token_pos[: self.batch_size, :, : self.current_length]
+
+    # -- the rest of the reference's cache surface (keys_values/kvcache/base.py:249-377,669-712) ------------
+
+    def reset(self) -> None:
+        """``input_pos == 0`` afterwards: the next ``forward`` is the prefill of a new sequence
+        (keys_values/kvcache/base.py:343-350,700-702)."""
+        self.wait_for_selection()
+        self._input_pos = 0
+        self._have_next = False
+
+    def update_requires_attn_weights(self) -> bool:
+        return True  # keys_values/kvcache/attn_weights.py: the H2O family scores slots by attention weights
+
+    def get_params(self) -> KVCacheParams:
+        return KVCacheParams(self.max_batch_size, self.n_query_groups, self.cache_length, self.head_size, self.n_head, self.dtype)
+
+    def get_keys_values(self):
+        """A ``KeysAndValues`` holder over the slots in use, or None before the first prefill
+        (keys_values/kvcache/base.py:249-257). Quantised stores hand out holders that dequantise on ``keys()`` /
+        ``values()``."""
+        from .buffers import BlockQuantizedKeysAndValues, DefaultKeysAndValues, QuantizedKeysAndValues
+
+        if self.batch_size is None or self.current_length is None or self._input_pos == 0:
+            return None
+        self.wait_for_selection()
+        b, t = self.batch_size, self.current_length
+        if self.blocks_over_heads:
+            for q in (self.block_store_k, self.block_store_v):
+                q.allocate_buffers(b)
+            return BlockQuantizedKeysAndValues(self.block_store_k, self.block_store_v, b, t)
+        if not self.quantized:
+            return DefaultKeysAndValues(self.k[:b, :, :t], self.v[:b, :, :t])
+        return QuantizedKeysAndValues(self.k[:b, :, :t], self.v[:b, :, :t], self._quant_state(t), self.head_size, self.num_bits, self.dtype)
+
+    def get_v_norm(self) -> torch.Tensor:
+        """Norms of the stored V rows, (batch, n_query_groups, current_length) (keys_values/kvcache/h2o.py:273-283)."""
+        if self.v_norm is None:
+            raise AttributeError("this cache does not weight its scores by the V norms")
+        if self.current_length is None:
+            raise IndexError("Cache is not initialized, call 'prefill' first")
+        return self.v_norm[: self.batch_size, :, : self.current_length]
+
+    def size_estimate(self):
+        """(bits in total, bits by part) of the buffers this cache holds (keys_values/kvcache/attn_weights.py:900-909,
+        keys_values/kvcache/h2o.py:235-242). The working buffer that caches with blocks over the heads share is not
+        counted: it belongs to the device, not to a cache."""
+        def bits(*ts):
+            return 8 * sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+        if self.blocks_over_heads:
+            qs = (self.block_store_k, self.block_store_v)
+            parts = {"buffers": bits(*(q.quant_buffer for q in qs)), "quant_state": bits(*(t for q in qs for t in (q.quant_scales, q.quant_zero_points)))}
+        elif self.quantized:
+            parts = {"buffers": bits(self._kv), "quant_state": bits(self._kv_scale, self._kv_zp)}
+        else:
+            parts = {"buffers": bits(self._kv)}
+        parts["token_pos"] = bits(self.token_pos)
+        score_parts = {"scores": self.scores, "v_norm": self.v_norm, "q_errors": self.q_errors}
+        total_scores = 0
+        for name, t in score_parts.items():
+            if t is not None:
+                total_scores += bits(t)
+                if name != "scores":
+                    parts[name] = bits(t)
+        parts["scores"] = total_scores  # all score buffers together, as the reference reports them
+        return sum(v for k, v in parts.items() if k not in ("v_norm", "q_errors")), parts
+
+    @classmethod
+    def size_estimate_apriori(cls, params: KVCacheParams, **kwargs):
+        """The same without a cache (keys_values/kvcache/attn_weights.py:911-937, keys_values/kvcache/h2o.py:244-255).
+        ``kwargs`` as the constructor's: ``quantized``, ``num_bits``, ``blocks_over_heads``, ``v_length``, ``q_hitter``."""
+        if params.dtype is None:
+            raise ValueError("params.dtype must be provided")
+        rows = params.max_batch_size * params.n_query_groups * params.cache_length
+        quantized, num_bits = kwargs.get("quantized", False), kwargs.get("num_bits", 8)
+        if quantized:
+            states = params.max_batch_size * params.cache_length if kwargs.get("blocks_over_heads") else rows
+            parts = {"buffers": 2 * rows * params.head_size * num_bits, "quant_state": 2 * states * 64}
+        else:
+            parts = {"buffers": 2 * rows * params.head_size * 8 * torch.empty((), dtype=params.dtype).element_size()}
+        parts["token_pos"] = rows * 32
+        n_scores = 1 + int(bool(kwargs.get("v_length"))) + int(bool(kwargs.get("q_hitter")))
+        if kwargs.get("v_length"):
+            parts["v_norm"] = rows * 32
+        if kwargs.get("q_hitter"):
+            parts["q_errors"] = rows * 32
+        parts["scores"] = n_scores * rows * 32
+        return sum(v for k, v in parts.items() if k not in ("v_norm", "q_errors")), parts
+
+    def clone(self) -> "H2OKVCache":
+        """A new, empty cache with this one's settings (keys_values/kvcache/base.py:364-377: buffers are not copied)."""
+        return type(self)(self.params, **self._init_kwargs)
 
     def _second_stream(self) -> torch.cuda.Stream:
         if self._side_stream is None:
@@ -726,6 +823,7 @@ class VLengthH2OKVCache(H2OKVCache):
     norm of the slot's V row, normalised to sum to the number of queries."""
 
     def __init__(self, params: KVCacheParams, **kwargs):
+        kwargs.pop("v_length", None)  # comes back through clone()
         super().__init__(params, v_length=True, **kwargs)
 
 
@@ -735,6 +833,7 @@ class QuantizedH2OKVCache(H2OKVCache):
 
     def __init__(self, params: KVCacheParams, **kwargs):
         kwargs.setdefault("quantized", True)
+        kwargs.pop("q_hitter", None)  # comes back through clone()
         super().__init__(params, q_hitter=True, **kwargs)
 
 
@@ -743,6 +842,8 @@ class QuantizedVLengthH2OKVCache(H2OKVCache):
 
     def __init__(self, params: KVCacheParams, **kwargs):
         kwargs.setdefault("quantized", True)
+        kwargs.pop("q_hitter", None)  # come back through clone()
+        kwargs.pop("v_length", None)
         super().__init__(params, q_hitter=True, v_length=True, **kwargs)
 
 

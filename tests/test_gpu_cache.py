@@ -803,3 +803,46 @@ def test_q_hitter_over_blocks_over_heads(gpu):
         pos += num
 
 
+@pytest.mark.parametrize("name,kw", [("h2o-default", {}), ("h2o-torch-quantized8", {}), ("qh2o-vlen-torch-quantized4", {}),
+                                     ("h2o-torch-quantized8", {"blocks_over_heads": True})])
+def test_cache_surface_beyond_forward(gpu, name, kw):
+    """reset, get_keys_values, get_params, size_estimate (= size_estimate_apriori), update_requires_attn_weights,
+    clone, get_v_norm as the reference's caches have them (keys_values/kvcache/base.py:249-377,669-712,
+    keys_values/kvcache/attn_weights.py:900-937, keys_values/kvcache/h2o.py:235-283)."""
+    from keys_values_amd.kvcache import create_kv_cache
+
+    B, Hq, Hkv, L, D, chunk = 2, 4, 2, 128, 64, 16
+    params = KVCacheParams(B, Hkv, L, D, Hq)
+    cache = create_kv_cache(name, params, max_chunk_size=chunk, device=gpu, **kw)
+    assert cache.update_requires_attn_weights() and cache.get_params() == params
+    assert cache.get_keys_values() is None
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(B, Hq, L + chunk, D, generator=gen).to(torch.bfloat16).to(gpu)
+    k = torch.randn(B, Hkv, L + chunk, D, generator=gen).to(torch.bfloat16).to(gpu)
+    v = torch.randn(B, Hkv, L + chunk, D, generator=gen).to(torch.bfloat16).to(gpu)
+    cache.forward(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    cache.forward(q[:, :, L:], k[:, :, L:], v[:, :, L:])
+    kv = cache.get_keys_values()
+    keys, values = kv.keys(), kv.values()
+    assert keys.shape == (B, Hkv, L, D) and values.dtype == torch.bfloat16
+    tp = cache.token_positions().long()
+    gi = tp.unsqueeze(-1).expand(-1, -1, -1, D)
+    err = rel_err(keys.float().cpu(), k.gather(2, gi).float().cpu())  # slot s holds the row of the token at position tp[s]
+    assert err < (1e-6 if cache.num_bits is None else 2e-2 if cache.num_bits == 8 else 2e-1), err
+    total, parts = cache.size_estimate()
+    quantized, bits = cache.quantized, cache.num_bits or 8
+    total_a, parts_a = type(cache).size_estimate_apriori(params, quantized=quantized, num_bits=bits, v_length=cache.v_length, q_hitter=cache.q_hitter, **kw)
+    assert (total, parts) == (total_a, parts_a)
+    rows = B * Hkv * L
+    assert parts["token_pos"] == rows * 32 and parts["buffers"] == 2 * rows * D * (bits if quantized else 16)
+    if cache.v_length:
+        vn = cache.get_v_norm()
+        torch.testing.assert_close(vn.cpu(), torch.linalg.vector_norm(v.gather(2, gi).float(), dim=-1).cpu(), rtol=1e-2, atol=1e-3)
+    twin = cache.clone()
+    assert type(twin) is type(cache) and twin.get_keys_values() is None and twin.quantized == cache.quantized
+    # a new sequence after reset gives what a new cache gives
+    cache.reset()
+    assert cache.input_pos == 0
+    o1 = cache.forward(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    o2 = twin.forward(q[:, :, :L], k[:, :, :L], v[:, :, :L])
+    assert torch.equal(o1, o2) and torch.equal(cache.token_pos, twin.token_pos) and torch.equal(cache.scores, twin.scores)
